@@ -1,0 +1,312 @@
+"""CPU oracle for the K-FAC hot path of cybertronai/pytorch-sso.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the product package may import this
+module; it is the checker that tests, the smoke run and the CPU-baseline leg of
+the benchmark compare the HIP kernels against.
+
+Every function restates, from the mathematics, what one reference function
+computes on CPU tensors, and cites the reference file:line it follows.  The
+arithmetic type is selectable: ``dtype=torch.float32`` follows the reference's
+CPU path operation by operation (torch CPU einsum / unfold / mm and SciPy's
+LU-based ``linalg.inv``), ``dtype=torch.float64`` is the high-precision truth
+that both the fp32 oracle and the GPU results are compared with.
+
+Pinning (what each function is checked against in tests/test_oracle.py, none of
+which retypes the formula):
+  factor_linear_*      brute-force loops, A[-1,-1]==1, A[-1,:-1]==mean(a)
+  factor_conv_a        7-nested-loop patch extraction, 1x1-conv == linear case,
+                       autograd weight.grad identity (row order c,kh,kw)
+  factor_conv_g        autograd identity, linear special case
+  ema / accumulate     hand-computed two-step recursion, beta==1 copy
+  pi_damped_inverse    scalar-identity special case, residual X·X^-1 == I,
+                       2x2 by hand
+  precondition         Kronecker identity via torch.kron
+  bn_diag              per-sample gradient identity through autograd
+  cholesky_upper       U^T U == X, U upper, diag > 0
+  sample               injected-noise Kronecker identity
+  kfac_step / vi_step  golden vectors written by the reference itself
+                       (tests/golden/*.npz) and torch.optim.SGD equivalence
+The reference ships no golden vectors or known-answer tests for this path.
+"""
+import math
+
+import numpy as np
+import scipy.linalg
+import torch
+import torch.nn.functional as F
+
+
+# --------------------------------------------------------------------------
+# factors
+# --------------------------------------------------------------------------
+
+def factor_linear_a(a, bias=True, dtype=torch.float32):
+    """A = [a,1]^T [a,1] / n   (torchsso/curv/cov/linear.py:50-59).
+
+    a: [n, f_in].  The ones column is the LAST column (linear.py:52-55)."""
+    a = a.to(dtype)
+    n = a.shape[0]
+    if bias:
+        a = torch.cat((a, a.new_ones((n, 1))), 1)
+    return (a.t() @ a) / n
+
+
+def factor_linear_g(g, dtype=torch.float32, scale_by_batch=True):
+    """G = g^T g / n, then *= n^2   (torchsso/curv/cov/linear.py:61-67 followed by
+    torchsso/curv/curvature.py:154-155,299-300)."""
+    g = g.to(dtype)
+    n = g.shape[0]
+    G = (g.t() @ g) / n
+    if scale_by_batch:
+        G = G * float(n ** 2)
+    return G
+
+
+def factor_conv_a(x, kernel_size, stride=(1, 1), padding=(0, 0), dilation=(1, 1),
+                  bias=True, dtype=torch.float32):
+    """A = M M^T / n with M = unfold(x) as [c_in*kh*kw (+1), n*h_out*w_out]
+    (torchsso/curv/cov/conv.py:47-67).  Divides by n only (conv.py:66); the ones
+    ROW is last (conv.py:60-62); row order is (c_in, kh, kw) as F.unfold."""
+    x = x.to(dtype)
+    n = x.shape[0]
+    u = F.unfold(x, kernel_size=kernel_size, stride=stride, padding=padding,
+                 dilation=dilation)                       # n x a x L'
+    m = u.transpose(0, 1).reshape(u.shape[1], -1)         # a x (n L')
+    if bias:
+        m = torch.cat((m, m.new_ones((1, m.shape[1]))), 0)
+    return (m @ m.t()) / n
+
+
+def factor_conv_g(g, dtype=torch.float32, scale_by_batch=True):
+    """G = m m^T / (n h w), m = grad_out as [c_out, n*h*w], then *= n^2
+    (torchsso/curv/cov/conv.py:69-74; curvature.py:154-155,299-300)."""
+    g = g.to(dtype)
+    n, c, h, w = g.shape
+    m = g.transpose(0, 1).reshape(c, -1)
+    G = (m @ m.t()) / (n * h * w)
+    if scale_by_batch:
+        G = G * float(n ** 2)
+    return G
+
+
+def bn_diag(xhat, g, bias=True, dtype=torch.float32, scale_by_batch=True):
+    """Diagonal curvature of BatchNorm (torchsso/curv/cov/batchnorm.py:12-25 for
+    [n,f], :36-49 for [n,c,h,w]); every data tensor is then multiplied by n^2
+    (curvature.py:154-158)."""
+    xhat = xhat.to(dtype)
+    g = g.to(dtype)
+    n = g.shape[0]
+    if g.dim() == 4:
+        in_in = (xhat * xhat).sum(dim=(2, 3))
+        gg = (g * g).sum(dim=(2, 3))
+    else:
+        in_in = xhat * xhat
+        gg = g * g
+    out = [(in_in * gg).mean(dim=0)]
+    if bias:
+        out.append(gg.mean(dim=0))
+    if scale_by_batch:
+        out = [o * float(n ** 2) for o in out]
+    return out
+
+
+def bn_restore_input(out, weight, bias):
+    """x_hat = (out - bias) / weight   (torchsso/curv/curvature.py:123-134)."""
+    shape = (1, -1) + (1,) * (out.dim() - 2)
+    return (out - bias.view(shape)) / weight.view(shape)
+
+
+# --------------------------------------------------------------------------
+# accumulate / EMA
+# --------------------------------------------------------------------------
+
+def accumulate(acc, data, scale):
+    """acc = scale*data on first use else acc + scale*data
+    (torchsso/utils/accumulator.py:23-38)."""
+    if acc is None:
+        return [d * scale for d in data]
+    return [a + scale * d for a, d in zip(acc, data)]
+
+
+def ema_update(data, ema, beta):
+    """First call or beta == 1: copy.  Else ema = beta*data + (1-beta)*ema_old;
+    ``beta`` weighs the NEW data (torchsso/curv/curvature.py:174-187)."""
+    if ema is None or beta == 1:
+        return [d.clone() for d in data]
+    return [d * beta + (1 - beta) * e for d, e in zip(data, ema)]
+
+
+def l2_reg_ema_update(l2_reg, l2_reg_ema, beta, first):
+    """Scalar recursion next to the factor EMA (curvature.py:183,187)."""
+    if first or beta == 1:
+        return l2_reg
+    return l2_reg * beta + l2_reg_ema * (1 - beta)
+
+
+# --------------------------------------------------------------------------
+# inverse
+# --------------------------------------------------------------------------
+
+def _inv(m):
+    """torchsso.utils.inv on CPU = scipy.linalg.inv, general LU
+    (torchsso/utils/inv_cupy.py:32-34).  fp64 input gives the truth."""
+    return torch.from_numpy(scipy.linalg.inv(m.numpy()))
+
+
+def pi_and_damping(A, G, damping):
+    """pi = sqrt((trA/dA)/(trG/dG)); r = sqrt(damping); shifts r*pi and r/pi
+    (torchsso/curv/curvature.py:302-312)."""
+    pi = math.sqrt((A.trace().item() / A.shape[0]) / (G.trace().item() / G.shape[0]))
+    r = damping ** 0.5
+    return pi, r * pi, r / pi
+
+
+def pi_damped_inverse(A, G, damping, dtype=torch.float32):
+    """A^-1 = (A + r*pi*I)^-1, G^-1 = (G + r/pi*I)^-1
+    (curvature.py:302-312, add_value_to_diagonal :334-340, inv_cupy.py:27-34)."""
+    A = A.to(dtype)
+    G = G.to(dtype)
+    _, da, dg = pi_and_damping(A, G, damping)
+    Ad = A + torch.eye(A.shape[0], dtype=dtype) * da
+    Gd = G + torch.eye(G.shape[0], dtype=dtype) * dg
+    return _inv(Ad), _inv(Gd)
+
+
+def damped_inverse(X, value, dtype=torch.float32):
+    """(X + value*I)^-1 for one matrix (Curvature._inv, curvature.py:197-200)."""
+    X = X.to(dtype)
+    return _inv(X + torch.eye(X.shape[0], dtype=dtype) * value)
+
+
+def diag_inverse(X, damping, use_sqrt_ema=False):
+    """DiagCurvature._inv: 1 / (X(+sqrt) + damping)  (curvature.py:226-232)."""
+    if use_sqrt_ema:
+        X = X.sqrt()
+    return 1 / (X + damping)
+
+
+def cholesky_upper(X, dtype=torch.float32):
+    """torchsso.utils.cholesky(X, upper=True): U = (lower Cholesky factor)^T so
+    X = U^T U  (torchsso/utils/cholesky_cupy.py:9-14).  The reference has no CPU
+    implementation (cupy only); torch.linalg.cholesky is the library stand-in."""
+    return torch.linalg.cholesky(X.to(dtype)).mT.contiguous()
+
+
+# --------------------------------------------------------------------------
+# precondition / sampling
+# --------------------------------------------------------------------------
+
+def precondition(G_inv, A_inv, grad_w, grad_b=None, dtype=torch.float32):
+    """U = G^-1 [dW | db] A^-1, split back into dW (same shape as given) and db
+    (torchsso/curv/cov/linear.py:69-84, cov/conv.py:76-92)."""
+    oc = grad_w.shape[0]
+    g2 = grad_w.reshape(oc, -1).to(dtype)
+    if grad_b is not None:
+        g2 = torch.cat((g2, grad_b.to(dtype).view(-1, 1)), 1)
+    u = G_inv.to(dtype) @ g2 @ A_inv.to(dtype)
+    if grad_b is not None:
+        return u[:, :-1].reshape(grad_w.shape), u[:, -1].clone()
+    return u.reshape(grad_w.shape), None
+
+
+def sample(mean_w, mean_b, U_G, U_A, noise, std_scale, dtype=torch.float32):
+    """P = [mean_W | mean_b] + std_scale * U_G @ noise @ U_A with U = upper
+    Cholesky factors of the inverses; ``noise`` is what randn_like(m) returned
+    (torchsso/curv/cov/linear.py:86-100, cov/conv.py:94-108)."""
+    oc = mean_w.shape[0]
+    m = mean_w.reshape(oc, -1).to(dtype)
+    if mean_b is not None:
+        m = torch.cat((m, mean_b.to(dtype).view(-1, 1)), 1)
+    p = m + std_scale * (U_G.to(dtype) @ noise.to(dtype) @ U_A.to(dtype))
+    if mean_b is not None:
+        return p[:, :-1].reshape(mean_w.shape), p[:, -1].clone()
+    return p.reshape(mean_w.shape), None
+
+
+# --------------------------------------------------------------------------
+# straight-line optimizer steps (host sequencing)
+# --------------------------------------------------------------------------
+
+class KronLayerState(object):
+    """EMA/inverse state of one Kron layer as Curvature keeps it
+    (curvature.py:37-48)."""
+
+    def __init__(self):
+        self.ema = None
+        self.inv = None
+        self.std = None
+        self.l2_reg_ema = 0.
+        self.momentum = None
+
+
+def kron_curvature_step(state, A, G, damping, ema_decay, l2_reg=0., dtype=torch.float32,
+                        update_std=False):
+    """Curvature.step for a Kron layer: EMA, then pi-damped inverses with
+    damping + l2_reg_ema, then optionally std (curvature.py:166-191,302-321)."""
+    first = state.ema is None
+    state.ema = ema_update([A.to(dtype), G.to(dtype)], state.ema, ema_decay)
+    state.l2_reg_ema = l2_reg_ema_update(l2_reg, state.l2_reg_ema, ema_decay, first)
+    state.inv = list(pi_damped_inverse(state.ema[0], state.ema[1],
+                                       damping + state.l2_reg_ema, dtype))
+    if update_std:
+        state.std = [cholesky_upper(X, dtype) for X in state.inv]
+    return state
+
+
+def sgd_tail(p, grad, buf, lr, momentum=0., weight_decay=0.):
+    """Preconditioned-gradient tail of SecondOrderOptimizer.step with
+    momentum_type='preconditioned': g += wd*p; buf = m*buf + g; g = buf;
+    p -= lr*g  (torchsso/optim/secondorder.py:248-261,225-231)."""
+    if weight_decay != 0:
+        grad = grad + weight_decay * p
+    if momentum != 0:
+        buf = buf * momentum + grad
+        grad = buf.clone()
+    return p - lr * grad, grad, buf
+
+
+def kfac_layer_step(state, params, grads, A, G, *, lr, damping, ema_decay, l2_reg=0.,
+                    momentum=0., weight_decay=0., dtype=torch.float32, update_std=False):
+    """One pass of the per-group body of SecondOrderOptimizer.step for a Kron
+    layer (secondorder.py:195-209): raw l2, curvature step, precondition,
+    weight decay / momentum on the preconditioned gradient, update."""
+    w, b = params
+    gw, gb = grads
+    w = w.to(dtype)
+    gw = gw.to(dtype)
+    if b is not None:
+        b, gb = b.to(dtype), gb.to(dtype)
+    if l2_reg != 0:
+        gw = gw + l2_reg * w
+        if b is not None:
+            gb = gb + l2_reg * b
+    kron_curvature_step(state, A, G, damping, ema_decay, l2_reg, dtype, update_std)
+    pw, pb = precondition(state.inv[1], state.inv[0], gw, gb, dtype)
+    if state.momentum is None:
+        state.momentum = [torch.zeros_like(w), None if b is None else torch.zeros_like(b)]
+    w, pw, state.momentum[0] = sgd_tail(w, pw, state.momentum[0], lr, momentum, weight_decay)
+    if b is not None:
+        b, pb, state.momentum[1] = sgd_tail(b, pb, state.momentum[1], lr, momentum, weight_decay)
+    return (w, b), (pw, pb)
+
+
+# --------------------------------------------------------------------------
+# helpers
+# --------------------------------------------------------------------------
+
+def rel_fro(x, ref):
+    """||x - ref||_F / ||ref||_F in float64."""
+    x = torch.as_tensor(x).double().cpu()
+    ref = torch.as_tensor(ref).double().cpu()
+    d = (x - ref).norm().item()
+    r = ref.norm().item()
+    return d / r if r > 0 else d
+
+
+def conv_out_size(size, k, s, p, d):
+    return (size + 2 * p - d * (k - 1) - 1) // s + 1
+
+
+def np_seeded(shape, seed, scale=1.0):
+    rng = np.random.RandomState(seed)
+    return torch.from_numpy((rng.standard_normal(shape) * scale).astype(np.float32))

@@ -1,0 +1,219 @@
+// fp32 MFMA GEMM tile engine for gfx950 (CDNA4, wave64).
+//
+// One workgroup of 256 threads (4 waves, 2x2) computes a 128x128 tile of
+//     C[m][n] = sum_k  P(k, m) * Q(k, n)          k in [kbeg, kend)
+// with v_mfma_f32_32x32x2_f32.  Each wave owns a 64x64 sub-tile (2x2 MFMA
+// blocks, 64 accumulator registers).  Operands are described by functors that
+// map (k, m) to a global-memory element, so the same engine serves
+//   * factor builds (X^T X for Linear, implicit im2col for Conv2d),
+//   * the trailing updates / triangular products of the blocked inverse,
+//   * the two chained preconditioning GEMMs,
+// without ever materialising a transposed, concatenated or unfolded copy.
+//
+// Operand functor contract (see operands.h):
+//   static constexpr int layout;      KM: consecutive m are contiguous in memory
+//                                     MK: consecutive k are contiguous in memory
+//   MS mstate(int m) / KS kstate(int k): per-index precomputation
+//   float load(MS, KS): the element, 0 outside the operand's own bounds
+// The layout only chooses how the 256 threads sweep the 16x128 chunk so that
+// global loads coalesce, and how the chunk sits in LDS:
+//   KM chunk -> lds[k][m]   (row length 128), MFMA lanes read ds_read_b32
+//   MK chunk -> lds[m][k+4] (row length 20),  MFMA lanes read ds_read_b128
+// Within a 16-deep chunk the k values are consumed in the order
+//   step (j,s), lane half h  ->  k = 8j + 4h + s
+// for both operands, which is a permutation of the reduction index and so does
+// not change the product.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace kfac {
+
+constexpr int BM = 128;          // tile rows
+constexpr int BN = 128;          // tile cols
+constexpr int KC = 16;           // reduction depth per LDS stage
+constexpr int NTHREADS = 256;
+constexpr int LDS_MK = KC + 4;   // padded row of an MK chunk (bank-conflict free b128)
+constexpr int TILE_FLOATS = 2560;  // >= KC*BM and >= BM*LDS_MK
+constexpr int SMEM_FLOATS = 4 * TILE_FLOATS;  // 2 operands x 2 stages = 40 KiB
+
+enum { KM = 0, MK = 1 };
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// ---------------------------------------------------------------------------
+// global -> register -> LDS staging of one operand chunk
+// ---------------------------------------------------------------------------
+template <class OP>
+struct Stager {
+  static constexpr int NM = (OP::layout == KM) ? 1 : 8;
+  typename OP::MS ms[NM];
+  float regs[8];
+
+  __device__ __forceinline__ void init(const OP& op, int m0) {
+    const int t = threadIdx.x;
+    if (OP::layout == KM) {
+      ms[0] = op.mstate(m0 + (t & 127));
+    } else {
+#pragma unroll
+      for (int i = 0; i < NM; ++i) ms[i] = op.mstate(m0 + (t >> 4) + 16 * i);
+    }
+  }
+
+  __device__ __forceinline__ void fetch(const OP& op, int k0, int kend) {
+    const int t = threadIdx.x;
+    if (OP::layout == KM) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int k = k0 + (t >> 7) + 2 * i;
+        regs[i] = (k < kend) ? op.load(ms[0], op.kstate(k)) : 0.f;
+      }
+    } else {
+      const int k = k0 + (t & 15);
+      const bool kin = k < kend;
+      const typename OP::KS ks = op.kstate(kin ? k : k0);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) regs[i] = kin ? op.load(ms[i], ks) : 0.f;
+    }
+  }
+
+  __device__ __forceinline__ void commit(float* tile) const {
+    const int t = threadIdx.x;
+    if (OP::layout == KM) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) tile[((t >> 7) + 2 * i) * BM + (t & 127)] = regs[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) tile[((t >> 4) + 16 * i) * LDS_MK + (t & 15)] = regs[i];
+    }
+  }
+};
+
+// fragments of one operand for the 8 MFMA steps of a chunk: f[sub][4j+s]
+template <int LAYOUT>
+__device__ __forceinline__ void load_frags(const float* tile, int base, int r, int h,
+                                           float (&f)[2][8]) {
+  if (LAYOUT == KM) {
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+          f[sub][4 * j + s] = tile[(8 * j + 4 * h + s) * BM + base + 32 * sub + r];
+  } else {
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const float4 v =
+            *reinterpret_cast<const float4*>(&tile[(base + 32 * sub + r) * LDS_MK + 8 * j + 4 * h]);
+        f[sub][4 * j + 0] = v.x;
+        f[sub][4 * j + 1] = v.y;
+        f[sub][4 * j + 2] = v.z;
+        f[sub][4 * j + 3] = v.w;
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// The tile engine.  `same` = P and Q describe the same 128 columns (diagonal
+// tile of a symmetric product): Q is then neither fetched nor stored.
+// EPI::store(row, col, value) receives every element of the 128x128 tile
+// (global coordinates row = m0 + ..., col = n0 + ...).
+// ---------------------------------------------------------------------------
+template <class OPP, class OPQ, class EPI>
+__device__ __forceinline__ void gemm_tile(const OPP& P, const OPQ& Q, int m0, int n0, int kbeg,
+                                          int kend, bool same, EPI& epi, float* smem) {
+  const int t = threadIdx.x;
+  const int lane = t & 63;
+  const int wave = t >> 6;
+  const int r = lane & 31;
+  const int h = lane >> 5;
+  const int wm = (wave >> 1) * 64;
+  const int wn = (wave & 1) * 64;
+
+  v16f acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
+
+  Stager<OPP> sp;
+  Stager<OPQ> sq;
+  sp.init(P, m0);
+  if (!same) sq.init(Q, n0);
+
+  float* tp[2] = {smem, smem + 2 * TILE_FLOATS};
+  float* tq[2] = {smem + TILE_FLOATS, smem + 3 * TILE_FLOATS};
+
+  const int nchunks = (kend - kbeg + KC - 1) / KC;
+  if (nchunks > 0) {
+    sp.fetch(P, kbeg, kend);
+    if (!same) sq.fetch(Q, kbeg, kend);
+    sp.commit(tp[0]);
+    if (!same) sq.commit(tq[0]);
+  }
+  __syncthreads();
+
+  for (int c = 0; c < nchunks; ++c) {
+    const int cur = c & 1;
+    const bool more = (c + 1) < nchunks;
+    if (more) {
+      sp.fetch(P, kbeg + (c + 1) * KC, kend);
+      if (!same) sq.fetch(Q, kbeg + (c + 1) * KC, kend);
+    }
+    float fa[2][8], fb[2][8];
+    load_frags<OPP::layout>(tp[cur], wm, r, h, fa);
+    if (same)
+      load_frags<OPP::layout>(tp[cur], wn, r, h, fb);
+    else
+      load_frags<OPQ::layout>(tq[cur], wn, r, h, fb);
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a][s], fb[b][s], acc[a][b], 0, 0, 0);
+    if (more) {
+      sp.commit(tp[cur ^ 1]);
+      if (!same) sq.commit(tq[cur ^ 1]);
+    }
+    __syncthreads();
+  }
+
+  // accumulator element i of lane (r, h) in block (a, b):
+  //   row = 32a + 8*(i/4) + 4h + i%4 ,  col = 32b + r
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int row = m0 + wm + 32 * a + 8 * (i >> 2) + 4 * h + (i & 3);
+        const int col = n0 + wn + 32 * b + r;
+        epi.store(row, col, acc[a][b][i]);
+      }
+}
+
+// tile index t (0-based, row-major over the upper triangle incl. diagonal of a
+// T x T block grid) -> (bi, bj), bi <= bj
+__device__ __forceinline__ void upper_tile(int t, int T, int& bi, int& bj) {
+  int i = 0;
+  int rowlen = T;
+  // closed form guess then fix-up (T is at most a few hundred)
+  const float fT = 2.f * T + 1.f;
+  i = (int)((fT - sqrtf(fT * fT - 8.f * (float)t)) * 0.5f);
+  if (i < 0) i = 0;
+  if (i > T - 1) i = T - 1;
+  // start(i) = i*T - i*(i-1)/2
+  while (i > 0 && (i * T - (i * (i - 1)) / 2) > t) --i;
+  while (i + 1 < T && ((i + 1) * T - ((i + 1) * i) / 2) <= t) ++i;
+  (void)rowlen;
+  bi = i;
+  bj = i + (t - (i * T - (i * (i - 1)) / 2));
+}
+
+}  // namespace kfac

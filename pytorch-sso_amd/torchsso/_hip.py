@@ -1,0 +1,126 @@
+"""ctypes binding of libkfac_hip.so, the hand-written HIP (gfx950) K-FAC engine.
+
+There is no fallback: if the library is missing, or a tensor is not a
+contiguous fp32 tensor on a HIP device, the call raises.  torch is used only
+for device memory (tensors, the caching allocator for scratch) and for the
+current stream handle.
+"""
+import ctypes
+import os
+import threading
+
+import torch
+
+_LIB_NAME = 'libkfac_hip.so'
+_lib = None
+_lock = threading.Lock()
+
+c_int = ctypes.c_int
+c_i64 = ctypes.c_int64
+c_f32 = ctypes.c_float
+c_ptr = ctypes.c_void_p
+c_size = ctypes.c_size_t
+
+ERRORS = {1: 'invalid argument', 2: 'workspace too small', 3: 'HIP launch failed',
+          4: 'size above the static scratch limit'}
+
+
+class KfacHipError(RuntimeError):
+    pass
+
+
+def lib_path():
+    return os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
+
+
+_SIGNATURES = {
+    'kfac_abi_version': (c_int, []),
+    'kfac_factor_workspace_bytes': (c_size, [c_int, c_i64]),
+    'kfac_factor_linear': (c_int, [c_ptr, c_i64, c_int, c_i64, c_int, c_f32, c_f32, c_ptr,
+                                   c_ptr, c_size, c_ptr]),
+    'kfac_factor_conv_a': (c_int, [c_ptr] + [c_int] * 13 + [c_f32, c_f32, c_ptr,
+                                                           c_ptr, c_size, c_ptr]),
+    'kfac_factor_conv_g': (c_int, [c_ptr, c_int, c_int, c_int, c_int, c_f32, c_f32, c_ptr,
+                                   c_ptr, c_size, c_ptr]),
+}
+
+
+def signatures():
+    return dict(_SIGNATURES)
+
+
+def load():
+    """Load the shared library once; raises KfacHipError if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        path = lib_path()
+        if not os.path.exists(path):
+            raise KfacHipError(
+                '%s is not built: run `python pytorch-sso_amd/build_ext.py` '
+                '(there is no CPU or PyTorch fallback for the K-FAC kernels)' % path)
+        lib = ctypes.CDLL(path)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def check(status, what):
+    if status != 0:
+        raise KfacHipError('%s failed: %s (code %d)' % (what, ERRORS.get(status, '?'), status))
+
+
+def dev_ptr(t, what='tensor'):
+    """Device address of a contiguous fp32 HIP tensor (loud otherwise)."""
+    if not isinstance(t, torch.Tensor):
+        raise KfacHipError('%s: expected a torch.Tensor' % what)
+    if not t.is_cuda:
+        raise KfacHipError('%s is on %s: the K-FAC kernels run on a HIP device only '
+                           '(no CPU path exists in this package)' % (what, t.device))
+    if t.dtype != torch.float32:
+        raise KfacHipError('%s has dtype %s, expected float32' % (what, t.dtype))
+    if not t.is_contiguous():
+        raise KfacHipError('%s is not contiguous' % what)
+    return t.data_ptr()
+
+
+def stream_ptr(device=None):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+class _Workspace(threading.local):
+    """Per-thread, per-device scratch taken from torch's caching allocator and
+    grown on demand (forward hooks run on the caller's thread, backward hooks
+    on autograd's worker thread; each gets its own buffer)."""
+
+    def __init__(self):
+        self.bufs = {}
+
+    def get(self, device, nbytes):
+        nbytes = int(nbytes)
+        if nbytes == 0:
+            return None, 0
+        key = (device.type, device.index)
+        buf = self.bufs.get(key)
+        if buf is None or buf.numel() < nbytes:
+            # round up so that a slowly growing request does not reallocate each time
+            size = max(nbytes, 1 << 20)
+            size = 1 << (size - 1).bit_length()
+            buf = torch.empty(size, dtype=torch.uint8, device=device)
+            self.bufs[key] = buf
+        return buf, buf.numel()
+
+
+_workspace = _Workspace()
+
+
+def workspace(device, nbytes):
+    """(tensor-or-None, usable bytes); the tensor must stay referenced until the
+    kernels using it have been enqueued (stream order then protects it)."""
+    return _workspace.get(device, nbytes)
