@@ -72,6 +72,130 @@ int kfac_factor_conv_g(const float* g, int n, int c, int h, int w,
                        float alpha, float beta, float* C,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- Damped factor inversion ------------------------------------------- */
+
+/* Scratch for the three batched routines below: a descriptor table plus one
+ * n x n buffer per matrix.  `dims` is a HOST array of `count` sizes. */
+size_t kfac_inverse_workspace_bytes(int count, const int* dims);
+
+/* For every layer l:  pi = sqrt((tr A/dA) / (tr G/dG)), r = sqrt(damping[l]),
+ *   Ainv = (A + r*pi*I)^-1 ,  Ginv = (G + (r/pi)*I)^-1 .
+ * The traces, pi and the diagonal shift are computed on the device and the
+ * shift is added while the factor is copied into the Cholesky work area; all
+ * 2*layers matrices are factored, triangular-inverted and multiplied back in
+ * one shared launch sequence (blocked Cholesky, 128-wide panels).
+ * Replaces KronCurvature.update_inv, torchsso/curv/curvature.py:302-312, with
+ * add_value_to_diagonal :334-340 and torchsso.utils.inv,
+ * utils/inv_cupy.py:27-34 (cuSOLVER potrf + potrs against I, :114-128).
+ * dA, dG, damping and the four pointer arrays are HOST arrays of length
+ * `layers` (the pointers in them are device pointers; A and G are only read;
+ * Ainv/Ginv must not alias A/G).  damping[l] is the layer's damping + l2_reg_ema
+ * (curvature.py:102-104).  info is a DEVICE array of 2*layers ints: info[2l]
+ * for A_l, info[2l+1] for G_l; 0 = success, k > 0 = the leading minor of order
+ * k is not positive definite (the reference never reads cuSOLVER's dev_info,
+ * inv_cupy.py:124,130). */
+int kfac_pi_damped_inverse_batched(int layers, const int* dA, const int* dG,
+                                   const float* const* A, const float* const* G,
+                                   const float* damping,
+                                   float* const* Ainv, float* const* Ginv, int* info,
+                                   void* workspace, size_t workspace_bytes, void* stream);
+
+/* dst[i] = (src[i] + damp[i]*I)^-1 for `count` symmetric positive definite
+ * matrices of sizes dims[i]; damp may be NULL (no shift).  Host arrays as
+ * above; info is a DEVICE array of `count` ints.
+ * Replaces Curvature._inv, curvature.py:197-200, and torchsso.utils.inv. */
+int kfac_damped_inverse_batched(int count, const int* dims, const float* const* src,
+                                const float* damp, float* const* dst, int* info,
+                                void* workspace, size_t workspace_bytes, void* stream);
+
+/* dst[i] = U with src[i] = U^T U, U upper triangular (strictly lower part
+ * written as zero).  Replaces torchsso.utils.cholesky(m, upper=True),
+ * utils/cholesky_cupy.py:9-14, as used by KronCurvature.update_std,
+ * curvature.py:317-321. */
+int kfac_cholesky_upper_batched(int count, const int* dims, const float* const* src,
+                                float* const* dst, int* info,
+                                void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- Preconditioning and posterior sampling ---------------------------- */
+
+/* Scratch for the two routines below (dG, dA: HOST arrays). */
+size_t kfac_precondition_workspace_bytes(int layers, const int* dG, const int* dA);
+
+/* For every layer:  [gradW | gradb] <- Ginv * [gradW | gradb] * Ainv, in place.
+ * gradW is [dG, dA - 1] when gradb[l] != NULL (dA counts the bias column,
+ * which is LAST) and [dG, dA] otherwise; for Conv2d gradW is the weight
+ * gradient viewed as [c_out, c_in*kh*kw].  Two chained MFMA products per
+ * launch pair for the whole layer set; no concatenated copy is made.
+ * Replaces torch.cat + G_inv.mm(grad).mm(A_inv) + copy_ in
+ * torchsso/curv/cov/linear.py:69-84 and cov/conv.py:76-92.
+ * All array arguments are HOST arrays of length `layers`. */
+int kfac_precondition_batched(int layers, const int* dG, const int* dA,
+                              const float* const* Ginv, const float* const* Ainv,
+                              float* const* gradW, float* const* gradb,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
+/* For every layer:  [paramW | paramb] = [meanW | meanb] + std_scale * U_G * E * U_A
+ * with U_G, U_A the upper Cholesky factors of the inverses and E = noise[l], a
+ * [dG, dA] standard-normal matrix drawn by the caller (so that the random
+ * stream stays the host framework's).  Replaces
+ * torchsso/curv/cov/linear.py:86-100 and cov/conv.py:94-108. */
+int kfac_sample_batched(int layers, const int* dG, const int* dA,
+                        const float* const* U_G, const float* const* U_A,
+                        const float* const* noise,
+                        const float* const* meanW, const float* const* meanb,
+                        float* const* paramW, float* const* paramb, float std_scale,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- HBM-bound tails (one launch per tensor list) ----------------------- */
+
+/* Scratch for the four *_batched routines below. */
+size_t kfac_vector_workspace_bytes(int count);
+
+/* y[i] = a * x[i] + b * y[i]  (b == 0: y is not read).
+ * Running average of curvature.py:185-186 (a = ema_decay, b = 1 - ema_decay,
+ * x = data, y = ema), accumulation of utils/accumulator.py:23-38 (b = 1) and
+ * the l2 term grad += l2_reg * param of optim/secondorder.py:238-243. */
+int kfac_axpby_batched(int count, const int64_t* numel, const float* const* x,
+                       float* const* y, float a, float b,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+/* inv[i] = 1 / ((use_sqrt ? sqrt(ema[i]) : ema[i]) + damping[i])
+ * DiagCurvature._inv, curvature.py:226-232. */
+int kfac_diag_inverse_batched(int count, const int64_t* numel, const float* const* ema,
+                              float* const* inv, const float* damping, int use_sqrt,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
+/* grad[i] *= inv[i]   DiagCurvature.precondition_grad, curvature.py:234-238. */
+int kfac_diag_precondition_batched(int count, const int64_t* numel, const float* const* inv,
+                                   float* const* grad,
+                                   void* workspace, size_t workspace_bytes, void* stream);
+
+/* g += weight_decay*p ; if momentum: buf = momentum*buf + g, g = buf ; p -= lr*g
+ * with g written back, per tensor i with its own lr/momentum/weight_decay
+ * (HOST arrays).  The preconditioned-gradient tail of
+ * SecondOrderOptimizer.update_preprocess / update,
+ * optim/secondorder.py:248-261 and :225-231. */
+int kfac_sgd_update_batched(int count, const int64_t* numel, float* const* param,
+                            float* const* grad, float* const* momentum_buf,
+                            const float* lr, const float* momentum, const float* weight_decay,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- BatchNorm diagonal curvature -------------------------------------- */
+
+/* out[row] = sum_i ((x[row*len + i] - shift[c]) / scale[c])^2, c = row % channels;
+ * scale/shift may be NULL.  With x = the BatchNorm output and scale/shift its
+ * weight/bias this is sum_hw x_hat^2 of cov/batchnorm.py:36-37 without
+ * materialising x_hat (curvature.py:123-134); with NULLs on grad_output it is
+ * sum_hw g^2 (:38). */
+int kfac_rowsq_sum(const float* x, int64_t rows, int channels, int len,
+                   const float* scale, const float* shift, float* out, void* stream);
+
+/* w_curv[c] = alpha * sum_n sx[n][c]*sg[n][c] ; b_curv[c] = alpha * sum_n sg[n][c]
+ * (b_curv may be NULL).  cov/batchnorm.py:40-49 with alpha = n^2 / n from the
+ * rescale of curvature.py:154-158. */
+int kfac_bn_diag_combine(const float* sx, const float* sg, int n, int channels, float alpha,
+                         float* w_curv, float* b_curv, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,223 @@
+// HBM-bound tails of the K-FAC step, each one launch over a whole list of
+// tensors: running average / accumulation, diagonal (BatchNorm) curvature,
+// diagonal inverse and preconditioning, and the fused parameter update.
+#include <algorithm>
+#include <vector>
+
+#include "common.h"
+
+namespace kfac {
+
+struct VecDesc {
+  float* a;
+  float* b;
+  float* c;
+  long numel;
+  float s0, s1, s2, s3;
+};
+
+constexpr int VEC_CHUNK = 64;
+struct VecChunk {
+  VecDesc d[VEC_CHUNK];
+};
+
+__global__ void vec_setup_kernel(VecChunk chunk, VecDesc* table, int offset, int count) {
+  const int i = threadIdx.x;
+  if (i < count) table[offset + i] = chunk.d[i];
+}
+
+enum { OP_AXPBY = 0, OP_DIAG_INV = 1, OP_MUL = 2, OP_SGD = 3 };
+
+constexpr int EW_THREADS = 256;
+constexpr int EW_PER_THREAD = 4;
+constexpr int EW_BLOCK = EW_THREADS * EW_PER_THREAD;
+
+template <int OP>
+__device__ __forceinline__ void apply(const VecDesc& m, long i) {
+  if (OP == OP_AXPBY) {
+    // b = s0 * a + s1 * b     (s1 == 0: b is not read)
+    float v = m.s0 * m.a[i];
+    if (m.s1 != 0.f) v += m.s1 * m.b[i];
+    m.b[i] = v;
+  } else if (OP == OP_DIAG_INV) {
+    // b = 1 / ((s1 ? sqrt(a) : a) + s0)
+    float v = m.a[i];
+    if (m.s1 != 0.f) v = sqrtf(v);
+    m.b[i] = 1.f / (v + m.s0);
+  } else if (OP == OP_MUL) {
+    // b *= a
+    m.b[i] = m.b[i] * m.a[i];
+  } else {
+    // a = param, b = grad, c = momentum buffer; s0 = lr, s1 = momentum, s2 = weight decay
+    float g = m.b[i];
+    const float p = m.a[i];
+    if (m.s2 != 0.f) g += m.s2 * p;
+    if (m.s1 != 0.f) {
+      g = m.s1 * m.c[i] + g;
+      m.c[i] = g;
+    }
+    m.b[i] = g;
+    m.a[i] = p - m.s0 * g;
+  }
+}
+
+template <int OP>
+__global__ __launch_bounds__(EW_THREADS) void vec_kernel(const VecDesc* table) {
+  const VecDesc m = table[blockIdx.y];
+  const long nblocks = (m.numel + EW_BLOCK - 1) / EW_BLOCK;
+  for (long blk = blockIdx.x; blk < nblocks; blk += gridDim.x) {
+    const long base = blk * EW_BLOCK + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < EW_PER_THREAD; ++k) {
+      const long i = base + (long)k * EW_THREADS;
+      if (i < m.numel) apply<OP>(m, i);
+    }
+  }
+}
+
+static size_t vec_workspace(int count) { return (size_t)count * sizeof(VecDesc); }
+
+template <int OP>
+static int run_vec(std::vector<VecDesc>& descs, void* workspace, size_t workspace_bytes,
+                   hipStream_t stream) {
+  const int count = (int)descs.size();
+  if (count == 0) return KFAC_OK;
+  if (!workspace || workspace_bytes < vec_workspace(count)) return KFAC_ERR_WORKSPACE;
+  VecDesc* table = (VecDesc*)workspace;
+  long maxblocks = 1;
+  for (int s0 = 0; s0 < count; s0 += VEC_CHUNK) {
+    VecChunk chunk;
+    const int cnt = std::min(VEC_CHUNK, count - s0);
+    for (int k = 0; k < cnt; ++k) {
+      chunk.d[k] = descs[s0 + k];
+      maxblocks = std::max(maxblocks, (descs[s0 + k].numel + EW_BLOCK - 1) / EW_BLOCK);
+    }
+    hipLaunchKernelGGL(vec_setup_kernel, dim3(1), dim3(VEC_CHUNK), 0, stream, chunk, table, s0,
+                       cnt);
+  }
+  long gx = std::max<long>(64, 4096 / count);
+  gx = std::min(gx, maxblocks);
+  hipLaunchKernelGGL((vec_kernel<OP>), dim3((unsigned)gx, count), dim3(EW_THREADS), 0, stream,
+                     table);
+  return launch_status();
+}
+
+// ---- BatchNorm diagonal curvature ----------------------------------------
+
+// out[row] = sum_i ((x[row][i] - shift[c]) / scale[c])^2, row = (n, c), c = row % C
+__global__ __launch_bounds__(256) void rowsq_kernel(const float* x, const float* scale,
+                                                    const float* shift, int C, int len,
+                                                    float* out) {
+  __shared__ float red[256];
+  const long row = blockIdx.x;
+  const int c = (int)(row % C);
+  const float sh = shift ? shift[c] : 0.f;
+  const float rs = scale ? 1.f / scale[c] : 1.f;
+  const float* p = x + row * (long)len;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < len; i += 256) {
+    const float v = (p[i] - sh) * rs;
+    s += v * v;
+  }
+  red[threadIdx.x] = s;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if (threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[row] = red[0];
+}
+
+// w_curv[c] = alpha * sum_n sx[n][c] * sg[n][c] ; b_curv[c] = alpha * sum_n sg[n][c]
+__global__ void bn_combine_kernel(const float* sx, const float* sg, int N, int C, float alpha,
+                                  float* w_curv, float* b_curv) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  float sw = 0.f, sb = 0.f;
+  for (int n = 0; n < N; ++n) {
+    const float g = sg[(long)n * C + c];
+    sw += sx[(long)n * C + c] * g;
+    sb += g;
+  }
+  w_curv[c] = alpha * sw;
+  if (b_curv) b_curv[c] = alpha * sb;
+}
+
+}  // namespace kfac
+
+using namespace kfac;
+
+extern "C" {
+
+size_t kfac_vector_workspace_bytes(int count) { return count > 0 ? vec_workspace(count) : 0; }
+
+int kfac_axpby_batched(int count, const int64_t* numel, const float* const* x, float* const* y,
+                       float a, float b, void* workspace, size_t workspace_bytes, void* stream) {
+  if (count < 0 || (count > 0 && (!numel || !x || !y))) return KFAC_ERR_ARG;
+  std::vector<VecDesc> d(count);
+  for (int i = 0; i < count; ++i) {
+    if (numel[i] <= 0 || !x[i] || !y[i]) return KFAC_ERR_ARG;
+    d[i] = VecDesc{(float*)x[i], y[i], nullptr, (long)numel[i], a, b, 0.f, 0.f};
+  }
+  return run_vec<OP_AXPBY>(d, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int kfac_diag_inverse_batched(int count, const int64_t* numel, const float* const* ema,
+                              float* const* inv, const float* damping, int use_sqrt,
+                              void* workspace, size_t workspace_bytes, void* stream) {
+  if (count < 0 || (count > 0 && (!numel || !ema || !inv || !damping))) return KFAC_ERR_ARG;
+  std::vector<VecDesc> d(count);
+  for (int i = 0; i < count; ++i) {
+    if (numel[i] <= 0 || !ema[i] || !inv[i]) return KFAC_ERR_ARG;
+    d[i] = VecDesc{(float*)ema[i], inv[i], nullptr, (long)numel[i], damping[i],
+                   use_sqrt ? 1.f : 0.f, 0.f, 0.f};
+  }
+  return run_vec<OP_DIAG_INV>(d, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int kfac_diag_precondition_batched(int count, const int64_t* numel, const float* const* inv,
+                                   float* const* grad, void* workspace, size_t workspace_bytes,
+                                   void* stream) {
+  if (count < 0 || (count > 0 && (!numel || !inv || !grad))) return KFAC_ERR_ARG;
+  std::vector<VecDesc> d(count);
+  for (int i = 0; i < count; ++i) {
+    if (numel[i] <= 0 || !inv[i] || !grad[i]) return KFAC_ERR_ARG;
+    d[i] = VecDesc{(float*)inv[i], grad[i], nullptr, (long)numel[i], 0.f, 0.f, 0.f, 0.f};
+  }
+  return run_vec<OP_MUL>(d, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int kfac_sgd_update_batched(int count, const int64_t* numel, float* const* param,
+                            float* const* grad, float* const* momentum_buf, const float* lr,
+                            const float* momentum, const float* weight_decay, void* workspace,
+                            size_t workspace_bytes, void* stream) {
+  if (count < 0 || (count > 0 && (!numel || !param || !grad || !lr || !momentum || !weight_decay)))
+    return KFAC_ERR_ARG;
+  std::vector<VecDesc> d(count);
+  for (int i = 0; i < count; ++i) {
+    if (numel[i] <= 0 || !param[i] || !grad[i]) return KFAC_ERR_ARG;
+    if (momentum[i] != 0.f && (!momentum_buf || !momentum_buf[i])) return KFAC_ERR_ARG;
+    d[i] = VecDesc{param[i], grad[i], momentum_buf ? momentum_buf[i] : nullptr, (long)numel[i],
+                   lr[i], momentum[i], weight_decay[i], 0.f};
+  }
+  return run_vec<OP_SGD>(d, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int kfac_rowsq_sum(const float* x, int64_t rows, int channels, int len, const float* scale,
+                   const float* shift, float* out, void* stream) {
+  if (!x || !out || rows <= 0 || channels <= 0 || len <= 0 || rows >= (int64_t)1 << 31)
+    return KFAC_ERR_ARG;
+  hipLaunchKernelGGL(rowsq_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, x,
+                     scale, shift, channels, len, out);
+  return launch_status();
+}
+
+int kfac_bn_diag_combine(const float* sx, const float* sg, int n, int channels, float alpha,
+                         float* w_curv, float* b_curv, void* stream) {
+  if (!sx || !sg || !w_curv || n <= 0 || channels <= 0) return KFAC_ERR_ARG;
+  hipLaunchKernelGGL(bn_combine_kernel, dim3(cdiv(channels, 128)), dim3(128), 0,
+                     (hipStream_t)stream, sx, sg, n, channels, alpha, w_curv, b_curv);
+  return launch_status();
+}
+
+}  // extern "C"

@@ -38,6 +38,8 @@ constexpr int SMEM_FLOATS = 4 * TILE_FLOATS;  // 2 operands x 2 stages = 40 KiB
 
 enum { KM = 0, MK = 1 };
 
+__host__ __device__ inline int tiles128(int d) { return (d + BM - 1) / BM; }
+
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 // ---------------------------------------------------------------------------

@@ -1,0 +1,534 @@
+// Batched damped SPD inverse:  dst_i = (src_i + damp_i * I)^-1  for a whole set
+// of matrices of different sizes in one sequence of launches.
+//
+//   1. copy the upper triangle of src into dst and add damp to the diagonal
+//      (damp is either given, or computed on the device from the traces of a
+//      pair of Kronecker factors: the pi-damping split);
+//   2. blocked right-looking Cholesky  S = U^T U  (upper, in place in dst) with
+//      128-wide panels: one workgroup factors AND inverts the 128x128 diagonal
+//      block in LDS; the row panel is a product with that small inverse; the
+//      trailing update is a symmetric rank-128 product on the MFMA tile engine;
+//   3. Y = U^-1 by recursive doubling over the 128-blocks:
+//      Y12 = -Y11 * U12 * Y22, two MFMA products per level, log2(n/128) levels;
+//   4. dst = Y Y^T on the MFMA tile engine (upper tiles, mirrored).
+//
+// Every launch covers all matrices that still have work at that step (matrices
+// are processed in descending size order so the active ones form a prefix),
+// so small factors ride along with the large ones instead of getting a launch
+// sequence each.
+#include <algorithm>
+#include <vector>
+
+#include "common.h"
+#include "operands.h"
+
+namespace kfac {
+
+struct MatDesc {
+  const float* src;
+  float* U;      // = dst
+  float* Y;      // workspace, n*n
+  int n;
+  int T;         // number of 128-blocks
+  float damp;    // given damping, or sqrt(damping) in pi mode
+  int partner;   // -1: damp is final; else index of the other factor of the pair
+  int is_a;      // pi mode: 1 -> damp*pi, 0 -> damp/pi
+  int out;       // position in the caller's info array
+  float trace;
+  int pad;
+};
+
+constexpr int SETUP_CHUNK = 64;
+struct DescChunk {
+  MatDesc d[SETUP_CHUNK];
+};
+
+__global__ void inv_setup_kernel(DescChunk chunk, MatDesc* table, int offset, int count) {
+  const int i = threadIdx.x;
+  if (i < count) table[offset + i] = chunk.d[i];
+}
+
+// trace of src (one workgroup per matrix)
+__global__ __launch_bounds__(256) void inv_trace_kernel(MatDesc* table) {
+  __shared__ float red[256];
+  MatDesc& m = table[blockIdx.x];
+  const int n = m.n;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < n; i += 256) s += m.src[(size_t)i * n + i];
+  red[threadIdx.x] = s;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if (threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) m.trace = red[0];
+}
+
+__device__ __forceinline__ float effective_damp(const MatDesc* table, const MatDesc& m) {
+  if (m.partner < 0) return m.damp;
+  const MatDesc& o = table[m.partner];
+  const float ta = m.is_a ? m.trace / m.n : o.trace / o.n;
+  const float tg = m.is_a ? o.trace / o.n : m.trace / m.n;
+  const float pi = sqrtf(ta / tg);
+  return m.is_a ? m.damp * pi : m.damp / pi;
+}
+
+// U = upper tiles of (src + damp I); also clears info
+__global__ __launch_bounds__(256) void inv_copy_damp_kernel(const MatDesc* table, int* info) {
+  const MatDesc m = table[blockIdx.y];
+  const int ntiles = m.T * (m.T + 1) / 2;
+  if ((int)blockIdx.x >= ntiles) return;
+  if (blockIdx.x == 0 && threadIdx.x == 0) info[m.out] = 0;
+  int bi, bj;
+  upper_tile(blockIdx.x, m.T, bi, bj);
+  const float damp = effective_damp(table, m);
+  const int n = m.n;
+  for (int e = threadIdx.x; e < BM * BN; e += 256) {
+    const int row = bi * BM + (e >> 7);
+    const int col = bj * BN + (e & 127);
+    if (row < n && col < n) {
+      float v = m.src[(size_t)row * n + col];
+      if (row == col) v += damp;
+      m.U[(size_t)row * n + col] = v;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// 128x128 diagonal block: Cholesky (upper) and its inverse, in LDS.
+// ---------------------------------------------------------------------------
+constexpr int DB = 128;          // diagonal block size
+constexpr int DLD = DB + 1;      // LDS leading dimension
+constexpr int WLD = 65;
+constexpr int DIAG_SMEM_BYTES = (2 * DB * DLD + 64 * WLD) * (int)sizeof(float);
+
+__device__ __forceinline__ float bcast(float v, int lane) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+// One wave factors the 32x32 block at (c0, c0) of S in registers (lane j holds
+// column j), inverts the factor, and writes U_qq to S and Y_qq to Yb.
+__device__ __forceinline__ void chol_inv_32(float* S, float* Yb, int c0, int row_base, int* info) {
+  const int lane = threadIdx.x & 63;
+  const int j = lane & 31;
+  float a[32];
+#pragma unroll
+  for (int i = 0; i < 32; ++i) a[i] = S[(c0 + i) * DLD + c0 + j];
+  int bad = 0;
+#pragma unroll
+  for (int c = 0; c < 32; ++c) {
+    const float piv = bcast(a[c], c);
+    if (!(piv > 0.f) && bad == 0) bad = row_base + c0 + c + 1;
+    const float d = sqrtf(piv);
+    const float rd = 1.f / d;
+    float ucj = (j >= c) ? a[c] * rd : 0.f;
+    if (j == c) ucj = d;
+    a[c] = ucj;
+#pragma unroll
+    for (int i = c + 1; i < 32; ++i) {
+      const float uci = bcast(ucj, i);
+      a[i] -= uci * ucj;
+    }
+  }
+  if (bad != 0 && lane == 0) {
+    if (*info == 0) *info = bad;
+  }
+  // inverse by back substitution, column j of Y in lane j
+  float y[32];
+#pragma unroll
+  for (int i = 31; i >= 0; --i) {
+    float s = (j == i) ? 1.f : 0.f;
+#pragma unroll
+    for (int k = i + 1; k < 32; ++k) s -= bcast(a[i], k) * y[k];
+    y[i] = s / bcast(a[i], i);
+  }
+  if (lane < 32) {
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      S[(c0 + i) * DLD + c0 + j] = (i <= j) ? a[i] : 0.f;
+      Yb[(c0 + i) * DLD + c0 + j] = (i <= j) ? y[i] : 0.f;
+    }
+  }
+}
+
+// In-LDS off-diagonal inverse block:  Y12 = -Y11 * (U12 * Y22) for the pair
+// X1 = [s1, s1+b), X2 = [s1+b, s1+2b);  W is a b x b scratch (b <= 64).
+__device__ __forceinline__ void tri_pair(const float* S, float* Yb, float* Wt, int s1, int b) {
+  const int s2 = s1 + b;
+  const int t = threadIdx.x;
+  // W[i][j] = sum_{k<=j} U12[i][k] * Y22[k][j]
+  for (int e = t; e < b * b; e += 256) {
+    const int i = e / b, j = e - i * b;
+    float s = 0.f;
+    for (int k = 0; k <= j; ++k) s += S[(s1 + i) * DLD + s2 + k] * Yb[(s2 + k) * DLD + s2 + j];
+    Wt[i * WLD + j] = s;
+  }
+  __syncthreads();
+  // Y12[i][j] = - sum_{k>=i} Y11[i][k] * W[k][j]
+  for (int e = t; e < b * b; e += 256) {
+    const int i = e / b, j = e - i * b;
+    float s = 0.f;
+    for (int k = i; k < b; ++k) s += Yb[(s1 + i) * DLD + s1 + k] * Wt[k * WLD + j];
+    Yb[(s1 + i) * DLD + s2 + j] = -s;
+  }
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, int p, int* info) {
+  extern __shared__ __attribute__((aligned(16))) float dsm[];
+  float* S = dsm;
+  float* Yb = dsm + DB * DLD;
+  float* Wt = dsm + 2 * DB * DLD;
+  const MatDesc m = table[blockIdx.x];
+  const int n = m.n;
+  const int r0 = p * DB;
+  const int nb = min(DB, n - r0);
+  const int t = threadIdx.x;
+
+  // load the upper triangle; pad with the identity up to the next multiple of 32
+  for (int e = t; e < DB * DB; e += 256) {
+    const int i = e >> 7, j = e & 127;
+    float v = 0.f;
+    if (i < nb && j < nb) {
+      if (j >= i) v = m.U[(size_t)(r0 + i) * n + r0 + j];
+    } else if (i == j) {
+      v = 1.f;
+    }
+    S[i * DLD + j] = v;
+    Yb[i * DLD + j] = 0.f;
+  }
+  __syncthreads();
+
+  const int nq = (nb + 31) / 32;
+  for (int q = 0; q < nq; ++q) {
+    const int c0 = 32 * q;
+    if (t < 64) chol_inv_32(S, Yb, c0, r0, info + m.out);
+    __syncthreads();
+    const int c1 = c0 + 32;
+    const int rest = 32 * nq - c1;   // columns to the right
+    if (rest > 0) {
+      // row panel: U[c0+i][c1+j] = sum_k Yqq[k][i] * A[c0+k][c1+j]   (k <= i)
+      float out[12];
+      int cnt = 0;
+      for (int e = t; e < 32 * rest; e += 256, ++cnt) {
+        const int i = e / rest, jj = e - i * rest;
+        float s = 0.f;
+        for (int k = 0; k <= i; ++k) s += Yb[(c0 + k) * DLD + c0 + i] * S[(c0 + k) * DLD + c1 + jj];
+        out[cnt] = s;
+      }
+      __syncthreads();
+      cnt = 0;
+      for (int e = t; e < 32 * rest; e += 256, ++cnt) {
+        const int i = e / rest, jj = e - i * rest;
+        S[(c0 + i) * DLD + c1 + jj] = out[cnt];
+      }
+      __syncthreads();
+      // trailing update: A[c1+i][c1+j] -= sum_k U[c0+k][c1+i] * U[c0+k][c1+j],  j >= i
+      for (int e = t; e < rest * rest; e += 256) {
+        const int i = e / rest, jj = e - i * rest;
+        if (jj >= i) {
+          float s = 0.f;
+#pragma unroll 8
+          for (int k = 0; k < 32; ++k) s += S[(c0 + k) * DLD + c1 + i] * S[(c0 + k) * DLD + c1 + jj];
+          S[(c1 + i) * DLD + c1 + jj] -= s;
+        }
+      }
+      __syncthreads();
+    }
+  }
+
+  // inverse of the whole block by doubling: 32 -> 64 -> 128
+  if (nq > 1) {
+    tri_pair(S, Yb, Wt, 0, 32);
+    if (nq > 3) tri_pair(S, Yb, Wt, 64, 32);
+    else if (nq > 2) { /* X2 of the second pair is padding: nothing to do */ }
+  }
+  if (nq > 2) tri_pair(S, Yb, Wt, 0, 64);
+
+  for (int e = t; e < DB * DB; e += 256) {
+    const int i = e >> 7, j = e & 127;
+    if (i < nb && j < nb) {
+      m.U[(size_t)(r0 + i) * n + r0 + j] = S[i * DLD + j];
+      m.Y[(size_t)(r0 + i) * n + r0 + j] = Yb[i * DLD + j];
+    }
+  }
+}
+
+// row panel of the blocked Cholesky: U[p, j] = Ypp^T * A[p, j], j > p
+__global__ __launch_bounds__(NTHREADS) void potrf_panel_kernel(const MatDesc* table, int p) {
+  __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
+  const MatDesc m = table[blockIdx.y];
+  const int bj = p + 1 + blockIdx.x;
+  if (bj >= m.T) return;
+  const int n = m.n;
+  const int r0 = p * DB;
+  DenseKM P{m.Y + (size_t)r0 * n + r0, nullptr, n, DB, 0};
+  DenseKM Q{m.U + (size_t)r0 * n, nullptr, n, n, 0};
+  EpiStore epi{m.U + (size_t)r0 * n, n, DB, n, 1.f, 0.f, false};
+  gemm_tile(P, Q, 0, bj * BN, 0, DB, false, epi, smem);
+}
+
+// trailing update: A[i, j] -= U[p, i]^T U[p, j],  p < i <= j
+__global__ __launch_bounds__(NTHREADS) void potrf_trail_kernel(const MatDesc* table, int p) {
+  __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
+  const MatDesc m = table[blockIdx.y];
+  const int Tr = m.T - p - 1;
+  if (Tr <= 0) return;
+  const int ntiles = Tr * (Tr + 1) / 2;
+  if ((int)blockIdx.x >= ntiles) return;
+  int bi, bj;
+  upper_tile(blockIdx.x, Tr, bi, bj);
+  bi += p + 1;
+  bj += p + 1;
+  const int n = m.n;
+  DenseKM P{m.U + (size_t)p * DB * n, nullptr, n, n, 0};
+  EpiStore epi{m.U, n, n, n, -1.f, 1.f, false};
+  gemm_tile(P, P, bi * BM, bj * BN, 0, DB, bi == bj, epi, smem);
+}
+
+// level l of the doubling inverse, first product:
+//   W^T[j][i] = sum_{k <= j} Y22[k][j] * U12[i][k]   stored at Y[X2 rows][X1 cols]
+__global__ __launch_bounds__(NTHREADS) void trtri_w_kernel(const MatDesc* table, int l) {
+  __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
+  const MatDesc m = table[blockIdx.y];
+  const int tl = 1 << l;                     // 128-blocks per half
+  const int pair = blockIdx.x >> (2 * l);
+  const int within = blockIdx.x & ((1 << (2 * l)) - 1);
+  const int it = within >> l, jt = within & (tl - 1);
+  const int s1 = pair * 2 * tl, s2 = s1 + tl;   // in 128-blocks
+  if (s2 + jt >= m.T) return;
+  const int n = m.n;
+  const int X1 = s1 * DB, X2 = s2 * DB;
+  const int b1 = tl * DB;
+  const int b2 = min(b1, n - X2);
+  DenseKM P{m.Y + (size_t)X2 * n + X2, nullptr, n, b2, 0};
+  DenseMK Q{m.U + (size_t)X1 * n + X2, n, b1};
+  EpiStore epi{m.Y + (size_t)X2 * n + X1, n, b2, b1, 1.f, 0.f, false};
+  gemm_tile(P, Q, jt * BM, it * BN, 0, min(b2, (jt + 1) * DB), false, epi, smem);
+}
+
+// second product:  Y12[i][j] = - sum_{k >= i} Y11[i][k] * W^T[j][k]
+__global__ __launch_bounds__(NTHREADS) void trtri_y_kernel(const MatDesc* table, int l) {
+  __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
+  const MatDesc m = table[blockIdx.y];
+  const int tl = 1 << l;
+  const int pair = blockIdx.x >> (2 * l);
+  const int within = blockIdx.x & ((1 << (2 * l)) - 1);
+  const int it = within >> l, jt = within & (tl - 1);
+  const int s1 = pair * 2 * tl, s2 = s1 + tl;
+  if (s2 + jt >= m.T) return;
+  const int n = m.n;
+  const int X1 = s1 * DB, X2 = s2 * DB;
+  const int b1 = tl * DB;
+  const int b2 = min(b1, n - X2);
+  DenseMK P{m.Y + (size_t)X1 * n + X1, n, b1};
+  DenseMK Q{m.Y + (size_t)X2 * n + X1, n, b2};
+  EpiStore epi{m.Y + (size_t)X1 * n + X2, n, b1, b2, -1.f, 0.f, false};
+  gemm_tile(P, Q, it * BM, jt * BN, it * DB, b1, false, epi, smem);
+}
+
+// dst = Y Y^T over the upper tiles (k >= the later block), mirrored
+__global__ __launch_bounds__(NTHREADS) void lauum_kernel(const MatDesc* table) {
+  __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
+  const MatDesc m = table[blockIdx.y];
+  const int ntiles = m.T * (m.T + 1) / 2;
+  if ((int)blockIdx.x >= ntiles) return;
+  int bi, bj;
+  upper_tile(blockIdx.x, m.T, bi, bj);
+  const int n = m.n;
+  DenseMK P{m.Y, n, n};
+  EpiStore epi{m.U, n, n, n, 1.f, 0.f, bi != bj};
+  gemm_tile(P, P, bi * BM, bj * BN, bj * DB, n, bi == bj, epi, smem);
+}
+
+// zero the strictly lower triangle (Cholesky-factor output)
+__global__ __launch_bounds__(256) void zero_lower_kernel(const MatDesc* table) {
+  const MatDesc m = table[blockIdx.y];
+  const int n = m.n;
+  const int T = m.T;
+  if ((int)blockIdx.x >= T * T) return;
+  const int bi = blockIdx.x / T, bj = blockIdx.x - bi * T;
+  if (bj > bi) return;
+  for (int e = threadIdx.x; e < BM * BN; e += 256) {
+    const int row = bi * BM + (e >> 7);
+    const int col = bj * BN + (e & 127);
+    if (row < n && col < n && col < row) m.U[(size_t)row * n + col] = 0.f;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct HostMat {
+  const float* src;
+  float* dst;
+  int n;
+  float damp;
+  int partner;   // index in caller order, or -1
+  int is_a;
+  int out;
+};
+
+static size_t inverse_workspace_bytes(const std::vector<int>& dims) {
+  size_t bytes = align256(dims.size() * sizeof(MatDesc));
+  for (int n : dims) bytes += align256((size_t)n * n * sizeof(float));
+  return bytes;
+}
+
+enum { MODE_INVERSE = 0, MODE_CHOLESKY = 1 };
+
+static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* workspace,
+                       size_t workspace_bytes, hipStream_t stream) {
+  const int nmat = (int)mats.size();
+  if (nmat == 0) return KFAC_OK;
+  std::vector<int> dims(nmat);
+  for (int i = 0; i < nmat; ++i) dims[i] = mats[i].n;
+  if (workspace == nullptr || workspace_bytes < inverse_workspace_bytes(dims))
+    return KFAC_ERR_WORKSPACE;
+
+  // the diagonal-block kernel needs more than the default 64 KiB of LDS
+  if (hipFuncSetAttribute((const void*)potrf_diag_kernel,
+                          hipFuncAttributeMaxDynamicSharedMemorySize,
+                          DIAG_SMEM_BYTES) != hipSuccess)
+    return KFAC_ERR_LAUNCH;
+
+  // descending size order; remember where each caller index went
+  std::vector<int> order(nmat);
+  for (int i = 0; i < nmat; ++i) order[i] = i;
+  std::stable_sort(order.begin(), order.end(),
+                   [&](int a, int b) { return mats[a].n > mats[b].n; });
+  std::vector<int> pos(nmat);
+  for (int s = 0; s < nmat; ++s) pos[order[s]] = s;
+
+  MatDesc* table = (MatDesc*)workspace;
+  char* ybase = (char*)workspace + align256(nmat * sizeof(MatDesc));
+  size_t yoff = 0;
+  int Tmax = 0;
+  std::vector<int> Ts(nmat);
+  for (int s0 = 0; s0 < nmat; s0 += SETUP_CHUNK) {
+    DescChunk chunk;
+    const int cnt = std::min(SETUP_CHUNK, nmat - s0);
+    for (int k = 0; k < cnt; ++k) {
+      const HostMat& h = mats[order[s0 + k]];
+      MatDesc& d = chunk.d[k];
+      d.src = h.src;
+      d.U = h.dst;
+      d.Y = (float*)(ybase + yoff);
+      yoff += align256((size_t)h.n * h.n * sizeof(float));
+      d.n = h.n;
+      d.T = cdiv(h.n, DB);
+      d.damp = h.damp;
+      d.partner = h.partner < 0 ? -1 : pos[h.partner];
+      d.is_a = h.is_a;
+      d.out = h.out;
+      d.trace = 0.f;
+      d.pad = 0;
+      Ts[s0 + k] = d.T;
+      Tmax = std::max(Tmax, d.T);
+    }
+    hipLaunchKernelGGL(inv_setup_kernel, dim3(1), dim3(SETUP_CHUNK), 0, stream, chunk, table, s0,
+                       cnt);
+  }
+  auto active = [&](int minT) {   // matrices with T >= minT (a prefix of the sorted table)
+    int c = 0;
+    while (c < nmat && Ts[c] >= minT) ++c;
+    return c;
+  };
+
+  bool any_pi = false;
+  for (auto& h : mats) any_pi |= h.partner >= 0;
+  if (any_pi) hipLaunchKernelGGL(inv_trace_kernel, dim3(nmat), dim3(256), 0, stream, table);
+  hipLaunchKernelGGL(inv_copy_damp_kernel, dim3(Tmax * (Tmax + 1) / 2, nmat), dim3(256), 0, stream,
+                     table, info);
+
+  for (int p = 0; p < Tmax; ++p) {
+    const int na = active(p + 1);
+    hipLaunchKernelGGL(potrf_diag_kernel, dim3(na), dim3(256), DIAG_SMEM_BYTES, stream, table, p,
+                       info);
+    const int nb = active(p + 2);
+    if (nb > 0) {
+      const int Tr = Tmax - p - 1;
+      hipLaunchKernelGGL(potrf_panel_kernel, dim3(Tr, nb), dim3(NTHREADS), 0, stream, table, p);
+      hipLaunchKernelGGL(potrf_trail_kernel, dim3(Tr * (Tr + 1) / 2, nb), dim3(NTHREADS), 0,
+                         stream, table, p);
+    }
+  }
+  if (mode == MODE_CHOLESKY) {
+    hipLaunchKernelGGL(zero_lower_kernel, dim3(Tmax * Tmax, nmat), dim3(256), 0, stream, table);
+    return launch_status();
+  }
+  for (int l = 0; (1 << l) < Tmax; ++l) {
+    const int na = active((1 << l) + 1);
+    if (na == 0) break;
+    const int npairs = cdiv(Tmax, 2 << l);
+    const dim3 grid(npairs << (2 * l), na);
+    hipLaunchKernelGGL(trtri_w_kernel, grid, dim3(NTHREADS), 0, stream, table, l);
+    hipLaunchKernelGGL(trtri_y_kernel, grid, dim3(NTHREADS), 0, stream, table, l);
+  }
+  hipLaunchKernelGGL(lauum_kernel, dim3(Tmax * (Tmax + 1) / 2, nmat), dim3(NTHREADS), 0, stream,
+                     table);
+  return launch_status();
+}
+
+}  // namespace kfac
+
+using namespace kfac;
+
+extern "C" {
+
+size_t kfac_inverse_workspace_bytes(int count, const int* dims) {
+  if (count <= 0 || !dims) return 0;
+  std::vector<int> d(dims, dims + count);
+  for (int n : d)
+    if (n <= 0) return 0;
+  return inverse_workspace_bytes(d);
+}
+
+int kfac_damped_inverse_batched(int count, const int* dims, const float* const* src,
+                                const float* damp, float* const* dst, int* info,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+  if (count < 0 || (count > 0 && (!dims || !src || !dst || !info))) return KFAC_ERR_ARG;
+  std::vector<HostMat> mats(count);
+  for (int i = 0; i < count; ++i) {
+    if (dims[i] <= 0 || dims[i] > 46340 || !src[i] || !dst[i] || src[i] == dst[i])
+      return KFAC_ERR_ARG;
+    mats[i] = HostMat{src[i], dst[i], dims[i], damp ? damp[i] : 0.f, -1, 0, i};
+  }
+  return run_batched(mats, MODE_INVERSE, info, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int kfac_pi_damped_inverse_batched(int layers, const int* dA, const int* dG,
+                                   const float* const* A, const float* const* G,
+                                   const float* damping, float* const* Ainv, float* const* Ginv,
+                                   int* info, void* workspace, size_t workspace_bytes,
+                                   void* stream) {
+  if (layers < 0 || (layers > 0 && (!dA || !dG || !A || !G || !damping || !Ainv || !Ginv || !info)))
+    return KFAC_ERR_ARG;
+  std::vector<HostMat> mats(2 * layers);
+  for (int l = 0; l < layers; ++l) {
+    if (dA[l] <= 0 || dG[l] <= 0 || dA[l] > 46340 || dG[l] > 46340 || !A[l] || !G[l] ||
+        !Ainv[l] || !Ginv[l] || A[l] == Ainv[l] || G[l] == Ginv[l] || !(damping[l] >= 0.f))
+      return KFAC_ERR_ARG;
+    const float r = sqrtf(damping[l]);
+    mats[2 * l] = HostMat{A[l], Ainv[l], dA[l], r, 2 * l + 1, 1, 2 * l};
+    mats[2 * l + 1] = HostMat{G[l], Ginv[l], dG[l], r, 2 * l, 0, 2 * l + 1};
+  }
+  return run_batched(mats, MODE_INVERSE, info, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int kfac_cholesky_upper_batched(int count, const int* dims, const float* const* src,
+                                float* const* dst, int* info, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+  if (count < 0 || (count > 0 && (!dims || !src || !dst || !info))) return KFAC_ERR_ARG;
+  std::vector<HostMat> mats(count);
+  for (int i = 0; i < count; ++i) {
+    if (dims[i] <= 0 || dims[i] > 46340 || !src[i] || !dst[i] || src[i] == dst[i])
+      return KFAC_ERR_ARG;
+    mats[i] = HostMat{src[i], dst[i], dims[i], 0.f, -1, 0, i};
+  }
+  return run_batched(mats, MODE_CHOLESKY, info, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -42,7 +42,55 @@ _SIGNATURES = {
                                                            c_ptr, c_size, c_ptr]),
     'kfac_factor_conv_g': (c_int, [c_ptr, c_int, c_int, c_int, c_int, c_f32, c_f32, c_ptr,
                                    c_ptr, c_size, c_ptr]),
+    'kfac_inverse_workspace_bytes': (c_size, [c_int, c_ptr]),
+    'kfac_pi_damped_inverse_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
+                                               c_ptr, c_ptr, c_ptr, c_size, c_ptr]),
+    'kfac_damped_inverse_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
+                                            c_ptr, c_size, c_ptr]),
+    'kfac_cholesky_upper_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr,
+                                            c_ptr, c_size, c_ptr]),
+    'kfac_precondition_workspace_bytes': (c_size, [c_int, c_ptr, c_ptr]),
+    'kfac_precondition_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
+                                          c_ptr, c_size, c_ptr]),
+    'kfac_sample_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
+                                    c_ptr, c_ptr, c_f32, c_ptr, c_size, c_ptr]),
+    'kfac_vector_workspace_bytes': (c_size, [c_int]),
+    'kfac_axpby_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_f32, c_f32,
+                                   c_ptr, c_size, c_ptr]),
+    'kfac_diag_inverse_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_int,
+                                          c_ptr, c_size, c_ptr]),
+    'kfac_diag_precondition_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr,
+                                               c_ptr, c_size, c_ptr]),
+    'kfac_sgd_update_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
+                                        c_ptr, c_size, c_ptr]),
+    'kfac_rowsq_sum': (c_int, [c_ptr, c_i64, c_int, c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
+    'kfac_bn_diag_combine': (c_int, [c_ptr, c_ptr, c_int, c_int, c_f32, c_ptr, c_ptr, c_ptr]),
 }
+
+
+def int_array(values):
+    return (ctypes.c_int * len(values))(*[int(v) for v in values])
+
+
+def i64_array(values):
+    return (ctypes.c_int64 * len(values))(*[int(v) for v in values])
+
+
+def f32_array(values):
+    return (ctypes.c_float * len(values))(*[float(v) for v in values])
+
+
+def ptr_array(tensors, what='tensor', allow_none=False):
+    """Host array of device addresses (0 for None when allowed)."""
+    out = (ctypes.c_void_p * len(tensors))()
+    for i, t in enumerate(tensors):
+        if t is None:
+            if not allow_none:
+                raise KfacHipError('%s %d is None' % (what, i))
+            out[i] = None
+        else:
+            out[i] = dev_ptr(t, '%s %d' % (what, i))
+    return out
 
 
 def signatures():

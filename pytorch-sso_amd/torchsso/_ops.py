@@ -84,3 +84,247 @@ def factor_conv_g(g, alpha, out=None, beta=0.):
                                 _hip.stream_ptr(g.device))
     _hip.check(st, 'kfac_factor_conv_g')
     return out
+
+
+def _ws_ptr(ws):
+    return None if ws is None else ws.data_ptr()
+
+
+def _square_dims(mats, what):
+    dims = []
+    for i, m in enumerate(mats):
+        if m.dim() != 2 or m.shape[0] != m.shape[1]:
+            raise _hip.KfacHipError('%s %d is not square: %s' % (what, i, tuple(m.shape)))
+        dims.append(m.shape[0])
+    return dims
+
+
+def pi_damped_inverse_batched(As, Gs, dampings, A_invs=None, G_invs=None, info=None):
+    """A_inv, G_inv = (A + sqrt(d)*pi*I)^-1, (G + sqrt(d)/pi*I)^-1 for every layer.
+
+    Returns (A_invs, G_invs, info) with info a device int32 tensor of 2*layers
+    (nothing is synchronised; read it when you want to know)."""
+    lib = _hip.load()
+    layers = len(As)
+    if layers == 0:
+        return [], [], None
+    dev = As[0].device
+    dA = _square_dims(As, 'A')
+    dG = _square_dims(Gs, 'G')
+    if A_invs is None:
+        A_invs = [torch.empty_like(a) for a in As]
+    if G_invs is None:
+        G_invs = [torch.empty_like(g) for g in Gs]
+    if info is None:
+        info = torch.empty(2 * layers, dtype=torch.int32, device=dev)
+    dims = []
+    for a, g in zip(dA, dG):
+        dims += [a, g]
+    ws, ws_bytes = _hip.workspace(dev, lib.kfac_inverse_workspace_bytes(len(dims), _hip.int_array(dims)))
+    st = lib.kfac_pi_damped_inverse_batched(
+        layers, _hip.int_array(dA), _hip.int_array(dG), _hip.ptr_array(As, 'A'),
+        _hip.ptr_array(Gs, 'G'), _hip.f32_array(dampings), _hip.ptr_array(A_invs, 'A_inv'),
+        _hip.ptr_array(G_invs, 'G_inv'), info.data_ptr(), _ws_ptr(ws), ws_bytes,
+        _hip.stream_ptr(dev))
+    _hip.check(st, 'kfac_pi_damped_inverse_batched')
+    return A_invs, G_invs, info
+
+
+def damped_inverse_batched(mats, damps=None, outs=None, info=None):
+    """outs[i] = (mats[i] + damps[i]*I)^-1."""
+    lib = _hip.load()
+    count = len(mats)
+    if count == 0:
+        return [], None
+    dev = mats[0].device
+    dims = _square_dims(mats, 'matrix')
+    if outs is None:
+        outs = [torch.empty_like(m) for m in mats]
+    if info is None:
+        info = torch.empty(count, dtype=torch.int32, device=dev)
+    ws, ws_bytes = _hip.workspace(dev, lib.kfac_inverse_workspace_bytes(count, _hip.int_array(dims)))
+    st = lib.kfac_damped_inverse_batched(
+        count, _hip.int_array(dims), _hip.ptr_array(mats, 'matrix'),
+        None if damps is None else _hip.f32_array(damps), _hip.ptr_array(outs, 'inverse'),
+        info.data_ptr(), _ws_ptr(ws), ws_bytes, _hip.stream_ptr(dev))
+    _hip.check(st, 'kfac_damped_inverse_batched')
+    return outs, info
+
+
+def cholesky_upper_batched(mats, outs=None, info=None):
+    """outs[i] = U upper triangular with mats[i] = U^T U."""
+    lib = _hip.load()
+    count = len(mats)
+    if count == 0:
+        return [], None
+    dev = mats[0].device
+    dims = _square_dims(mats, 'matrix')
+    if outs is None:
+        outs = [torch.empty_like(m) for m in mats]
+    if info is None:
+        info = torch.empty(count, dtype=torch.int32, device=dev)
+    ws, ws_bytes = _hip.workspace(dev, lib.kfac_inverse_workspace_bytes(count, _hip.int_array(dims)))
+    st = lib.kfac_cholesky_upper_batched(
+        count, _hip.int_array(dims), _hip.ptr_array(mats, 'matrix'), _hip.ptr_array(outs, 'factor'),
+        info.data_ptr(), _ws_ptr(ws), ws_bytes, _hip.stream_ptr(dev))
+    _hip.check(st, 'kfac_cholesky_upper_batched')
+    return outs, info
+
+
+def _kron_dims(Ls, Rs, Ws, bs, what):
+    dG, dA = [], []
+    for l, (L, R, W, b) in enumerate(zip(Ls, Rs, Ws, bs)):
+        g, a = L.shape[0], R.shape[0]
+        aw = a - (0 if b is None else 1)
+        if W.numel() != g * aw or W.shape[0] != g:
+            raise _hip.KfacHipError('%s layer %d: weight-shaped tensor %s does not match factors '
+                                    '(%d, %d)' % (what, l, tuple(W.shape), g, a))
+        if b is not None and b.numel() != g:
+            raise _hip.KfacHipError('%s layer %d: bias-shaped tensor has %d elements, expected %d'
+                                    % (what, l, b.numel(), g))
+        dG.append(g)
+        dA.append(a)
+    return dG, dA
+
+
+def precondition_batched(G_invs, A_invs, grad_ws, grad_bs):
+    """[gW | gb] <- G_inv [gW | gb] A_inv in place for every layer (gb may be None)."""
+    lib = _hip.load()
+    layers = len(G_invs)
+    if layers == 0:
+        return
+    dev = G_invs[0].device
+    _square_dims(G_invs, 'G_inv')
+    _square_dims(A_invs, 'A_inv')
+    dG, dA = _kron_dims(G_invs, A_invs, grad_ws, grad_bs, 'precondition')
+    dGa, dAa = _hip.int_array(dG), _hip.int_array(dA)
+    ws, ws_bytes = _hip.workspace(dev, lib.kfac_precondition_workspace_bytes(layers, dGa, dAa))
+    st = lib.kfac_precondition_batched(
+        layers, dGa, dAa, _hip.ptr_array(G_invs, 'G_inv'), _hip.ptr_array(A_invs, 'A_inv'),
+        _hip.ptr_array(grad_ws, 'weight grad'), _hip.ptr_array(grad_bs, 'bias grad', True),
+        _ws_ptr(ws), ws_bytes, _hip.stream_ptr(dev))
+    _hip.check(st, 'kfac_precondition_batched')
+
+
+def sample_batched(U_Gs, U_As, noises, mean_ws, mean_bs, param_ws, param_bs, std_scale):
+    """[pW | pb] = [mW | mb] + std_scale * U_G @ noise @ U_A for every layer."""
+    lib = _hip.load()
+    layers = len(U_Gs)
+    if layers == 0:
+        return
+    dev = U_Gs[0].device
+    _square_dims(U_Gs, 'U_G')
+    _square_dims(U_As, 'U_A')
+    dG, dA = _kron_dims(U_Gs, U_As, param_ws, param_bs, 'sample')
+    for l, e in enumerate(noises):
+        if tuple(e.shape) != (dG[l], dA[l]):
+            raise _hip.KfacHipError('noise %d has shape %s, expected (%d, %d)'
+                                    % (l, tuple(e.shape), dG[l], dA[l]))
+    dGa, dAa = _hip.int_array(dG), _hip.int_array(dA)
+    ws, ws_bytes = _hip.workspace(dev, lib.kfac_precondition_workspace_bytes(layers, dGa, dAa))
+    st = lib.kfac_sample_batched(
+        layers, dGa, dAa, _hip.ptr_array(U_Gs, 'U_G'), _hip.ptr_array(U_As, 'U_A'),
+        _hip.ptr_array(noises, 'noise'), _hip.ptr_array(mean_ws, 'mean weight'),
+        _hip.ptr_array(mean_bs, 'mean bias', True), _hip.ptr_array(param_ws, 'weight'),
+        _hip.ptr_array(param_bs, 'bias', True), float(std_scale), _ws_ptr(ws), ws_bytes,
+        _hip.stream_ptr(dev))
+    _hip.check(st, 'kfac_sample_batched')
+
+
+def _vec_args(lib, tensors):
+    dev = tensors[0].device
+    numel = _hip.i64_array([t.numel() for t in tensors])
+    ws, ws_bytes = _hip.workspace(dev, lib.kfac_vector_workspace_bytes(len(tensors)))
+    return dev, numel, ws, ws_bytes
+
+
+def _check_same_numel(xs, ys, what):
+    for i, (x, y) in enumerate(zip(xs, ys)):
+        if x.numel() != y.numel():
+            raise _hip.KfacHipError('%s %d: %d vs %d elements' % (what, i, x.numel(), y.numel()))
+
+
+def axpby_batched(xs, ys, a, b):
+    """ys[i] = a*xs[i] + b*ys[i] in place."""
+    lib = _hip.load()
+    if len(xs) == 0:
+        return
+    _check_same_numel(xs, ys, 'axpby')
+    dev, numel, ws, ws_bytes = _vec_args(lib, xs)
+    st = lib.kfac_axpby_batched(len(xs), numel, _hip.ptr_array(xs, 'x'), _hip.ptr_array(ys, 'y'),
+                                float(a), float(b), _ws_ptr(ws), ws_bytes, _hip.stream_ptr(dev))
+    _hip.check(st, 'kfac_axpby_batched')
+
+
+def diag_inverse_batched(emas, invs, dampings, use_sqrt):
+    lib = _hip.load()
+    if len(emas) == 0:
+        return
+    _check_same_numel(emas, invs, 'diag inverse')
+    dev, numel, ws, ws_bytes = _vec_args(lib, emas)
+    st = lib.kfac_diag_inverse_batched(len(emas), numel, _hip.ptr_array(emas, 'ema'),
+                                       _hip.ptr_array(invs, 'inv'), _hip.f32_array(dampings),
+                                       int(bool(use_sqrt)), _ws_ptr(ws), ws_bytes,
+                                       _hip.stream_ptr(dev))
+    _hip.check(st, 'kfac_diag_inverse_batched')
+
+
+def diag_precondition_batched(invs, grads):
+    lib = _hip.load()
+    if len(invs) == 0:
+        return
+    _check_same_numel(invs, grads, 'diag precondition')
+    dev, numel, ws, ws_bytes = _vec_args(lib, invs)
+    st = lib.kfac_diag_precondition_batched(len(invs), numel, _hip.ptr_array(invs, 'inv'),
+                                            _hip.ptr_array(grads, 'grad'), _ws_ptr(ws), ws_bytes,
+                                            _hip.stream_ptr(dev))
+    _hip.check(st, 'kfac_diag_precondition_batched')
+
+
+def sgd_update_batched(params, grads, bufs, lrs, momenta, weight_decays):
+    """g += wd*p; buf = m*buf + g, g = buf (if m); p -= lr*g  for every tensor."""
+    lib = _hip.load()
+    if len(params) == 0:
+        return
+    _check_same_numel(params, grads, 'update')
+    for i, (p, buf, m) in enumerate(zip(params, bufs, momenta)):
+        if m != 0 and (buf is None or buf.numel() != p.numel()):
+            raise _hip.KfacHipError('update %d: momentum buffer missing or of wrong size' % i)
+    dev, numel, ws, ws_bytes = _vec_args(lib, params)
+    st = lib.kfac_sgd_update_batched(
+        len(params), numel, _hip.ptr_array(params, 'param'), _hip.ptr_array(grads, 'grad'),
+        _hip.ptr_array(bufs, 'momentum buffer', True), _hip.f32_array(lrs),
+        _hip.f32_array(momenta), _hip.f32_array(weight_decays), _ws_ptr(ws), ws_bytes,
+        _hip.stream_ptr(dev))
+    _hip.check(st, 'kfac_sgd_update_batched')
+
+
+def rowsq_sum(x, channels, scale=None, shift=None):
+    """[n, c] tensor of sum over the trailing dims of ((x - shift[c]) / scale[c])^2."""
+    lib = _hip.load()
+    x = x.contiguous()
+    n = x.shape[0]
+    if x.shape[1] != channels:
+        raise _hip.KfacHipError('expected %d channels, got %s' % (channels, tuple(x.shape)))
+    length = x.numel() // (n * channels)
+    out = torch.empty((n, channels), dtype=torch.float32, device=x.device)
+    st = lib.kfac_rowsq_sum(_hip.dev_ptr(x, 'input'), n * channels, channels, length,
+                            None if scale is None else _hip.dev_ptr(scale, 'scale'),
+                            None if shift is None else _hip.dev_ptr(shift, 'shift'),
+                            out.data_ptr(), _hip.stream_ptr(x.device))
+    _hip.check(st, 'kfac_rowsq_sum')
+    return out
+
+
+def bn_diag_combine(sx, sg, alpha, bias):
+    lib = _hip.load()
+    n, c = sx.shape
+    if tuple(sg.shape) != (n, c):
+        raise _hip.KfacHipError('bn_diag_combine: %s vs %s' % (tuple(sx.shape), tuple(sg.shape)))
+    w = torch.empty(c, dtype=torch.float32, device=sx.device)
+    b = torch.empty(c, dtype=torch.float32, device=sx.device) if bias else None
+    st = lib.kfac_bn_diag_combine(_hip.dev_ptr(sx, 'sx'), _hip.dev_ptr(sg, 'sg'), n, c,
+                                  float(alpha), w.data_ptr(), None if b is None else b.data_ptr(),
+                                  _hip.stream_ptr(sx.device))
+    _hip.check(st, 'kfac_bn_diag_combine')
+    return w, b
