@@ -227,67 +227,89 @@ def sample(mean_w, mean_b, U_G, U_A, noise, std_scale, dtype=torch.float32):
 # straight-line optimizer steps (host sequencing)
 # --------------------------------------------------------------------------
 
-class KronLayerState(object):
-    """EMA/inverse state of one Kron layer as Curvature keeps it
-    (curvature.py:37-48)."""
+class LayerState(object):
+    """EMA / inverse / momentum state of one layer as Curvature and the
+    optimizer keep it (curvature.py:37-48, secondorder.py:138-142)."""
 
-    def __init__(self):
+    def __init__(self, kind, bias):
+        self.kind = kind          # 'kron' or 'diag'
+        self.bias = bias
         self.ema = None
         self.inv = None
         self.std = None
+        self.l2_reg = 0.
         self.l2_reg_ema = 0.
-        self.momentum = None
+        self.momentum = None      # one buffer per parameter
 
 
-def kron_curvature_step(state, A, G, damping, ema_decay, l2_reg=0., dtype=torch.float32,
-                        update_std=False):
-    """Curvature.step for a Kron layer: EMA, then pi-damped inverses with
-    damping + l2_reg_ema, then optionally std (curvature.py:166-191,302-321)."""
+def curvature_step(state, data, damping, ema_decay, dtype=torch.float32, update_std=False):
+    """Curvature.step: EMA of the data and of l2_reg, then the inverse with
+    damping + l2_reg_ema -- pi-split for a Kron layer, element-wise for a
+    diagonal one -- then optionally std (curvature.py:166-191,226-232,302-321)."""
     first = state.ema is None
-    state.ema = ema_update([A.to(dtype), G.to(dtype)], state.ema, ema_decay)
-    state.l2_reg_ema = l2_reg_ema_update(l2_reg, state.l2_reg_ema, ema_decay, first)
-    state.inv = list(pi_damped_inverse(state.ema[0], state.ema[1],
-                                       damping + state.l2_reg_ema, dtype))
-    if update_std:
-        state.std = [cholesky_upper(X, dtype) for X in state.inv]
+    state.ema = ema_update([d.to(dtype) for d in data], state.ema, ema_decay)
+    state.l2_reg_ema = l2_reg_ema_update(state.l2_reg, state.l2_reg_ema, ema_decay, first)
+    damp = damping + state.l2_reg_ema
+    if state.kind == 'kron':
+        state.inv = list(pi_damped_inverse(state.ema[0], state.ema[1], damp, dtype))
+        if update_std:
+            state.std = [cholesky_upper(X, dtype) for X in state.inv]
+    else:
+        state.inv = [diag_inverse(e, damp) for e in state.ema]
+        if update_std:
+            state.std = [i.sqrt() for i in state.inv]
     return state
 
 
+def layer_step(state, params, grads, data, *, lr, damping, ema_decay, l2_reg=0., momentum=0.,
+               momentum_type='preconditioned', weight_decay=0., dtype=torch.float32,
+               update_std=False):
+    """The per-group body of SecondOrderOptimizer.step (secondorder.py:195-209):
+       raw:   g += l2_reg*p (and curv.l2_reg = l2_reg), momentum if type 'raw'
+       curv.step(); curv.precondition_grad()
+       preconditioned: g += weight_decay*p, momentum if type 'preconditioned'
+       p -= lr*g
+    params/grads: [w, b] or [w]; returns (new params, final grads)."""
+    params = [p.to(dtype) for p in params]
+    grads = [g.to(dtype) for g in grads]
+    if state.momentum is None:
+        state.momentum = [torch.zeros_like(p) for p in params]
+
+    def apply_momentum(gs):
+        if momentum == 0:
+            return gs
+        state.momentum = [b * momentum + g for b, g in zip(state.momentum, gs)]
+        return [b.clone() for b in state.momentum]
+
+    if l2_reg != 0:
+        grads = [g + l2_reg * p for g, p in zip(grads, params)]
+        state.l2_reg = l2_reg
+    if momentum_type == 'raw':
+        grads = apply_momentum(grads)
+    curvature_step(state, data, damping, ema_decay, dtype, update_std)
+    if state.kind == 'kron':
+        gw, gb = precondition(state.inv[1], state.inv[0], grads[0],
+                              grads[1] if state.bias else None, dtype)
+        grads = [gw, gb] if state.bias else [gw]
+    else:
+        grads = [i * g for i, g in zip(state.inv, grads)]
+    if weight_decay != 0:
+        grads = [g + weight_decay * p for g, p in zip(grads, params)]
+    if momentum_type == 'preconditioned':
+        grads = apply_momentum(grads)
+    params = [p - lr * g for p, g in zip(params, grads)]
+    return params, grads
+
+
 def sgd_tail(p, grad, buf, lr, momentum=0., weight_decay=0.):
-    """Preconditioned-gradient tail of SecondOrderOptimizer.step with
-    momentum_type='preconditioned': g += wd*p; buf = m*buf + g; g = buf;
-    p -= lr*g  (torchsso/optim/secondorder.py:248-261,225-231)."""
+    """Preconditioned-gradient tail for one tensor: g += wd*p; buf = m*buf + g;
+    g = buf; p -= lr*g  (secondorder.py:248-261,225-231)."""
     if weight_decay != 0:
         grad = grad + weight_decay * p
     if momentum != 0:
         buf = buf * momentum + grad
         grad = buf.clone()
     return p - lr * grad, grad, buf
-
-
-def kfac_layer_step(state, params, grads, A, G, *, lr, damping, ema_decay, l2_reg=0.,
-                    momentum=0., weight_decay=0., dtype=torch.float32, update_std=False):
-    """One pass of the per-group body of SecondOrderOptimizer.step for a Kron
-    layer (secondorder.py:195-209): raw l2, curvature step, precondition,
-    weight decay / momentum on the preconditioned gradient, update."""
-    w, b = params
-    gw, gb = grads
-    w = w.to(dtype)
-    gw = gw.to(dtype)
-    if b is not None:
-        b, gb = b.to(dtype), gb.to(dtype)
-    if l2_reg != 0:
-        gw = gw + l2_reg * w
-        if b is not None:
-            gb = gb + l2_reg * b
-    kron_curvature_step(state, A, G, damping, ema_decay, l2_reg, dtype, update_std)
-    pw, pb = precondition(state.inv[1], state.inv[0], gw, gb, dtype)
-    if state.momentum is None:
-        state.momentum = [torch.zeros_like(w), None if b is None else torch.zeros_like(b)]
-    w, pw, state.momentum[0] = sgd_tail(w, pw, state.momentum[0], lr, momentum, weight_decay)
-    if b is not None:
-        b, pb, state.momentum[1] = sgd_tail(b, pb, state.momentum[1], lr, momentum, weight_decay)
-    return (w, b), (pw, pb)
 
 
 # --------------------------------------------------------------------------

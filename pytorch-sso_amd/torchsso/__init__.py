@@ -1,1 +1,18 @@
+"""torchsso: K-FAC curvature engine for AMD Instinct MI355X (gfx950).
+
+The Python surface is the one of cybertronai/pytorch-sso for the K-FAC path
+(SecondOrderOptimizer / VIOptimizer, the Kron*/Diag* curvature classes looked
+up by name on this namespace, torchsso.utils.inv / cholesky); the arithmetic
+runs in hand-written HIP kernels behind the C ABI of libkfac_hip.so.
+"""
 from torchsso import _hip, _ops  # NOQA
+from torchsso import utils  # NOQA
+
+from torchsso.curv.curvature import Curvature, DiagCurvature, KronCurvature  # NOQA
+from torchsso.curv.cov.linear import CovLinear, KronCovLinear  # NOQA
+from torchsso.curv.cov.conv import CovConv2d, KronCovConv2d  # NOQA
+from torchsso.curv.cov.batchnorm import CovBatchNorm1d, DiagCovBatchNorm1d, CovBatchNorm2d, DiagCovBatchNorm2d  # NOQA
+
+from torchsso import optim  # NOQA
+
+__version__ = '0.1.0'

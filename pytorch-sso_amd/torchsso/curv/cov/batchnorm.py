@@ -1,0 +1,54 @@
+"""Diagonal curvature of BatchNorm layers.
+
+Mirrors torchsso/curv/cov/batchnorm.py:10-49 of the reference:
+    w_curv[c] = mean_n[(sum_hw x_hat^2)(sum_hw g^2)],  b_curv[c] = mean_n[sum_hw g^2]
+followed by the n^2 rescale (curvature.py:154-158), where
+x_hat = (out - bias) / weight is the normalised input (curvature.py:123-134).
+sum_hw x_hat^2 is reduced straight from the layer output in the forward hook
+(before an in-place activation can touch it) and x_hat itself is never stored.
+"""
+import torch.nn as nn
+
+from torchsso import _ops
+from torchsso.curv.curvature import Curvature, DiagCurvature
+
+
+class CovBatchNorm1d(Curvature):
+
+    def update_in_backward(self, grad_output_data):
+        pass
+
+
+class CovBatchNorm2d(Curvature):
+
+    def update_in_backward(self, grad_output):
+        pass
+
+
+class _DiagCovBatchNorm(DiagCurvature):
+
+    def forward_postprocess(self, module, input, output):
+        assert self._module == module
+        bn = module
+        if not isinstance(bn, (nn.BatchNorm1d, nn.BatchNorm2d, nn.BatchNorm3d)):
+            raise TypeError('expected a BatchNorm module, got %s' % type(bn).__name__)
+        out = output.detach()
+        # [n, c] sums over the spatial positions of ((out - bias) / weight)^2
+        self._sx = _ops.rowsq_sum(out, bn.num_features, bn.weight.detach(), bn.bias.detach())
+        setattr(module, 'data_output', output)
+        if output.requires_grad:
+            output.register_hook(self._on_grad_output)
+
+    def update_in_backward(self, grad_output):
+        n = grad_output.shape[0]
+        sg = _ops.rowsq_sum(grad_output, self._module.num_features)
+        w, b = _ops.bn_diag_combine(self._sx, sg, float(n), self.bias)   # n^2 / n
+        self._data = [w] if b is None else [w, b]
+
+
+class DiagCovBatchNorm1d(_DiagCovBatchNorm):
+    pass
+
+
+class DiagCovBatchNorm2d(_DiagCovBatchNorm):
+    pass

@@ -1,0 +1,40 @@
+"""Curvature of nn.Linear from the covariance of per-sample gradients.
+
+KronCovLinear mirrors torchsso/curv/cov/linear.py:48-114 of the reference; the
+factors come from the HIP factor kernel, with the bias column (LAST) synthesised
+in the kernel and the 1/n and n^2 scalings folded into its scale factor.
+"""
+from torchsso import _ops
+from torchsso.curv.curvature import Curvature, KronCurvature
+
+
+class CovLinear(Curvature):
+    """Full (dense) covariance of a Linear layer: named by the reference
+    (cov/linear.py:5-25) but not part of the K-FAC path; not implemented here."""
+
+    def update_in_backward(self, grad_output):
+        raise NotImplementedError('CovLinear (dense curvature) is outside the K-FAC path')
+
+    def precondition_grad(self, params):
+        pass
+
+
+class KronCovLinear(KronCurvature):
+
+    def update_in_forward(self, input_data):
+        # A = [a,1]^T [a,1] / n                       (reference: linear.py:50-59)
+        a = input_data.reshape(-1, input_data.shape[-1]) if input_data.dim() != 2 else input_data
+        n = input_data.shape[0]
+        self._A = _ops.factor_linear(a, self.bias, 1.0 / n)
+
+    def update_in_backward(self, grad_output):
+        # G = g^T g / n, then * n^2                   (reference: linear.py:61-67,
+        #                                              curvature.py:154-155,299-300)
+        g = grad_output.reshape(-1, grad_output.shape[-1]) if grad_output.dim() != 2 else grad_output
+        n = grad_output.shape[0]
+        self._G = _ops.factor_linear(g, False, float(n))
+
+    def _get_shape(self):
+        f_out, f_in = self._module.weight.shape
+        d_a = f_in + 1 if self.bias else f_in
+        return (d_a, d_a), (f_out, f_out)

@@ -1,0 +1,430 @@
+"""Per-layer curvature state: data -> ema -> inv (-> std).
+
+Host-side mirror of torchsso/curv/curvature.py of the reference (class names,
+constructor arguments, attributes and error behaviour are the same); all
+arithmetic runs in the HIP engine through torchsso._ops.  Differences in
+mechanics, none in results:
+
+* the per-layer methods (`step`, `update_ema`, `update_inv`, `update_std`,
+  `precondition_grad`, `sample_params`) are thin wrappers over list-based
+  functions at the bottom of this file (`step_all`, `precondition_all`,
+  `sample_all`), which the optimizers call once for all layers so that every
+  engine routine is launched once per step, not once per layer;
+* `ema` is updated in place and `inv` / `std` buffers are reused from step to
+  step (the reference allocates new tensors each time);
+* the output gradient is taken with a tensor hook on the module output instead
+  of the deprecated module backward hook (same tensor, and it also works with
+  an in-place activation after the module).
+"""
+import math
+
+import torch
+import torch.nn as nn
+
+from torchsso import _ops
+
+PI_TYPE_TRACENORM = 'tracenorm'
+
+
+class Curvature(object):
+    """Base class (reference: curvature.py:10-212)."""
+
+    def __init__(self, module: nn.Module, ema_decay=1., damping=1e-7,
+                 use_max_ema=False, use_sqrt_ema=False,
+                 pi_type=PI_TYPE_TRACENORM):
+
+        if ema_decay < 0 or 1 < ema_decay:
+            raise ValueError("Invalid ema_decay: {}".format(ema_decay))
+        if damping < 0:
+            raise ValueError("Invalid damping: {}".format(damping))
+        if pi_type not in [PI_TYPE_TRACENORM]:
+            raise ValueError("Invalid pi_type: {}".format(pi_type))
+
+        self._module = module
+        self.ema_decay = ema_decay
+        self._damping = damping
+        self._l2_reg = 0
+        self._l2_reg_ema = 0
+
+        self._data = None
+        self._acc_data = None
+        self.ema = None
+        self.ema_max = None
+        self.inv = None
+        self.std = None
+        self.info = None   # device int32 status of the last inversion (0 = ok)
+
+        self.use_sqrt_ema = use_sqrt_ema
+        self.use_max_ema = use_max_ema
+
+        self.pi_type = pi_type
+
+        module.register_forward_hook(self.forward_postprocess)
+
+    # ---- attributes the optimizers and users read -------------------------
+
+    @property
+    def data(self):
+        return self._data
+
+    @data.setter
+    def data(self, value):
+        self._data = value
+
+    @property
+    def shape(self):
+        if self._data is None:
+            return self._get_shape()
+        return tuple([d.shape for d in self._data])
+
+    @property
+    def device(self):
+        return next(self._module.parameters()).device
+
+    def _get_shape(self):
+        size = sum(p.numel() for p in self._module.parameters())
+        return tuple((size, size))
+
+    def element_wise_init(self, value):
+        self._data = [torch.diag(torch.full((s[0],), float(value), device=self.device))
+                      for s in self.shape]
+
+    @property
+    def module(self):
+        return self._module
+
+    @property
+    def bias(self):
+        return getattr(self._module, 'bias', None) is not None
+
+    @property
+    def damping(self):
+        return self._damping + self._l2_reg_ema
+
+    @property
+    def l2_reg(self):
+        return self._l2_reg
+
+    @l2_reg.setter
+    def l2_reg(self, value):
+        self._l2_reg = value
+
+    @property
+    def l2_reg_ema(self):
+        return self._l2_reg_ema
+
+    # ---- hooks ---------------------------------------------------------------
+
+    def forward_postprocess(self, module, input, output):
+        """Forward hook (reference: curvature.py:118-139)."""
+        assert self._module == module
+        data_input = input[0].detach()
+        setattr(module, 'data_input', data_input)
+        setattr(module, 'data_output', output)
+        self.update_in_forward(data_input)
+        if isinstance(output, torch.Tensor) and output.requires_grad:
+            output.register_hook(self._on_grad_output)
+
+    def _on_grad_output(self, grad_output):
+        self.backward_postprocess(self._module, None, (grad_output,))
+
+    def backward_postprocess(self, module, grad_input, grad_output):
+        """Reference: curvature.py:141-155."""
+        assert self._module == module
+        grad_output = grad_output[0].detach()
+        setattr(module, 'grad_output', grad_output)
+        self.update_in_backward(grad_output)
+
+    def adjust_data_scale(self, scale):
+        """Multiply the current data by `scale` (reference: curvature.py:157-158).
+        The hooks do not call it: the batch-size^2 rescale of curvature.py:154-155
+        is folded into the scale factor of the factor kernels."""
+        self._data = [d.mul_(scale) for d in self._data]
+
+    def update_in_forward(self, data_input):
+        pass
+
+    def update_in_backward(self, grad_output):
+        raise NotImplementedError
+
+    # ---- per-layer step (wrappers over the list-based engine calls) --------
+
+    def step(self, update_std=False, update_inv=True):
+        step_all([self], update_std=update_std, update_inv=update_inv)
+
+    def update_ema(self):
+        update_ema_all([self])
+
+    def update_inv(self):
+        update_inv_all([self])
+
+    def update_std(self):
+        update_std_all([self])
+
+    def precondition_grad(self, params):
+        precondition_all([(self, params)])
+
+    def sample_params(self, params, mean, std_scale):
+        sample_all([(self, params, mean, std_scale)])
+
+    def std_norm(self):
+        raise NotImplementedError
+
+    # ---- what the list-based functions need from a subclass ---------------
+
+    kind = 'full'   # 'kron' | 'diag' | 'full'
+
+    def _inv_one(self, X):
+        """Curvature._inv of the reference (curvature.py:197-200)."""
+        outs, self.info = _ops.damped_inverse_batched([X], [self.damping])
+        return outs[0]
+
+
+class DiagCurvature(Curvature):
+    """Element-wise curvature (reference: curvature.py:215-252)."""
+
+    kind = 'diag'
+
+    def _get_shape(self):
+        return tuple(p.shape for p in self.module.parameters())
+
+    def element_wise_init(self, value):
+        self._data = [torch.full(tuple(s), float(value), device=self.device) for s in self.shape]
+
+    def std_norm(self):
+        if self.std is None:
+            return 0
+        return sum(std.norm().item() for std in self.std)
+
+
+class KronCurvature(Curvature):
+    """Kronecker-factored curvature A (x) G (reference: curvature.py:255-331)."""
+
+    kind = 'kron'
+
+    def __init__(self, *args, **kwargs):
+        super(KronCurvature, self).__init__(*args, **kwargs)
+        self._A = None
+        self._G = None
+
+    @property
+    def data(self):
+        return [self._A, self._G]
+
+    @data.setter
+    def data(self, value):
+        self._A, self._G = value
+
+    @property
+    def shape(self):
+        if self._A is None or self._G is None:
+            return self._get_shape()
+        return self._A.shape, self._G.shape
+
+    def _get_shape(self):
+        raise NotImplementedError
+
+    def element_wise_init(self, value):
+        # sqrt(value) on each factor so that A (x) G has `value` on its diagonal
+        super(KronCurvature, self).element_wise_init(math.sqrt(value))
+        self._A, self._G = self._data
+
+    @property
+    def A(self):
+        return self._A
+
+    @property
+    def G(self):
+        return self._G
+
+    def adjust_data_scale(self, scale):
+        self._G.mul_(scale)
+
+    def std_norm(self):
+        if self.std is None:
+            return 0
+        A_ic, G_ic = self.std
+        return A_ic.norm().item() * G_ic.norm().item()
+
+    # the 2-D [dG, dA(-1)] view of the weight-shaped tensor of this layer
+    def _weight2d(self, w):
+        return w.reshape(w.shape[0], -1)
+
+
+def add_value_to_diagonal(X, value):
+    """X + value*I as a new tensor (reference: curvature.py:334-340, which builds
+    a Python list of n index pairs; here one strided in-place add on a copy)."""
+    out = X.clone()
+    out.diagonal().add_(value)
+    return out
+
+
+# ---------------------------------------------------------------------------
+# list-based engine calls
+# ---------------------------------------------------------------------------
+
+def update_ema_all(curvs):
+    """Curvature.update_ema for every curvature in the list
+    (reference: curvature.py:174-191).  ema_decay weighs the NEW data."""
+    by_beta = {}
+    for c in curvs:
+        data = c.data
+        beta = c.ema_decay
+        if c.ema is None or beta == 1:
+            if c.ema is None:
+                c.ema = [d.clone() for d in data]
+            else:
+                for e, d in zip(c.ema, data):
+                    e.copy_(d)
+            if c.use_max_ema and c.ema_max is None:
+                c.ema_max = [e.clone() for e in c.ema]
+            c._l2_reg_ema = c._l2_reg
+        else:
+            xs, ys = by_beta.setdefault(beta, ([], []))
+            xs.extend(d.contiguous() for d in data)
+            ys.extend(c.ema)
+            c._l2_reg_ema = c._l2_reg * beta + c._l2_reg_ema * (1 - beta)
+    for beta, (xs, ys) in by_beta.items():
+        _ops.axpby_batched(xs, ys, beta, 1 - beta)
+    for c in curvs:
+        if c.use_max_ema:
+            for e, e_max in zip(c.ema, c.ema_max):
+                torch.max(e, e_max, out=e_max)
+
+
+def update_inv_all(curvs):
+    """update_inv for every curvature: one batched pi-damped inversion for all
+    Kronecker layers (reference: curvature.py:302-312), one element-wise launch
+    for all diagonal layers (curvature.py:193-195,226-232)."""
+    kron = [c for c in curvs if c.kind == 'kron']
+    diag = [c for c in curvs if c.kind == 'diag']
+    full = [c for c in curvs if c.kind == 'full']
+    if kron:
+        for c in kron:
+            if c.inv is None or c.inv[0].shape != c.ema[0].shape or c.inv[1].shape != c.ema[1].shape:
+                c.inv = [torch.empty_like(c.ema[0]), torch.empty_like(c.ema[1])]
+        _, _, info = _ops.pi_damped_inverse_batched(
+            [c.ema[0] for c in kron], [c.ema[1] for c in kron], [c.damping for c in kron],
+            [c.inv[0] for c in kron], [c.inv[1] for c in kron])
+        for i, c in enumerate(kron):
+            c.info = info[2 * i:2 * i + 2]
+    if diag:
+        by_sqrt = {False: ([], [], []), True: ([], [], [])}
+        for c in diag:
+            ema = c.ema if not c.use_max_ema else c.ema_max
+            if c.inv is None or any(i.shape != e.shape for i, e in zip(c.inv, ema)):
+                c.inv = [torch.empty_like(e) for e in ema]
+            emas, invs, damps = by_sqrt[bool(c.use_sqrt_ema)]
+            emas.extend(ema)
+            invs.extend(c.inv)
+            damps.extend([c.damping] * len(ema))
+        for use_sqrt, (emas, invs, damps) in by_sqrt.items():
+            _ops.diag_inverse_batched(emas, invs, damps, use_sqrt)
+    for c in full:
+        ema = c.ema if not c.use_max_ema else c.ema_max
+        c.inv = [c._inv_one(e) for e in ema]
+
+
+def update_std_all(curvs):
+    """update_std: upper Cholesky factors of the inverses for Kronecker layers
+    (reference: curvature.py:317-321), sqrt of the inverse for diagonal ones
+    (curvature.py:240-241)."""
+    kron = [c for c in curvs if c.kind == 'kron']
+    mats, outs = [], []
+    for c in kron:
+        if c.std is None or any(s.shape != i.shape for s, i in zip(c.std, c.inv)):
+            c.std = [torch.empty_like(i) for i in c.inv]
+        mats.extend(c.inv)
+        outs.extend(c.std)
+    if mats:
+        _ops.cholesky_upper_batched(mats, outs)
+    for c in curvs:
+        if c.kind == 'diag':
+            c.std = [i.sqrt() for i in c.inv]
+        elif c.kind == 'full':
+            raise NotImplementedError
+
+
+def step_all(curvs, update_std=False, update_inv=True):
+    """Curvature.step for a list (reference: curvature.py:166-172).
+    `update_std` may be a bool or a list of bools, one per curvature."""
+    update_ema_all(curvs)
+    if update_inv:
+        update_inv_all(curvs)
+    if isinstance(update_std, (list, tuple)):
+        sel = [c for c, u in zip(curvs, update_std) if u]
+    else:
+        sel = list(curvs) if update_std else []
+    if sel:
+        update_std_all(sel)
+
+
+def precondition_all(pairs):
+    """precondition_grad for a list of (curvature, params): grads are replaced
+    in place by G^-1 [dW|db] A^-1 (reference: cov/linear.py:69-84,
+    cov/conv.py:76-92) or inv * grad (curvature.py:234-238)."""
+    Gi, Ai, gw, gb = [], [], [], []
+    dinv, dgrad = [], []
+    for c, params in pairs:
+        if c.kind == 'kron':
+            A_inv, G_inv = c.inv
+            w = params[0]
+            if not w.grad.is_contiguous():
+                w.grad = w.grad.contiguous()
+            Gi.append(G_inv)
+            Ai.append(A_inv)
+            gw.append(w.grad)
+            if c.bias:
+                b = params[1]
+                if not b.grad.is_contiguous():
+                    b.grad = b.grad.contiguous()
+                gb.append(b.grad)
+            else:
+                gb.append(None)
+        elif c.kind == 'diag':
+            for p, inv in zip(params, c.inv):
+                if not p.grad.is_contiguous():
+                    p.grad = p.grad.contiguous()
+                dinv.append(inv)
+                dgrad.append(p.grad)
+        # 'full' curvatures do not precondition (reference: cov/linear.py:24-25)
+    if Gi:
+        _ops.precondition_batched(Gi, Ai, gw, gb)
+    if dinv:
+        _ops.diag_precondition_batched(dinv, dgrad)
+
+
+def sample_all(items):
+    """sample_params for a list of (curvature, params, mean, std_scale).
+
+    The standard-normal noise is drawn with torch.randn_like in list order, one
+    [dG, dA] matrix per Kronecker layer and one tensor per parameter of a
+    diagonal layer, which is the order and shape in which the reference consumes
+    the generator (cov/linear.py:92-93, cov/conv.py:100-101,
+    curvature.py:243-246); the products run batched afterwards."""
+    by_scale = {}
+    for c, params, mean, std_scale in items:
+        if c.kind == 'kron':
+            A_ic, G_ic = c.std
+            dG, dA = G_ic.shape[0], A_ic.shape[0]
+            noise = torch.randn((dG, dA), dtype=mean[0].dtype, device=mean[0].device)
+            lst = by_scale.setdefault(float(std_scale), [])
+            w = params[0].data
+            if not w.is_contiguous():
+                params[0].data = w = w.contiguous()
+            pb = None
+            mb = None
+            if c.bias:
+                pb = params[1].data
+                mb = mean[1].contiguous()
+            lst.append((G_ic, A_ic, noise, mean[0].contiguous(), mb, w, pb))
+        elif c.kind == 'diag':
+            for p, m, std in zip(params, mean, c.std):
+                noise = torch.randn_like(m)
+                p.data.copy_(torch.addcmul(m, noise, std, value=std_scale))
+        else:
+            raise NotImplementedError
+    for std_scale, lst in by_scale.items():
+        _ops.sample_batched([x[0] for x in lst], [x[1] for x in lst], [x[2] for x in lst],
+                            [x[3] for x in lst], [x[4] for x in lst], [x[5] for x in lst],
+                            [x[6] for x in lst], std_scale)

@@ -1,0 +1,2 @@
+from torchsso.optim.secondorder import SecondOrderOptimizer  # NOQA
+from torchsso.optim.vi import VIOptimizer  # NOQA

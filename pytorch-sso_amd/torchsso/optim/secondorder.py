@@ -1,0 +1,332 @@
+"""SecondOrderOptimizer: K-FAC style preconditioned SGD driven by per-layer
+curvature objects.
+
+Same constructor, param_group layout, `step(closure)` contract and update rule
+as torchsso/optim/secondorder.py:15-330 of the reference.  The per-layer loop
+of the reference (secondorder.py:195-209) is regrouped by phase -- layers are
+independent, so the results are the same -- and every phase is one batched call
+into the HIP engine:
+
+    raw phase            grad += l2_reg * p                    (axpby kernel)
+    curvature phase      EMA, pi-damped inverses of all layers (batched Cholesky)
+    precondition phase   G^-1 [dW|db] A^-1 for all layers      (two MFMA launches)
+    update phase         weight decay, momentum, p -= lr * g   (one fused kernel)
+
+Options that need norms or extra buffers (raw-gradient momentum, gradient EMA,
+bias correction, LARS, weight normalisation) run as in-place torch tensor ops
+on the device, in the reference's order.
+"""
+import math
+
+import numpy as np
+import torch
+import torch.nn as nn
+from torch.optim import Optimizer
+
+import torchsso
+from torchsso import _ops
+from torchsso.curv import curvature as _curv
+from torchsso.utils import TensorAccumulator
+
+
+class SecondOrderOptimizer(Optimizer):
+    r"""Optimizer that preconditions each layer's gradient with the inverse of
+    that layer's curvature.
+
+    Args (as the reference, secondorder.py:23-49):
+        model (torch.nn.Module): model with parameters to be trained
+        curv_type (str): 'Cov' (this package builds the 'Cov' curvatures)
+        curv_shapes (dict): curvature shape per module class name, e.g.
+            {"Conv2d": "Kron", "Linear": "Kron", "BatchNorm2d": "Diag"}
+        curv_kwargs (dict): keyword arguments of torchsso.Curvature.__init__
+        lr, momentum, momentum_type ('raw' | 'preconditioned'),
+        grad_ema_decay, grad_ema_type, l2_reg, weight_decay,
+        normalizing_weights, weight_scale, acc_steps, non_reg_for_bn,
+        bias_correction, lars, lars_type, update_inv, precondition_grad
+    """
+
+    def __init__(self, model: nn.Module, curv_type: str, curv_shapes: dict, curv_kwargs: dict,
+                 lr=0.01, momentum=0., momentum_type='preconditioned',
+                 grad_ema_decay=1., grad_ema_type='raw', l2_reg=0., weight_decay=0.,
+                 normalizing_weights=False, weight_scale=None,
+                 acc_steps=1, non_reg_for_bn=False, bias_correction=False,
+                 lars=False, lars_type='preconditioned', update_inv=True, precondition_grad=True):
+
+        if lr < 0:
+            raise ValueError("Invalid learning rate: {}".format(lr))
+        if momentum < 0:
+            raise ValueError("Invalid momentum: {}".format(momentum))
+        if momentum > 0 and momentum_type not in ['raw', 'preconditioned']:
+            raise ValueError("Invalid momentum type: {}".format(momentum_type))
+        if grad_ema_decay < 0 or 1 < grad_ema_decay:
+            raise ValueError("Invalid grad_ema value: {}".format(grad_ema_decay))
+        if grad_ema_decay > 0 and grad_ema_type not in ['raw', 'preconditioned']:
+            raise ValueError("Invalid grad_ema type: {}".format(grad_ema_type))
+        if l2_reg < 0:
+            raise ValueError("Invalid l2_reg value: {}".format(l2_reg))
+        if weight_decay < 0:
+            raise ValueError("Invalid weight_decay value: {}".format(weight_decay))
+        if acc_steps < 1:
+            raise ValueError("Invalid acc_steps: {}".format(acc_steps))
+        if lars and lars_type not in ['raw', 'preconditioned']:
+            raise ValueError("Invalid LARS type: {}".format(lars_type))
+        if normalizing_weights and weight_scale is not None and weight_scale <= 0:
+            raise ValueError("Invalid weight scale for LARS: {}".format(weight_scale))
+
+        self.model = model
+        defaults = {'lr': lr, 'momentum': momentum, 'momentum_type': momentum_type,
+                    'grad_ema_decay': grad_ema_decay, 'grad_ema_type': grad_ema_type,
+                    'l2_reg': l2_reg, 'weight_decay': weight_decay,
+                    'normalizing_weights': normalizing_weights, 'weight_scale': weight_scale,
+                    'acc_steps': acc_steps, 'bias_correction': bias_correction,
+                    'lars': lars, 'lars_type': lars_type}
+        defaults.update(curv_kwargs)
+
+        self.curv_type = curv_type
+        self.curv_shapes = {} if curv_shapes is None else curv_shapes
+        self.update_inv = update_inv
+        self.precondition_grad = precondition_grad
+        self.optim_state = {'step': 0, 'acc_step': 0}
+
+        # one param_group per leaf module that owns parameters
+        groups = []
+        bn_groups = []
+        for module in model.modules():
+            if len(list(module.children())) > 0:
+                continue
+            params = list(module.parameters())
+            if len(params) == 0:
+                continue
+            curv_class = self.get_curv_class(module)
+            curvature = curv_class(module, **curv_kwargs)
+            group = {'params': params, 'curv': curvature,
+                     'acc_curv': TensorAccumulator(), 'acc_grads': TensorAccumulator()}
+            groups.append(group)
+            if non_reg_for_bn and isinstance(module, (nn.BatchNorm1d, nn.BatchNorm2d, nn.BatchNorm3d)):
+                bn_groups.append(group)
+        if len(groups) == 0:
+            raise ValueError("model has no parameters to optimize")
+
+        # torch's base class fills every group with the defaults and sets up
+        # `state`; the reference assigns those fields by hand instead
+        # (secondorder.py:94-106), which current torch no longer tolerates.
+        super(SecondOrderOptimizer, self).__init__(groups, defaults)
+
+        for group in self.param_groups:
+            self.init_buffer(group['params'])
+        for group in bn_groups:
+            group['l2_reg'] = 0
+            group['weight_decay'] = 0
+            group['normalizing_weights'] = False
+
+    def init_buffer(self, params):
+        for p in params:
+            state = self.state[p]
+            state['momentum_buffer'] = torch.zeros_like(p.data)
+            state['grad_ema_buffer'] = torch.zeros_like(p.data)
+
+    @property
+    def local_param_groups(self):
+        return self.param_groups
+
+    def get_curv_class(self, module):
+        """Class looked up by name on the package namespace: shape + type + module
+        class, e.g. 'Kron' + 'Cov' + 'Linear' (reference: secondorder.py:148-156)."""
+        module_name = module.__class__.__name__
+        curv_shape = self.curv_shapes.get(module_name, '')
+        curv_name = curv_shape + self.curv_type + module_name
+        curv_class = getattr(torchsso, curv_name, None)
+
+        assert curv_class is not None, f"Failed to lookup Curvature class {curv_name} for {module}."
+
+        return curv_class
+
+    # ------------------------------------------------------------------ step
+
+    def step(self, closure=None):
+        """One optimization step.  `closure` runs forward and backward and returns
+        the loss or (loss, output); its return value is passed through."""
+        n = self.defaults['acc_steps']
+        loss = None
+
+        if closure is not None:
+            loss = closure()
+
+            if n > 1:
+                for group in self.param_groups:
+                    grads = [p.grad.data for p in group['params']]
+                    group['acc_grads'].update(grads, scale=1 / n)
+                    curv = group['curv']
+                    if curv is not None:
+                        group['acc_curv'].update(curv.data, scale=1 / n)
+
+            self.optim_state['acc_step'] += 1
+            if self.optim_state['acc_step'] < n:
+                return loss
+            self.optim_state['acc_step'] = 0
+
+            if n > 1:
+                self.backward_postprocess()
+            # n == 1: the accumulated values are the gradients and factors
+            # themselves (scale 1), so they are used where they lie
+
+        self.optim_state['step'] += 1
+        self._update_groups(self.local_param_groups, target='params',
+                            update_inv=self.update_inv, update_std=False,
+                            precondition=self.precondition_grad)
+        return loss
+
+    def _update_groups(self, groups, target, update_inv, update_std, precondition):
+        for group in groups:
+            self.update_preprocess(group, target=target, grad_type='raw')
+
+        curvs = [g['curv'] for g in groups if g['curv'] is not None]
+        if curvs:
+            if isinstance(update_std, (list, tuple)):
+                update_std = [u for g, u in zip(groups, update_std) if g['curv'] is not None]
+            _curv.step_all(curvs, update_std=update_std, update_inv=update_inv)
+            if precondition:
+                _curv.precondition_all([(g['curv'], g[target]) for g in groups
+                                        if g['curv'] is not None])
+
+        fused = []
+        for group in groups:
+            if self._can_fuse_update(group):
+                fused.append(group)
+            else:
+                self.update_preprocess(group, target=target, grad_type='preconditioned')
+                self.update(group, target=target)
+        self._fused_update(fused, target)
+        for group in groups:
+            self.update_postprocess(group, target=target)
+
+    def backward_postprocess(self, target='params'):
+        """Accumulated gradients and factors become the current ones
+        (reference: secondorder.py:213-223)."""
+        for group in self.param_groups:
+            acc_grads = group['acc_grads'].get()
+            for p, acc_grad in zip(group[target], acc_grads):
+                p.grad = acc_grad
+            curv = group['curv']
+            if curv is not None:
+                curv.data = group['acc_curv'].get()
+
+    # ------------------------------------------------------------ update tail
+
+    @staticmethod
+    def _can_fuse_update(group):
+        """The fused kernel covers weight decay, momentum on the preconditioned
+        gradient and the parameter update."""
+        # (momentum on the raw gradient was already applied in the raw phase)
+        if group['grad_ema_decay'] != 1 and group['grad_ema_type'] == 'preconditioned':
+            return False
+        if group['bias_correction']:
+            return False
+        if group['lars'] and group['lars_type'] == 'preconditioned':
+            return False
+        return True
+
+    def _fused_update(self, groups, target):
+        ps, gs, bufs, lrs, moms, wds = [], [], [], [], [], []
+        for group in groups:
+            mom = group['momentum'] if group['momentum_type'] == 'preconditioned' else 0.
+            for p in group[target]:
+                grad = p.grad
+                if grad is None:
+                    continue
+                if not grad.is_contiguous():
+                    p.grad = grad = grad.contiguous()
+                ps.append(p.data)
+                gs.append(grad)
+                bufs.append(self.state[p]['momentum_buffer'] if mom != 0 else None)
+                lrs.append(group['lr'])
+                moms.append(mom)
+                wds.append(group['weight_decay'])
+        _ops.sgd_update_batched(ps, gs, bufs, lrs, moms, wds)
+
+    def update(self, group, target='params'):
+        """p -= lr * grad (reference: secondorder.py:225-231)."""
+        ps, gs = [], []
+        for p in group[target]:
+            if p.grad is None:
+                continue
+            ps.append(p.data)
+            gs.append(p.grad)
+        if ps:
+            _ops.axpby_batched(gs, ps, -group['lr'], 1.)
+
+    def update_preprocess(self, group, target='params', grad_type='raw'):
+        """Gradient transformations before ('raw') and after ('preconditioned')
+        preconditioning, in the reference's order (secondorder.py:233-312)."""
+        assert grad_type in ['raw', 'preconditioned'], 'Invalid grad type: {}.'.format(grad_type)
+        params = [p for p in group[target] if p.grad is not None]
+        if not params:
+            return
+        state = self.state
+
+        if grad_type == 'raw' and group['l2_reg'] != 0:
+            for p in params:
+                if p.grad.is_sparse:
+                    raise RuntimeError(
+                        "l2 regularization option is not compatible with sparse gradients")
+            _ops.axpby_batched([p.data for p in params], [p.grad for p in params],
+                               group['l2_reg'], 1.)
+            curv = group['curv']
+            if curv is not None:
+                curv.l2_reg = group['l2_reg']
+
+        if grad_type == 'preconditioned' and group['weight_decay'] != 0:
+            for p in params:
+                if p.grad.is_sparse:
+                    raise RuntimeError(
+                        "weight_decay option is not compatible with sparse gradients")
+            _ops.axpby_batched([p.data for p in params], [p.grad for p in params],
+                               group['weight_decay'], 1.)
+
+        if group['momentum_type'] == grad_type and group['momentum'] != 0:
+            bufs = [state[p]['momentum_buffer'] for p in params]
+            grads = [p.grad for p in params]
+            _ops.axpby_batched(grads, bufs, 1., group['momentum'])      # buf = m*buf + g
+            _ops.axpby_batched(bufs, grads, 1., 0.)                     # g = buf
+
+        if group['grad_ema_type'] == grad_type and group['grad_ema_decay'] != 1:
+            decay = group['grad_ema_decay']
+            bufs = [state[p]['grad_ema_buffer'] for p in params]
+            grads = [p.grad for p in params]
+            _ops.axpby_batched(grads, bufs, decay, 1 - decay)           # buf = (1-d)*buf + d*g
+            _ops.axpby_batched(bufs, grads, 1., 0.)
+
+        if grad_type == 'preconditioned' and group['bias_correction']:
+            curv = group['curv']
+            beta1 = 1 - group['grad_ema_decay']
+            beta2 = 1 - curv.ema_decay
+            bias_correction1 = 1 - beta1 ** self.optim_state['step']
+            bias_correction2 = 1 - beta2 ** self.optim_state['step']
+            if getattr(curv, 'use_sqrt_ema', False):
+                bias_correction2 = math.sqrt(bias_correction2)
+            for p in params:
+                p.grad.mul_(bias_correction2 / bias_correction1)
+
+        if group['lars_type'] == grad_type and group['lars']:
+            thr, eps = 1e-2, 1e-9
+            for p in params:
+                d_norm = p.data.norm()
+                if d_norm > thr:
+                    g_norm = p.grad.norm()
+                    p.grad.mul_(d_norm / (g_norm + eps))
+
+    def update_postprocess(self, group, target='params'):
+        """Optional weight normalisation (reference: secondorder.py:314-330)."""
+        if not group['normalizing_weights']:
+            return
+        curv = group['curv']
+        thr, eps = 1e-2, 1e-9
+        for p, _p in zip(group[target], group['params']):
+            w = getattr(curv.module, 'weight', None)
+            if w is not None and w is _p:
+                d_norm = p.data.norm()
+                if d_norm > thr:
+                    scale = group['weight_scale']
+                    if scale is None:
+                        scale = np.sqrt(2.0 * w.data.shape[0])
+                    p.data.div_(d_norm + eps).mul_(scale)

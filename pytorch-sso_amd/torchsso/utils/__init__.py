@@ -1,0 +1,2 @@
+from torchsso.utils.linalg import inv, cholesky  # NOQA
+from torchsso.utils.accumulator import TensorAccumulator  # NOQA

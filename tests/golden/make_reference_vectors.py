@@ -1,0 +1,140 @@
+"""Writes golden vectors for the host sequencing of the K-FAC step by running the
+reference implementation itself (cybertronai/pytorch-sso mounted read-only at
+/root/reference) on its CPU path.
+
+Run once, in the development container only (the reference does not exist on
+the GPU box):
+
+    python tests/golden/make_reference_vectors.py
+
+What it pins (behaviour that is convention rather than mathematics, so that a
+restatement could silently disagree): the order of operations inside
+SecondOrderOptimizer.step when l2_reg, damping, momentum and weight decay
+interact; what the hooks take as layer input / output gradient on current
+torch; the accumulation scales of VIOptimizer's MC loop.  The numerical kernels
+themselves are pinned by mathematics in tests/test_oracle.py.
+
+The reference imports `chainer` at module level for its multi-GPU communicator
+(torchsso/utils/chainer_communicators/_utility.py:11), which is out of scope and
+not installed; empty placeholder modules are put in sys.modules before the
+import so that the single-process classes load.  No reference file is modified
+or copied; only inputs and outputs (arrays) are saved.
+
+VIOptimizer's posterior sampling cannot be produced this way: the reference's
+`torchsso.utils.cholesky` exists for CuPy only (utils/cholesky_cupy.py:9-14).
+The VI case below therefore uses prior_variance=0 (no sampling, std_scale=0).
+"""
+import os
+import sys
+import types
+import warnings
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+REFERENCE = '/root/reference'
+
+
+def _import_reference():
+    for name in ('chainer', 'chainer.backends', 'chainer.backends.cuda'):
+        sys.modules.setdefault(name, types.ModuleType(name))
+    sys.modules['chainer'].backends = sys.modules['chainer.backends']
+    sys.modules['chainer.backends'].cuda = sys.modules['chainer.backends.cuda']
+    sys.path.insert(0, REFERENCE)
+    import torchsso  # noqa: the reference package
+    assert os.path.realpath(torchsso.__file__).startswith(REFERENCE), torchsso.__file__
+    return torchsso
+
+
+def build_mlp(torch, nn):
+    torch.manual_seed(1)
+    return nn.Sequential(nn.Linear(12, 16), nn.ReLU(), nn.Linear(16, 10), nn.ReLU(),
+                         nn.Linear(10, 5))
+
+
+def build_convnet(torch, nn):
+    torch.manual_seed(1)
+    return nn.Sequential(
+        nn.Conv2d(2, 4, 3, padding=1), nn.BatchNorm2d(4), nn.ReLU(),
+        nn.Conv2d(4, 6, 3, stride=2, bias=False), nn.ReLU(),
+        nn.Flatten(), nn.Linear(6 * 3 * 3, 5))
+
+
+def snapshot(optimizer, out, tag):
+    for gi, group in enumerate(optimizer.param_groups):
+        curv = group['curv']
+        for pi, p in enumerate(group['params']):
+            out['%s.g%d.param%d' % (tag, gi, pi)] = p.detach().numpy().copy()
+            out['%s.g%d.grad%d' % (tag, gi, pi)] = p.grad.detach().numpy().copy()
+        for name in ('ema', 'inv'):
+            val = getattr(curv, name)
+            for k, t in enumerate(val):
+                out['%s.g%d.%s%d' % (tag, gi, name, k)] = t.detach().numpy().copy()
+        out['%s.g%d.damping' % (tag, gi)] = np.float64(curv.damping)
+
+
+def run_case(torchsso, torch, nn, F, name, model, x, y, opt_cls, opt_args, steps):
+    out = {'x': x.numpy().copy(), 'y': y.numpy().copy()}
+    for k, v in model.state_dict().items():
+        out['init.' + k] = v.numpy().copy()
+    optimizer = opt_cls(model, **opt_args)
+
+    def closure():
+        model.zero_grad()
+        output = model(x)
+        loss = F.cross_entropy(output, y)
+        loss.backward()
+        return loss, output
+
+    for s in range(steps):
+        ret = optimizer.step(closure=closure)
+        loss = ret[0]
+        out['step%d.loss' % s] = np.float64(loss.item())
+        snapshot(optimizer, out, 'step%d' % s)
+    path = os.path.join(HERE, name + '.npz')
+    np.savez_compressed(path, **out)
+    print('wrote', path, os.path.getsize(path), 'bytes')
+
+
+def main():
+    warnings.simplefilter('ignore')
+    torchsso = _import_reference()
+    import torch
+    import torch.nn as nn
+    import torch.nn.functional as F
+    torch.set_num_threads(1)
+
+    # 1. MLP, Kron curvature for every Linear, all interacting options on
+    torch.manual_seed(0)
+    x = torch.randn(8, 12)
+    y = torch.randint(0, 5, (8,))
+    run_case(torchsso, torch, nn, F, 'ref_mlp_kfac', build_mlp(torch, nn), x, y,
+             torchsso.optim.SecondOrderOptimizer,
+             dict(curv_type='Cov', curv_shapes={'Linear': 'Kron'},
+                  curv_kwargs={'damping': 1e-3, 'ema_decay': 0.95},
+                  lr=0.05, momentum=0.9, l2_reg=1e-3, weight_decay=1e-3), steps=3)
+
+    # 2. Conv + BatchNorm (diagonal) + strided bias-free conv + Linear
+    torch.manual_seed(0)
+    x = torch.randn(6, 2, 8, 8)
+    y = torch.randint(0, 5, (6,))
+    run_case(torchsso, torch, nn, F, 'ref_convnet_kfac', build_convnet(torch, nn), x, y,
+             torchsso.optim.SecondOrderOptimizer,
+             dict(curv_type='Cov',
+                  curv_shapes={'Linear': 'Kron', 'Conv2d': 'Kron', 'BatchNorm2d': 'Diag'},
+                  curv_kwargs={'damping': 1e-2, 'ema_decay': 0.9},
+                  lr=0.02, momentum=0.5, momentum_type='raw', l2_reg=1e-4), steps=2)
+
+    # 3. VI sequencing without sampling (prior_variance=0 -> l2_reg=0, std_scale=0)
+    torch.manual_seed(0)
+    x = torch.randn(8, 12)
+    y = torch.randint(0, 5, (8,))
+    run_case(torchsso, torch, nn, F, 'ref_mlp_vi_nosample', build_mlp(torch, nn), x, y,
+             torchsso.optim.VIOptimizer,
+             dict(dataset_size=100, curv_type='Cov', curv_shapes={'Linear': 'Kron'},
+                  curv_kwargs={'damping': 1e-3, 'ema_decay': 0.95},
+                  lr=0.05, momentum=0.9, num_mc_samples=3, prior_variance=0), steps=2)
+
+
+if __name__ == '__main__':
+    main()

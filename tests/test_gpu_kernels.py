@@ -1,0 +1,268 @@
+"""Parity of every HIP kernel with the CPU oracle, called through the C ABI
+(torchsso._ops is a ctypes shim over libkfac_hip.so).  Bar: relative Frobenius
+error <= 1e-4 in fp32 against the float64 oracle."""
+import pytest
+import torch
+
+from oracle import kfac_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+D = torch.float64
+
+
+@pytest.fixture(scope='module')
+def ops():
+    from torchsso import _ops
+    return _ops
+
+
+@pytest.fixture(scope='module')
+def dev():
+    return torch.device('cuda:0')
+
+
+def spd(n, L=None, seed=0):
+    g = torch.Generator().manual_seed(seed + n)
+    L = L or max(2 * n, 64)
+    x = torch.randn(L, n, dtype=D, generator=g)
+    return ((x.t() @ x) / L).float()
+
+
+@pytest.mark.parametrize('n,f,bias', [(1, 1, True), (1, 1, False), (8, 5, True), (128, 784, True),
+                                      (128, 1000, False), (37, 129, True), (300, 130, True),
+                                      (5000, 64, False), (20000, 200, True), (256, 2048, True)])
+def test_factor_linear(ops, dev, n, f, bias):
+    torch.manual_seed(n + f)
+    x = torch.randn(n, f)
+    out = ops.factor_linear(x.to(dev), bias, 1.0 / n)
+    assert O.rel_fro(out, O.factor_linear_a(x, bias, D)) < TOL
+    assert torch.equal(out, out.t())
+    # G convention: alpha = n
+    g = torch.randn(n, f) * 1e-2
+    outg = ops.factor_linear(g.to(dev), False, float(n))
+    assert O.rel_fro(outg, O.factor_linear_g(g, D)) < TOL
+
+
+def test_factor_linear_fused_running_average(ops, dev):
+    torch.manual_seed(0)
+    for n, f in [(64, 300), (9000, 70)]:     # single pass and split-k paths
+        x = torch.randn(n, f)
+        old = spd(f + 1)
+        out = ops.factor_linear(x.to(dev), True, 0.95 / n, out=old.to(dev).clone(), beta=0.05)
+        ref = 0.95 * O.factor_linear_a(x, True, D) + 0.05 * old.double()
+        assert O.rel_fro(out, ref) < TOL
+
+
+@pytest.mark.parametrize('shape,k,s,p,d,bias', [
+    ((2, 3, 8, 8), (3, 3), (1, 1), (1, 1), (1, 1), True),
+    ((4, 3, 32, 32), (5, 5), (1, 1), (0, 0), (1, 1), True),
+    ((3, 5, 9, 11), (3, 3), (2, 2), (1, 1), (1, 1), False),
+    ((2, 4, 12, 12), (3, 3), (1, 1), (2, 2), (2, 2), True),
+    ((2, 3, 10, 9), (3, 2), (2, 1), (1, 0), (1, 2), True),
+    ((8, 64, 14, 14), (3, 3), (1, 1), (1, 1), (1, 1), False),
+    ((4, 16, 8, 8), (1, 1), (1, 1), (0, 0), (1, 1), True),
+    ((2, 3, 30, 30), (7, 7), (2, 2), (3, 3), (1, 1), False),
+    ((1, 1, 1, 1), (1, 1), (1, 1), (0, 0), (1, 1), True),
+    ((16, 32, 28, 28), (3, 3), (2, 2), (1, 1), (1, 1), False),
+])
+def test_factor_conv_a(ops, dev, shape, k, s, p, d, bias):
+    torch.manual_seed(sum(shape))
+    x = torch.randn(*shape)
+    out = ops.factor_conv_a(x.to(dev), k, s, p, d, bias, 1.0 / shape[0])
+    ref = O.factor_conv_a(x, k, s, p, d, bias, D)
+    assert out.shape == ref.shape
+    assert O.rel_fro(out, ref) < TOL
+    assert torch.equal(out, out.t())
+
+
+@pytest.mark.parametrize('shape', [(1, 1, 1, 1), (2, 3, 4, 4), (8, 64, 7, 7), (4, 130, 14, 14),
+                                   (16, 64, 56, 56), (3, 257, 5, 3)])
+def test_factor_conv_g(ops, dev, shape):
+    torch.manual_seed(sum(shape))
+    g = torch.randn(*shape) * 1e-2
+    n, c, h, w = shape
+    out = ops.factor_conv_g(g.to(dev), float(n) / (h * w))
+    assert O.rel_fro(out, O.factor_conv_g(g, D)) < TOL
+
+
+DIMS = [1, 2, 31, 32, 33, 64, 96, 97, 127, 128, 129, 255, 256, 257, 300, 513, 785]
+
+
+def test_damped_inverse_batched_mixed_sizes(ops, dev):
+    mats = [spd(n) for n in DIMS]
+    damps = [0.05 + 0.01 * i for i in range(len(DIMS))]
+    outs, info = ops.damped_inverse_batched([m.to(dev) for m in mats], damps)
+    assert info.cpu().tolist() == [0] * len(DIMS)
+    for m, d, o in zip(mats, damps, outs):
+        assert O.rel_fro(o, O.damped_inverse(m, d, D)) < TOL
+        assert torch.equal(o, o.t())
+
+
+def test_pi_damped_inverse_pairs(ops, dev):
+    As = [spd(785), spd(76), spd(1601), spd(10)]
+    Gs = [spd(1000) * 3, spd(64) * 0.01, spd(128) * 0.5, spd(129) * 40]
+    damp = [1e-3, 1e-2, 1e-3, 5e-3]
+    Ai, Gi, info = ops.pi_damped_inverse_batched([a.to(dev) for a in As], [g.to(dev) for g in Gs], damp)
+    assert info.cpu().tolist() == [0] * 8
+    for a, g, d, ai, gi in zip(As, Gs, damp, Ai, Gi):
+        ra, rg = O.pi_damped_inverse(a, g, d, D)
+        assert O.rel_fro(ai, ra) < TOL and O.rel_fro(gi, rg) < TOL
+
+
+def test_inverse_reports_non_spd_and_leaves_others_intact(ops, dev):
+    bad = spd(300)
+    bad[150, 150] = -5.0
+    good = spd(40)
+    outs, info = ops.damped_inverse_batched([bad.to(dev), good.to(dev)], [0.0, 0.0])
+    info = info.cpu().tolist()
+    assert info[0] == 151 and info[1] == 0
+    assert O.rel_fro(outs[1], O.damped_inverse(good, 0.0, D)) < TOL
+
+
+def test_cholesky_upper_batched(ops, dev):
+    mats = [spd(n) + 0.1 * torch.eye(n) for n in DIMS]
+    outs, info = ops.cholesky_upper_batched([m.to(dev) for m in mats])
+    assert info.cpu().tolist() == [0] * len(DIMS)
+    for m, o in zip(mats, outs):
+        assert O.rel_fro(o, O.cholesky_upper(m, D)) < TOL
+        assert torch.equal(o, torch.triu(o))
+
+
+SHAPES = [(10, 193, True), (64, 76, True), (1000, 785, True), (128, 1601, True),
+          (512, 1152, False), (1, 2, True), (3, 1, False), (64, 64, False), (130, 257, True)]
+
+
+def test_precondition_batched(ops, dev):
+    torch.manual_seed(1)
+    Gis = [spd(g) for g, a, b in SHAPES]
+    Ais = [spd(a) for g, a, b in SHAPES]
+    gws = [torch.randn(g, a - (1 if b else 0)) for g, a, b in SHAPES]
+    gbs = [torch.randn(g) if b else None for g, a, b in SHAPES]
+    dgw = [x.to(dev).clone() for x in gws]
+    dgb = [None if x is None else x.to(dev).clone() for x in gbs]
+    ops.precondition_batched([x.to(dev) for x in Gis], [x.to(dev) for x in Ais], dgw, dgb)
+    for i in range(len(SHAPES)):
+        rw, rb = O.precondition(Gis[i], Ais[i], gws[i], gbs[i], D)
+        assert O.rel_fro(dgw[i], rw) < TOL
+        if rb is not None:
+            assert O.rel_fro(dgb[i], rb) < TOL
+
+
+def test_precondition_conv_shaped_gradient(ops, dev):
+    torch.manual_seed(2)
+    Gi, Ai = spd(6), spd(4 * 3 * 3 + 1)
+    gw, gb = torch.randn(6, 4, 3, 3), torch.randn(6)
+    dw, db = gw.to(dev).clone(), gb.to(dev).clone()
+    ops.precondition_batched([Gi.to(dev)], [Ai.to(dev)], [dw], [db])
+    rw, rb = O.precondition(Gi, Ai, gw, gb, D)
+    assert dw.shape == gw.shape and O.rel_fro(dw, rw) < TOL and O.rel_fro(db, rb) < TOL
+
+
+def test_sample_batched(ops, dev):
+    torch.manual_seed(3)
+    UG = [O.cholesky_upper(spd(g) + 0.1 * torch.eye(g)) for g, a, b in SHAPES]
+    UA = [O.cholesky_upper(spd(a) + 0.1 * torch.eye(a)) for g, a, b in SHAPES]
+    noise = [torch.randn(g, a) for g, a, b in SHAPES]
+    mws = [torch.randn(g, a - (1 if b else 0)) for g, a, b in SHAPES]
+    mbs = [torch.randn(g) if b else None for g, a, b in SHAPES]
+    pw = [torch.empty_like(x).to(dev) for x in mws]
+    pb = [None if x is None else torch.empty_like(x).to(dev) for x in mbs]
+    ops.sample_batched([x.to(dev) for x in UG], [x.to(dev) for x in UA], [x.to(dev) for x in noise],
+                       [x.to(dev) for x in mws], [None if x is None else x.to(dev) for x in mbs],
+                       pw, pb, 0.37)
+    for i in range(len(SHAPES)):
+        rw, rb = O.sample(mws[i], mbs[i], UG[i], UA[i], noise[i], 0.37, D)
+        assert O.rel_fro(pw[i], rw) < TOL
+        if rb is not None:
+            assert O.rel_fro(pb[i], rb) < TOL
+
+
+def test_elementwise_tails(ops, dev):
+    torch.manual_seed(4)
+    sizes = [1, 100, 5000, 785000]
+    xs = [torch.randn(n) for n in sizes]
+    ys = [torch.randn(n) for n in sizes]
+    dys = [y.to(dev).clone() for y in ys]
+    ops.axpby_batched([x.to(dev) for x in xs], dys, 0.95, 0.05)
+    for d, x, y in zip(dys, xs, ys):
+        assert O.rel_fro(d, 0.95 * x.double() + 0.05 * y.double()) < 1e-6
+    lrs, moms, wds = [0.1, 0.2, 0.3], [0.9, 0.0, 0.5], [0.0, 1e-2, 1e-3]
+    ps = [torch.randn(n) for n in [7, 4097, 300000]]
+    gs = [torch.randn(n) for n in [7, 4097, 300000]]
+    bs = [torch.randn(n) for n in [7, 4097, 300000]]
+    dp = [p.to(dev).clone() for p in ps]
+    dg = [g.to(dev).clone() for g in gs]
+    db = [b.to(dev).clone() for b in bs]
+    ops.sgd_update_batched(dp, dg, [db[0], None, db[2]], lrs, moms, wds)
+    for i in range(3):
+        rp, rg, rb = O.sgd_tail(ps[i].double(), gs[i].double(), bs[i].double(), lrs[i], moms[i], wds[i])
+        assert O.rel_fro(dp[i], rp) < 1e-6 and O.rel_fro(dg[i], rg) < 1e-6
+        assert O.rel_fro(db[i], rb) < 1e-6
+    ema = torch.rand(50) + 0.1
+    inv = [torch.empty(50, device=dev)]
+    ops.diag_inverse_batched([ema.to(dev)], inv, [1e-3], False)
+    assert O.rel_fro(inv[0], O.diag_inverse(ema.double(), 1e-3)) < 1e-6
+    ops.diag_inverse_batched([ema.to(dev)], inv, [1e-3], True)
+    assert O.rel_fro(inv[0], O.diag_inverse(ema.double(), 1e-3, True)) < 1e-6
+    g = torch.randn(50)
+    dgr = [g.to(dev).clone()]
+    ops.diag_precondition_batched(inv, dgr)
+    assert O.rel_fro(dgr[0], g.double() * inv[0].cpu().double()) < 1e-6
+
+
+@pytest.mark.parametrize('shape', [(6, 10, 5, 5), (4, 3, 1, 1), (32, 64, 56, 56), (16, 7)])
+def test_batchnorm_diag(ops, dev, shape):
+    torch.manual_seed(5)
+    c = shape[1]
+    out = torch.randn(*shape)
+    w = torch.rand(c) + 0.5
+    b = torch.randn(c)
+    g = torch.randn(*shape) * 1e-2
+    ref = O.bn_diag(O.bn_restore_input(out.double(), w.double(), b.double()), g, True, D)
+    sx = ops.rowsq_sum(out.to(dev), c, w.to(dev), b.to(dev))
+    sg = ops.rowsq_sum(g.to(dev), c)
+    wc, bc = ops.bn_diag_combine(sx, sg, float(shape[0]), True)
+    assert O.rel_fro(wc, ref[0]) < TOL and O.rel_fro(bc, ref[1]) < TOL
+
+
+# ---- size-independent properties at the benchmark's sizes ---------------------
+
+def test_large_inverse_against_float64_library_inverse(ops, dev):
+    """4608 (largest ResNet-50 factor, batch 32) and 9217 (AlexNet fc6, batch
+    256, rank-deficient before damping): compared on the device with
+    torch.linalg.inv in float64 (a library routine, not the oracle's formula),
+    plus the residual X X^-1 - I, which for a float32 result scales with the
+    condition number (about 7e2 for the second case)."""
+    for n, L in [(4608, 1568), (9217, 256)]:
+        g = torch.Generator(device='cpu').manual_seed(n)
+        x = torch.randn(L, n, generator=g).to(dev)
+        X = ops.factor_linear(x, False, 1.0 / L)
+        damp = 0.05 * X.diagonal().mean().item()
+        outs, info = ops.damped_inverse_batched([X], [damp])
+        assert info.cpu().tolist() == [0]
+        Xd = X.double()
+        Xd.diagonal().add_(damp)
+        ref = torch.linalg.inv(Xd)
+        err = ((outs[0].double() - ref).norm() / ref.norm()).item()
+        res = (Xd @ outs[0].double() - torch.eye(n, device=dev, dtype=D)).norm().item() / n ** 0.5
+        print('n=%d rel err %.2e residual %.2e' % (n, err, res))
+        assert err < TOL, (n, err)
+        assert res < 1e-3, (n, res)
+        assert torch.equal(outs[0], outs[0].t())
+        del Xd, ref
+
+
+def test_factor_linearity_at_full_size(ops, dev):
+    """factor(x stacked with y) = factor(x) + factor(y) (sums of outer products),
+    on the ResNet-50 layer1 3x3 shape (c=64, 56x56, batch 32)."""
+    torch.manual_seed(6)
+    x = torch.randn(32, 64, 56, 56, device=dev)
+    full = ops.factor_conv_a(x, (3, 3), (1, 1), (1, 1), (1, 1), False, 1.0)
+    a = ops.factor_conv_a(x[:16].contiguous(), (3, 3), (1, 1), (1, 1), (1, 1), False, 1.0)
+    b = ops.factor_conv_a(x[16:].contiguous(), (3, 3), (1, 1), (1, 1), (1, 1), False, 1.0)
+    assert O.rel_fro(full, (a.double() + b.double())) < 1e-5
+    # and against F.unfold on the device in float64 for one image (library routine)
+    u = torch.nn.functional.unfold(x[:1].double(), 3, padding=1)[0]
+    one = ops.factor_conv_a(x[:1].contiguous(), (3, 3), (1, 1), (1, 1), (1, 1), False, 1.0)
+    assert O.rel_fro(one, u @ u.t()) < TOL

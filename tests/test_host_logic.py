@@ -1,0 +1,180 @@
+"""Host-side logic of the torchsso package without a GPU.
+
+The engine calls (torchsso._ops) are replaced, for these tests only, by the
+oracle-backed stand-in from kfac_testlib, so that the optimizers' sequencing --
+group construction, hook timing, accumulation, phase order, update rule -- can
+be checked on CPU tensors against the golden vectors the reference wrote.
+The product itself has no CPU path: the last tests check that it refuses."""
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+import torchsso
+from torchsso import _hip, _ops
+import kfac_testlib as T
+
+
+@pytest.fixture
+def oracle_ops(monkeypatch):
+    fake = T.OracleOps()
+    for name in dir(fake):
+        if not name.startswith('_') and callable(getattr(fake, name)) and hasattr(_ops, name):
+            monkeypatch.setattr(_ops, name, getattr(fake, name))
+    return fake
+
+
+def _closure(model, x, y):
+    def closure():
+        model.zero_grad()
+        out = model(x)
+        loss = F.cross_entropy(out, y)
+        loss.backward()
+        return loss, out
+    return closure
+
+
+def test_second_order_optimizer_matches_reference_mlp(oracle_ops):
+    gold = T.load_golden('ref_mlp_kfac')
+    model = T.load_init(T.build_mlp(), gold)
+    x, y = torch.from_numpy(gold['x']), torch.from_numpy(gold['y'])
+    opt = torchsso.optim.SecondOrderOptimizer(
+        model, 'Cov', {'Linear': 'Kron'}, {'damping': 1e-3, 'ema_decay': 0.95},
+        lr=0.05, momentum=0.9, l2_reg=1e-3, weight_decay=1e-3)
+    snaps = []
+    for s in range(3):
+        loss, _ = opt.step(closure=_closure(model, x, y))
+        assert abs(loss.item() - float(gold['step%d.loss' % s])) < 1e-4
+        snaps.append(T.snapshot_optimizer(opt))
+        assert abs(opt.param_groups[0]['curv'].damping - float(gold['step%d.g0.damping' % s])) < 1e-12
+    T.compare_with_golden(snaps, gold, 2e-4)
+    assert opt.optim_state == {'step': 3, 'acc_step': 0}
+
+
+def test_second_order_optimizer_matches_reference_convnet(oracle_ops):
+    gold = T.load_golden('ref_convnet_kfac')
+    model = T.load_init(T.build_convnet(), gold)
+    x, y = torch.from_numpy(gold['x']), torch.from_numpy(gold['y'])
+    opt = torchsso.optim.SecondOrderOptimizer(
+        model, 'Cov', {'Linear': 'Kron', 'Conv2d': 'Kron', 'BatchNorm2d': 'Diag'},
+        {'damping': 1e-2, 'ema_decay': 0.9}, lr=0.02, momentum=0.5, momentum_type='raw', l2_reg=1e-4)
+    names = [type(g['curv']).__name__ for g in opt.param_groups]
+    assert names == ['KronCovConv2d', 'DiagCovBatchNorm2d', 'KronCovConv2d', 'KronCovLinear']
+    snaps = []
+    for s in range(2):
+        opt.step(closure=_closure(model, x, y))
+        snaps.append(T.snapshot_optimizer(opt))
+    T.compare_with_golden(snaps, gold, 2e-4)
+
+
+def test_vi_optimizer_accumulation_matches_reference(oracle_ops):
+    gold = T.load_golden('ref_mlp_vi_nosample')
+    model = T.load_init(T.build_mlp(), gold)
+    x, y = torch.from_numpy(gold['x']), torch.from_numpy(gold['y'])
+    opt = torchsso.optim.VIOptimizer(
+        model, 100, 'Cov', {'Linear': 'Kron'}, {'damping': 1e-3, 'ema_decay': 0.95},
+        lr=0.05, momentum=0.9, num_mc_samples=3, prior_variance=0)
+    assert all(g['std_scale'] == 0 for g in opt.param_groups)
+    snaps = []
+    for s in range(2):
+        loss, prob = opt.step(closure=_closure(model, x, y))
+        assert abs(loss.item() - float(gold['step%d.loss' % s])) < 1e-4
+        # prob is accumulated with 1/acc_steps per MC sample (reference quirk, vi.py:209)
+        assert abs(prob.sum().item() - 3 * x.shape[0]) < 1e-3
+        snaps.append(T.snapshot_optimizer(opt))
+    T.compare_with_golden(snaps, gold, 2e-4)
+
+
+def test_vi_sampling_consumes_generator_in_group_order(oracle_ops):
+    """With a std present, params = mean + std_scale * U_G E U_A with E drawn by
+    torch.randn in param_group order after manual_seed(step + seed)."""
+    torch.manual_seed(3)
+    model = nn.Sequential(nn.Linear(6, 5), nn.ReLU(), nn.Linear(5, 3))
+    x, y = torch.randn(16, 6), torch.randint(0, 3, (16,))
+    opt = torchsso.optim.VIOptimizer(model, 200, 'Cov', {'Linear': 'Kron'},
+                                     {'damping': 1e-2, 'ema_decay': 0.9}, lr=0.01,
+                                     num_mc_samples=2, seed=5)
+    opt.step(closure=_closure(model, x, y))          # first step: no std yet -> mean only
+    assert all(g['curv'].std is not None for g in opt.param_groups)
+    means = [[m.clone() for m in g['mean']] for g in opt.param_groups]
+    opt.set_random_seed()
+    opt.sample_params()
+    torch.manual_seed(opt.optim_state['step'] + 5)
+    from oracle import kfac_oracle as O
+    for g, mean in zip(opt.param_groups, means):
+        A_ic, G_ic = g['curv'].std
+        E = torch.randn(G_ic.shape[0], A_ic.shape[0])
+        w, b = O.sample(mean[0], mean[1], G_ic, A_ic, E, g['std_scale'])
+        assert torch.allclose(g['params'][0].data, w, atol=1e-6)
+        assert torch.allclose(g['params'][1].data, b, atol=1e-6)
+    assert abs(opt.defaults['l2_reg'] - 1 / 200) < 1e-12
+    assert abs(opt.param_groups[0]['std_scale'] - (1 / 200) ** 0.5) < 1e-12
+
+
+def test_accumulation_steps_average_gradients_and_factors(oracle_ops):
+    torch.manual_seed(0)
+    model = nn.Sequential(nn.Linear(4, 3))
+    xs = [torch.randn(5, 4) for _ in range(2)]
+    ys = [torch.randint(0, 3, (5,)) for _ in range(2)]
+    opt = torchsso.optim.SecondOrderOptimizer(model, 'Cov', {'Linear': 'Kron'},
+                                              {'damping': 1e-2, 'ema_decay': 1.}, acc_steps=2)
+    w0 = model[0].weight.detach().clone()
+    opt.step(closure=_closure(model, xs[0], ys[0]))
+    assert torch.equal(model[0].weight.detach(), w0)          # no update yet
+    assert opt.optim_state == {'step': 0, 'acc_step': 1}
+    A0 = opt.param_groups[0]['curv'].A.clone()
+    seen = {}
+    inner = _closure(model, xs[1], ys[1])
+
+    def second():
+        ret = inner()
+        seen['A1'] = opt.param_groups[0]['curv'].A.clone()    # this pass's factor
+        return ret
+    opt.step(closure=second)
+    A1 = seen['A1']
+    assert opt.optim_state == {'step': 1, 'acc_step': 0}
+    assert not torch.equal(model[0].weight.detach(), w0)
+    assert torch.allclose(opt.param_groups[0]['curv'].ema[0], 0.5 * (A0 + A1), atol=1e-6)
+
+
+def test_constructor_validation_and_class_lookup():
+    model = nn.Sequential(nn.Linear(4, 3))
+    kw = dict(curv_type='Cov', curv_shapes={'Linear': 'Kron'}, curv_kwargs={'damping': 1e-3})
+    for bad in (dict(lr=-1), dict(momentum=-1), dict(momentum=0.9, momentum_type='x'),
+                dict(grad_ema_decay=2), dict(l2_reg=-1), dict(weight_decay=-1), dict(acc_steps=0),
+                dict(lars=True, lars_type='x')):
+        with pytest.raises(ValueError):
+            torchsso.optim.SecondOrderOptimizer(model, **kw, **bad)
+    for bad in ({'ema_decay': 1.5}, {'damping': -1e-3}, {'pi_type': 'other'}):
+        with pytest.raises(ValueError):
+            torchsso.optim.SecondOrderOptimizer(model, 'Cov', {'Linear': 'Kron'}, bad)
+    with pytest.raises(AssertionError):
+        torchsso.optim.SecondOrderOptimizer(model, 'Nope', {'Linear': 'Kron'}, {})
+    for bad in (dict(dataset_size=-1), dict(dataset_size=10, num_mc_samples=0),
+                dict(dataset_size=10, kl_weighting=-1), dict(dataset_size=10, prior_variance=-1)):
+        with pytest.raises(ValueError):
+            torchsso.optim.VIOptimizer(model, curv_type='Cov', curv_shapes={'Linear': 'Kron'},
+                                       curv_kwargs={}, **bad)
+    opt = torchsso.optim.SecondOrderOptimizer(model, **kw, momentum=0.9)
+    g = opt.param_groups[0]
+    for key in ('params', 'curv', 'acc_curv', 'acc_grads', 'lr', 'momentum', 'damping'):
+        assert key in g
+    assert g['curv'].shape == ((5, 5), (3, 3)) and g['curv'].bias
+    st = opt.state[g['params'][0]]
+    assert set(st) == {'momentum_buffer', 'grad_ema_buffer'}
+    # Kron element_wise_init puts sqrt(value) on both diagonals
+    g['curv'].element_wise_init(4.0)
+    assert torch.equal(g['curv'].A, 2 * torch.eye(5)) and torch.equal(g['curv'].G, 2 * torch.eye(3))
+
+
+def test_product_has_no_cpu_path():
+    """Without the stand-in, CPU tensors are refused loudly."""
+    model = nn.Sequential(nn.Linear(4, 3))
+    torchsso.optim.SecondOrderOptimizer(model, 'Cov', {'Linear': 'Kron'}, {})
+    with pytest.raises(_hip.KfacHipError):
+        model(torch.randn(2, 4))
+    with pytest.raises(_hip.KfacHipError):
+        torchsso.utils.inv(torch.eye(3))
+    acc = torchsso.utils.TensorAccumulator()
+    with pytest.raises(AssertionError):
+        acc.update([1.0, 2.0])
