@@ -5,26 +5,47 @@
 
 namespace kfac {
 
-int choose_splits(int ntiles, long K, int* chunks_per_split) {
+// Tile configuration and k-split of a symmetric d x d product reduced over K:
+// 64-wide single-wave tiles for small factors (a 128-wide tile would be mostly
+// padding), 128-wide tiles otherwise; enough k-splits to put about 8 waves on
+// every SIMD, each split at least 128 deep.
+struct SyrkPlan {
+  int w;        // waves per tile side: 1 -> 64x64 tiles, 2 -> 128x128
+  int ts;       // tile size
+  int T;        // tiles per side
+  int ntiles;   // upper-triangular tiles
+  int splits;
+  int cps;      // 16-deep chunks per split
+};
+
+static SyrkPlan plan_syrk(int d, long K) {
+  SyrkPlan p;
+  p.w = d <= 256 ? 1 : 2;
+  p.ts = 64 * p.w;
+  p.T = cdiv(d, p.ts);
+  p.ntiles = p.T * (p.T + 1) / 2;
   const long nchunks = (K + KC - 1) / KC;
-  long splits = TARGET_BLOCKS / ntiles;
+  const long target = 2048 / (p.w * p.w);
+  long splits = target / p.ntiles;
   if (splits < 1) splits = 1;
-  const long max_splits = nchunks / 8 > 0 ? nchunks / 8 : 1;  // >= 128 k per split
+  const long max_splits = nchunks / 8 > 0 ? nchunks / 8 : 1;
   if (splits > max_splits) splits = max_splits;
   long cps = (nchunks + splits - 1) / splits;
   if (cps < 1) cps = 1;
   splits = (nchunks + cps - 1) / cps;
   if (splits < 1) splits = 1;
-  *chunks_per_split = (int)cps;
-  return (int)splits;
+  p.splits = (int)splits;
+  p.cps = (int)cps;
+  return p;
 }
 
-template <class OP>
-__global__ __launch_bounds__(NTHREADS) void syrk_kernel(OP op, int d, int K, int T, int ntiles,
-                                                         int splits, int chunks_per_split,
-                                                         float* C, float alpha, float beta,
-                                                         float* ws) {
-  __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
+template <class OP, int W>
+__global__ __launch_bounds__(64 * W * W) void syrk_kernel(OP op, int d, int K, int T, int ntiles,
+                                                          int splits, int chunks_per_split,
+                                                          float* C, float alpha, float beta,
+                                                          float* ws) {
+  constexpr int TS = 64 * W;
+  __shared__ __attribute__((aligned(16))) float smem[Cfg<W, W>::SMEM_FLOATS];
   const int tile = blockIdx.x;
   const int split = blockIdx.y;
   int bi, bj;
@@ -34,54 +55,98 @@ __global__ __launch_bounds__(NTHREADS) void syrk_kernel(OP op, int d, int K, int
   if (kend > K) kend = K;
   if (splits == 1) {
     EpiStore epi{C, d, d, d, alpha, beta, bi != bj};
-    gemm_tile(op, op, bi * BM, bj * BN, kbeg, kend, bi == bj, epi, smem);
+    gemm_tile_cfg<W, W>(op, op, bi * TS, bj * TS, kbeg, kend, bi == bj, epi, smem);
   } else {
-    EpiPartial epi{ws + ((size_t)split * ntiles + tile) * (BM * BN), bi * BM, bj * BN, d, d};
-    gemm_tile(op, op, bi * BM, bj * BN, kbeg, kend, bi == bj, epi, smem);
+    EpiPartial epi{ws + ((size_t)split * ntiles + tile) * (TS * TS), bi * TS, bj * TS, d, d, TS};
+    gemm_tile_cfg<W, W>(op, op, bi * TS, bj * TS, kbeg, kend, bi == bj, epi, smem);
   }
 }
 
-// sum the k-split partials of one tile and apply the epilogue (+ mirror)
+// Sum the k-split partials of one tile in a fixed order and apply the epilogue
+// (+ mirror).  One workgroup owns 64 consecutive elements of a tile row:
+// 16 float4 groups x 16 split lanes; lane s adds splits s, s+16, ... and the 16
+// lane sums are then added in lane order, so the result does not depend on
+// scheduling.
+template <int TS>
 __global__ __launch_bounds__(256) void syrk_reduce_kernel(const float* ws, int d, int T,
                                                            int ntiles, int splits, float* C,
                                                            float alpha, float beta) {
+  __shared__ float4 red[16][16];
   const int tile = blockIdx.x;
   int bi, bj;
   upper_tile(tile, T, bi, bj);
+  constexpr int SEGS = TS / 64;
+  const int lrow = blockIdx.y / SEGS;
+  const int seg = blockIdx.y - lrow * SEGS;
+  const int row = bi * TS + lrow;
+  const int col0 = bj * TS + seg * 64;
+  if (row >= d || col0 >= d) return;
+  const int g = threadIdx.x & 15;
+  const int sl = threadIdx.x >> 4;
+  const size_t e = (size_t)lrow * TS + seg * 64 + 4 * g;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  const size_t stride = (size_t)ntiles * (TS * TS);
+  const float* base = ws + (size_t)tile * (TS * TS) + e;
+#pragma unroll 4
+  for (int sp = sl; sp < splits; sp += 16) {
+    const float4 v = *reinterpret_cast<const float4*>(base + (size_t)sp * stride);
+    acc.x += v.x;
+    acc.y += v.y;
+    acc.z += v.z;
+    acc.w += v.w;
+  }
+  red[sl][g] = acc;
+  __syncthreads();
+  if (sl == 0) {
+    float4 s = red[0][g];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int e = blockIdx.y * 1024 + i * 256 + threadIdx.x;
-    const int row = bi * BM + (e >> 7);
-    const int col = bj * BN + (e & 127);
-    if (row < d && col < d) {
-      float s = 0.f;
-      for (int sp = 0; sp < splits; ++sp) s += ws[((size_t)sp * ntiles + tile) * (BM * BN) + e];
-      const size_t idx = (size_t)row * d + col;
-      float o = alpha * s;
-      if (beta != 0.f) o += beta * C[idx];
-      C[idx] = o;
-      if (bi != bj) C[(size_t)col * d + row] = o;
+    for (int k = 1; k < 16; ++k) {
+      const float4 v = red[k][g];
+      s.x += v.x;
+      s.y += v.y;
+      s.z += v.z;
+      s.w += v.w;
     }
+    const float vals[4] = {s.x, s.y, s.z, s.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int col = col0 + 4 * g + k;
+      if (col < d) {
+        const size_t idx = (size_t)row * d + col;
+        float o = alpha * vals[k];
+        if (beta != 0.f) o += beta * C[idx];
+        C[idx] = o;
+        if (bi != bj) C[(size_t)col * d + row] = o;
+      }
+    }
+  }
+}
+
+template <class OP, int W>
+static void launch_syrk_cfg(const OP& op, const SyrkPlan& p, int d, int64_t K, float alpha,
+                            float beta, float* C, void* workspace, hipStream_t stream) {
+  constexpr int TS = 64 * W;
+  hipLaunchKernelGGL((syrk_kernel<OP, W>), dim3(p.ntiles, p.splits), dim3(64 * W * W), 0, stream,
+                     op, d, (int)K, p.T, p.ntiles, p.splits, p.cps, C, alpha, beta,
+                     (float*)workspace);
+  if (p.splits > 1) {
+    hipLaunchKernelGGL((syrk_reduce_kernel<TS>), dim3(p.ntiles, TS * (TS / 64)), dim3(256), 0,
+                       stream, (const float*)workspace, d, p.T, p.ntiles, p.splits, C, alpha, beta);
   }
 }
 
 template <class OP>
 static int launch_syrk(const OP& op, int d, int64_t K, float alpha, float beta, float* C,
                        void* workspace, size_t workspace_bytes, hipStream_t stream) {
-  const int T = cdiv(d, BM);
-  const int ntiles = T * (T + 1) / 2;
-  int cps;
-  const int splits = choose_splits(ntiles, (long)K, &cps);
-  if (splits > 1) {
-    const size_t need = (size_t)splits * ntiles * BM * BN * sizeof(float);
+  const SyrkPlan p = plan_syrk(d, (long)K);
+  if (p.splits > 1) {
+    const size_t need = (size_t)p.splits * p.ntiles * p.ts * p.ts * sizeof(float);
     if (workspace == nullptr || workspace_bytes < need) return KFAC_ERR_WORKSPACE;
   }
-  hipLaunchKernelGGL((syrk_kernel<OP>), dim3(ntiles, splits), dim3(NTHREADS), 0, stream, op, d,
-                     (int)K, T, ntiles, splits, cps, C, alpha, beta, (float*)workspace);
-  if (splits > 1) {
-    hipLaunchKernelGGL(syrk_reduce_kernel, dim3(ntiles, 16), dim3(256), 0, stream,
-                       (const float*)workspace, d, T, ntiles, splits, C, alpha, beta);
-  }
+  if (p.w == 1)
+    launch_syrk_cfg<OP, 1>(op, p, d, K, alpha, beta, C, workspace, stream);
+  else
+    launch_syrk_cfg<OP, 2>(op, p, d, K, alpha, beta, C, workspace, stream);
   return launch_status();
 }
 
@@ -95,11 +160,8 @@ int kfac_abi_version(void) { return 1; }
 
 size_t kfac_factor_workspace_bytes(int d, int64_t K) {
   if (d <= 0 || K <= 0) return 0;
-  const int T = cdiv(d, BM);
-  const int ntiles = T * (T + 1) / 2;
-  int cps;
-  const int splits = choose_splits(ntiles, (long)K, &cps);
-  return splits > 1 ? (size_t)splits * ntiles * BM * BN * sizeof(float) : 0;
+  const SyrkPlan p = plan_syrk(d, (long)K);
+  return p.splits > 1 ? (size_t)p.splits * p.ntiles * p.ts * p.ts * sizeof(float) : 0;
 }
 
 int kfac_factor_linear(const float* x, int64_t rows, int f, int64_t ldx, int add_bias,

@@ -28,13 +28,26 @@
 
 namespace kfac {
 
-constexpr int BM = 128;          // tile rows
-constexpr int BN = 128;          // tile cols
+constexpr int BM = 128;          // tile rows of the default (2x2 waves) configuration
+constexpr int BN = 128;          // tile cols of the default configuration
 constexpr int KC = 16;           // reduction depth per LDS stage
-constexpr int NTHREADS = 256;
+constexpr int NTHREADS = 256;    // threads of the default configuration
 constexpr int LDS_MK = KC + 4;   // padded row of an MK chunk (bank-conflict free b128)
-constexpr int TILE_FLOATS = 2560;  // >= KC*BM and >= BM*LDS_MK
-constexpr int SMEM_FLOATS = 4 * TILE_FLOATS;  // 2 operands x 2 stages = 40 KiB
+
+// A configuration is WM x WN waves, each owning a 64x64 sub-tile:
+//   tile = (64*WM) x (64*WN), threads = 64*WM*WN.
+// 2x2 is the default; 1x1 (one wave, 64x64) serves small factors, where a
+// 128-wide tile would be mostly padding.
+template <int WM, int WN>
+struct Cfg {
+  static constexpr int TM = 64 * WM;
+  static constexpr int TN = 64 * WN;
+  static constexpr int NT = 64 * WM * WN;
+  static constexpr int P_FLOATS = LDS_MK * TM;   // >= KC*TM and TM*LDS_MK
+  static constexpr int Q_FLOATS = LDS_MK * TN;
+  static constexpr int SMEM_FLOATS = 2 * (P_FLOATS + Q_FLOATS);
+};
+constexpr int SMEM_FLOATS = Cfg<2, 2>::SMEM_FLOATS;   // 40 KiB
 
 enum { KM = 0, MK = 1 };
 
@@ -43,21 +56,25 @@ __host__ __device__ inline int tiles128(int d) { return (d + BM - 1) / BM; }
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 // ---------------------------------------------------------------------------
-// global -> register -> LDS staging of one operand chunk
+// global -> register -> LDS staging of one operand chunk (KC x ROWS elements
+// swept by NT threads)
 // ---------------------------------------------------------------------------
-template <class OP>
+template <class OP, int ROWS, int NT>
 struct Stager {
-  static constexpr int NM = (OP::layout == KM) ? 1 : 8;
+  static constexpr int CNT = KC * ROWS / NT;            // elements per thread
+  static constexpr int NM = (OP::layout == KM) ? 1 : CNT;
+  static constexpr int KSTEP = NT / ROWS;               // KM: k rows per sweep
+  static constexpr int MSTEP = NT / KC;                 // MK: m rows per sweep
   typename OP::MS ms[NM];
-  float regs[8];
+  float regs[CNT];
 
   __device__ __forceinline__ void init(const OP& op, int m0) {
     const int t = threadIdx.x;
     if (OP::layout == KM) {
-      ms[0] = op.mstate(m0 + (t & 127));
+      ms[0] = op.mstate(m0 + (t % ROWS));
     } else {
 #pragma unroll
-      for (int i = 0; i < NM; ++i) ms[i] = op.mstate(m0 + (t >> 4) + 16 * i);
+      for (int i = 0; i < NM; ++i) ms[i] = op.mstate(m0 + (t / KC) + MSTEP * i);
     }
   }
 
@@ -65,16 +82,16 @@ struct Stager {
     const int t = threadIdx.x;
     if (OP::layout == KM) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int k = k0 + (t >> 7) + 2 * i;
+      for (int i = 0; i < CNT; ++i) {
+        const int k = k0 + (t / ROWS) + KSTEP * i;
         regs[i] = (k < kend) ? op.load(ms[0], op.kstate(k)) : 0.f;
       }
     } else {
-      const int k = k0 + (t & 15);
+      const int k = k0 + (t % KC);
       const bool kin = k < kend;
       const typename OP::KS ks = op.kstate(kin ? k : k0);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) regs[i] = kin ? op.load(ms[i], ks) : 0.f;
+      for (int i = 0; i < CNT; ++i) regs[i] = kin ? op.load(ms[i], ks) : 0.f;
     }
   }
 
@@ -82,16 +99,16 @@ struct Stager {
     const int t = threadIdx.x;
     if (OP::layout == KM) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) tile[((t >> 7) + 2 * i) * BM + (t & 127)] = regs[i];
+      for (int i = 0; i < CNT; ++i) tile[((t / ROWS) + KSTEP * i) * ROWS + (t % ROWS)] = regs[i];
     } else {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) tile[((t >> 4) + 16 * i) * LDS_MK + (t & 15)] = regs[i];
+      for (int i = 0; i < CNT; ++i) tile[((t / KC) + MSTEP * i) * LDS_MK + (t % KC)] = regs[i];
     }
   }
 };
 
 // fragments of one operand for the 8 MFMA steps of a chunk: f[sub][4j+s]
-template <int LAYOUT>
+template <int LAYOUT, int ROWS>
 __device__ __forceinline__ void load_frags(const float* tile, int base, int r, int h,
                                            float (&f)[2][8]) {
   if (LAYOUT == KM) {
@@ -101,7 +118,7 @@ __device__ __forceinline__ void load_frags(const float* tile, int base, int r, i
       for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int s = 0; s < 4; ++s)
-          f[sub][4 * j + s] = tile[(8 * j + 4 * h + s) * BM + base + 32 * sub + r];
+          f[sub][4 * j + s] = tile[(8 * j + 4 * h + s) * ROWS + base + 32 * sub + r];
   } else {
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub)
@@ -118,21 +135,23 @@ __device__ __forceinline__ void load_frags(const float* tile, int base, int r, i
 }
 
 // ---------------------------------------------------------------------------
-// The tile engine.  `same` = P and Q describe the same 128 columns (diagonal
-// tile of a symmetric product): Q is then neither fetched nor stored.
-// EPI::store(row, col, value) receives every element of the 128x128 tile
-// (global coordinates row = m0 + ..., col = n0 + ...).
+// The tile engine.  `same` = P and Q describe the same columns (diagonal tile
+// of a symmetric product): Q is then neither fetched nor stored.
+// EPI::store(row, col, value) receives every element of the tile (global
+// coordinates row = m0 + ..., col = n0 + ...).
 // ---------------------------------------------------------------------------
-template <class OPP, class OPQ, class EPI>
-__device__ __forceinline__ void gemm_tile(const OPP& P, const OPQ& Q, int m0, int n0, int kbeg,
-                                          int kend, bool same, EPI& epi, float* smem) {
+template <int WM, int WN, class OPP, class OPQ, class EPI>
+__device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0, int n0,
+                                              int kbeg, int kend, bool same, EPI& epi,
+                                              float* smem) {
+  typedef Cfg<WM, WN> C;
   const int t = threadIdx.x;
   const int lane = t & 63;
   const int wave = t >> 6;
   const int r = lane & 31;
   const int h = lane >> 5;
-  const int wm = (wave >> 1) * 64;
-  const int wn = (wave & 1) * 64;
+  const int wm = (wave / WN) * 64;
+  const int wn = (wave % WN) * 64;
 
   v16f acc[2][2];
 #pragma unroll
@@ -142,13 +161,13 @@ __device__ __forceinline__ void gemm_tile(const OPP& P, const OPQ& Q, int m0, in
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
 
-  Stager<OPP> sp;
-  Stager<OPQ> sq;
+  Stager<OPP, C::TM, C::NT> sp;
+  Stager<OPQ, C::TN, C::NT> sq;
   sp.init(P, m0);
   if (!same) sq.init(Q, n0);
 
-  float* tp[2] = {smem, smem + 2 * TILE_FLOATS};
-  float* tq[2] = {smem + TILE_FLOATS, smem + 3 * TILE_FLOATS};
+  float* tp[2] = {smem, smem + C::P_FLOATS + C::Q_FLOATS};
+  float* tq[2] = {smem + C::P_FLOATS, smem + 2 * C::P_FLOATS + C::Q_FLOATS};
 
   const int nchunks = (kend - kbeg + KC - 1) / KC;
   if (nchunks > 0) {
@@ -167,11 +186,11 @@ __device__ __forceinline__ void gemm_tile(const OPP& P, const OPQ& Q, int m0, in
       if (!same) sq.fetch(Q, kbeg + (c + 1) * KC, kend);
     }
     float fa[2][8], fb[2][8];
-    load_frags<OPP::layout>(tp[cur], wm, r, h, fa);
+    load_frags<OPP::layout, C::TM>(tp[cur], wm, r, h, fa);
     if (same)
-      load_frags<OPP::layout>(tp[cur], wn, r, h, fb);
+      load_frags<OPP::layout, C::TM>(tp[cur], wn, r, h, fb);
     else
-      load_frags<OPQ::layout>(tq[cur], wn, r, h, fb);
+      load_frags<OPQ::layout, C::TN>(tq[cur], wn, r, h, fb);
 #pragma unroll
     for (int s = 0; s < 8; ++s)
 #pragma unroll
@@ -198,6 +217,13 @@ __device__ __forceinline__ void gemm_tile(const OPP& P, const OPQ& Q, int m0, in
         const int col = n0 + wn + 32 * b + r;
         epi.store(row, col, acc[a][b][i]);
       }
+}
+
+// default configuration: 128x128 tile, 256 threads
+template <class OPP, class OPQ, class EPI>
+__device__ __forceinline__ void gemm_tile(const OPP& P, const OPQ& Q, int m0, int n0, int kbeg,
+                                          int kend, bool same, EPI& epi, float* smem) {
+  gemm_tile_cfg<2, 2>(P, Q, m0, n0, kbeg, kend, same, epi, smem);
 }
 
 // tile index t (0-based, row-major over the upper triangle incl. diagonal of a

@@ -151,25 +151,61 @@ __device__ __forceinline__ void chol_inv_32(float* S, float* Yb, int c0, int row
   }
 }
 
+// One wave: acc(32x32) = sum_{k<K} A(k, i) * B(k, j) with operands in LDS,
+//   A(k, i) = a[k*a_ks + i*a_is],  B(k, j) = b[k*b_ks + j*b_js]   (K even).
+// Result element t of lane (r, h): row 8*(t/4) + 4h + t%4, column r.
+__device__ __forceinline__ v16f lds_mma32(const float* a, int a_ks, int a_is, const float* b,
+                                          int b_ks, int b_js, int K) {
+  const int lane = threadIdx.x & 63;
+  const int r = lane & 31, h = lane >> 5;
+  v16f acc;
+#pragma unroll
+  for (int t = 0; t < 16; ++t) acc[t] = 0.f;
+  const float* pa = a + h * a_ks + r * a_is;
+  const float* pb = b + h * b_ks + r * b_js;
+#pragma unroll 4
+  for (int k = 0; k < K; k += 2) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[k * a_ks], pb[k * b_ks], acc, 0, 0, 0);
+  }
+  return acc;
+}
+
+// store / subtract a 32x32 result block at c[row*ld + col]
+__device__ __forceinline__ void lds_put32(float* c, int ld, const v16f& acc, float scale) {
+  const int lane = threadIdx.x & 63;
+  const int r = lane & 31, h = lane >> 5;
+#pragma unroll
+  for (int t = 0; t < 16; ++t) c[(8 * (t >> 2) + 4 * h + (t & 3)) * ld + r] = scale * acc[t];
+}
+__device__ __forceinline__ void lds_sub32(float* c, int ld, const v16f& acc) {
+  const int lane = threadIdx.x & 63;
+  const int r = lane & 31, h = lane >> 5;
+#pragma unroll
+  for (int t = 0; t < 16; ++t) c[(8 * (t >> 2) + 4 * h + (t & 3)) * ld + r] -= acc[t];
+}
+
 // In-LDS off-diagonal inverse block:  Y12 = -Y11 * (U12 * Y22) for the pair
-// X1 = [s1, s1+b), X2 = [s1+b, s1+2b);  W is a b x b scratch (b <= 64).
-__device__ __forceinline__ void tri_pair(const float* S, float* Yb, float* Wt, int s1, int b) {
+// X1 = [s1, s1+b), X2 = [s1+b, s1+2b), b = 32 or 64; W is a b x b scratch.
+// 32x32 result blocks are dealt round-robin to the 4 waves.
+__device__ __forceinline__ void tri_pair(const float* S, float* Yb, float* Wt, int s1, int b,
+                                         int wave_first, int wave_count) {
   const int s2 = s1 + b;
-  const int t = threadIdx.x;
-  // W[i][j] = sum_{k<=j} U12[i][k] * Y22[k][j]
-  for (int e = t; e < b * b; e += 256) {
-    const int i = e / b, j = e - i * b;
-    float s = 0.f;
-    for (int k = 0; k <= j; ++k) s += S[(s1 + i) * DLD + s2 + k] * Yb[(s2 + k) * DLD + s2 + j];
-    Wt[i * WLD + j] = s;
+  const int wave = (int)(threadIdx.x >> 6) - wave_first;
+  const int nb = b / 32;
+  // W[i][j] = sum_k U12[i][k] * Y22[k][j]     (Y22 is zero below its diagonal)
+  for (int blk = wave; blk < nb * nb && wave >= 0; blk += wave_count) {
+    const int bi = blk / nb, bj = blk - bi * nb;
+    const v16f acc = lds_mma32(S + (s1 + 32 * bi) * DLD + s2, 1, DLD,
+                               Yb + s2 * DLD + s2 + 32 * bj, DLD, 1, 32 * (bj + 1));
+    lds_put32(Wt + 32 * bi * WLD + 32 * bj, WLD, acc, 1.f);
   }
   __syncthreads();
-  // Y12[i][j] = - sum_{k>=i} Y11[i][k] * W[k][j]
-  for (int e = t; e < b * b; e += 256) {
-    const int i = e / b, j = e - i * b;
-    float s = 0.f;
-    for (int k = i; k < b; ++k) s += Yb[(s1 + i) * DLD + s1 + k] * Wt[k * WLD + j];
-    Yb[(s1 + i) * DLD + s2 + j] = -s;
+  // Y12[i][j] = - sum_{k} Y11[i][k] * W[k][j]  (Y11 is zero below its diagonal)
+  for (int blk = wave; blk < nb * nb && wave >= 0; blk += wave_count) {
+    const int bi = blk / nb, bj = blk - bi * nb;
+    const v16f acc = lds_mma32(Yb + (s1 + 32 * bi) * DLD + s1 + 32 * bi, 1, DLD,
+                               Wt + 32 * bi * WLD + 32 * bj, WLD, 1, b - 32 * bi);
+    lds_put32(Yb + (s1 + 32 * bi) * DLD + s2 + 32 * bj, DLD, acc, -1.f);
   }
   __syncthreads();
 }
@@ -184,8 +220,9 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
   const int r0 = p * DB;
   const int nb = min(DB, n - r0);
   const int t = threadIdx.x;
+  const int wave = t >> 6;
 
-  // load the upper triangle; pad with the identity up to the next multiple of 32
+  // load the upper triangle; pad with the identity up to 128
   for (int e = t; e < DB * DB; e += 256) {
     const int i = e >> 7, j = e & 127;
     float v = 0.f;
@@ -204,34 +241,23 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
     const int c0 = 32 * q;
     if (t < 64) chol_inv_32(S, Yb, c0, r0, info + m.out);
     __syncthreads();
-    const int c1 = c0 + 32;
-    const int rest = 32 * nq - c1;   // columns to the right
+    const int rest = nq - q - 1;     // 32-blocks to the right
     if (rest > 0) {
-      // row panel: U[c0+i][c1+j] = sum_k Yqq[k][i] * A[c0+k][c1+j]   (k <= i)
-      float out[12];
-      int cnt = 0;
-      for (int e = t; e < 32 * rest; e += 256, ++cnt) {
-        const int i = e / rest, jj = e - i * rest;
-        float s = 0.f;
-        for (int k = 0; k <= i; ++k) s += Yb[(c0 + k) * DLD + c0 + i] * S[(c0 + k) * DLD + c1 + jj];
-        out[cnt] = s;
+      // row panel: U[q][j] = Yqq^T A[q][j], one 32x32 block per wave, in place
+      if (wave < rest) {
+        const int cj = c0 + 32 * (wave + 1);
+        const v16f acc = lds_mma32(Yb + c0 * DLD + c0, DLD, 1, S + c0 * DLD + cj, DLD, 1, 32);
+        lds_put32(S + c0 * DLD + cj, DLD, acc, 1.f);
       }
       __syncthreads();
-      cnt = 0;
-      for (int e = t; e < 32 * rest; e += 256, ++cnt) {
-        const int i = e / rest, jj = e - i * rest;
-        S[(c0 + i) * DLD + c1 + jj] = out[cnt];
-      }
-      __syncthreads();
-      // trailing update: A[c1+i][c1+j] -= sum_k U[c0+k][c1+i] * U[c0+k][c1+j],  j >= i
-      for (int e = t; e < rest * rest; e += 256) {
-        const int i = e / rest, jj = e - i * rest;
-        if (jj >= i) {
-          float s = 0.f;
-#pragma unroll 8
-          for (int k = 0; k < 32; ++k) s += S[(c0 + k) * DLD + c1 + i] * S[(c0 + k) * DLD + c1 + jj];
-          S[(c1 + i) * DLD + c1 + jj] -= s;
-        }
+      // trailing update: A[i][j] -= U[q][i]^T U[q][j], q < i <= j
+      const int nblk = rest * (rest + 1) / 2;
+      for (int blk = wave; blk < nblk; blk += 4) {
+        int bi, bj;
+        upper_tile(blk, rest, bi, bj);
+        const int ci = c0 + 32 * (bi + 1), cj = c0 + 32 * (bj + 1);
+        const v16f acc = lds_mma32(S + c0 * DLD + ci, DLD, 1, S + c0 * DLD + cj, DLD, 1, 32);
+        lds_sub32(S + ci * DLD + cj, DLD, acc);
       }
       __syncthreads();
     }
@@ -239,11 +265,16 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
 
   // inverse of the whole block by doubling: 32 -> 64 -> 128
   if (nq > 1) {
-    tri_pair(S, Yb, Wt, 0, 32);
-    if (nq > 3) tri_pair(S, Yb, Wt, 64, 32);
-    else if (nq > 2) { /* X2 of the second pair is padding: nothing to do */ }
+    // the two level-32 pairs use disjoint data: waves 0-1 take the first, 2-3 the second
+    // (both calls contain the same two barriers, reached by every wave)
+    if (nq > 3) {
+      const int s1 = wave < 2 ? 0 : 64;
+      tri_pair(S, Yb, Wt + (wave < 2 ? 0 : 32 * WLD), s1, 32, wave < 2 ? 0 : 2, 2);
+    } else {
+      tri_pair(S, Yb, Wt, 0, 32, 0, 4);
+    }
   }
-  if (nq > 2) tri_pair(S, Yb, Wt, 0, 64);
+  if (nq > 2) tri_pair(S, Yb, Wt, 0, 64, 0, 4);
 
   for (int e = t; e < DB * DB; e += 256) {
     const int i = e >> 7, j = e & 127;
@@ -286,45 +317,71 @@ __global__ __launch_bounds__(NTHREADS) void potrf_trail_kernel(const MatDesc* ta
   gemm_tile(P, P, bi * BM, bj * BN, 0, DB, bi == bj, epi, smem);
 }
 
-// level l of the doubling inverse, first product:
-//   W^T[j][i] = sum_{k <= j} Y22[k][j] * U12[i][k]   stored at Y[X2 rows][X1 cols]
-__global__ __launch_bounds__(NTHREADS) void trtri_w_kernel(const MatDesc* table, int l) {
+// ---- Y = U^-1 by balanced recursive halving over the 128-blocks ---------------
+// Depth d cuts the T blocks of a matrix into 2^d nearly equal segments
+// (boundaries floor(j*T/2^d)); the merge of the two children X1, X2 of a
+// depth-d segment computes  Y12 = -Y11 * U12 * Y22.  A pair of blocks
+// (bi < bj) belongs to the merge of the deepest segment that contains both, so
+// every launch below walks all strictly-upper block pairs and keeps those whose
+// merge is at its depth.
+struct MergeTile {
+  int X1, b1, X2, b2, it, jt;
+  bool valid;
+};
+
+__device__ __forceinline__ int seg_of(int b, int depth, int T) {
+  return (int)((((long)(b + 1) << depth) - 1) / T);
+}
+
+__device__ __forceinline__ MergeTile merge_tile(const MatDesc& m, int depth) {
+  MergeTile t;
+  t.valid = false;
+  const int T = m.T;
+  if (T < 2 || (int)blockIdx.x >= (T - 1) * T / 2) return t;
+  int bi, bj;
+  upper_tile(blockIdx.x, T - 1, bi, bj);
+  bj += 1;
+  const int P = seg_of(bi, depth, T);
+  if (seg_of(bj, depth, T) != P) return t;
+  if (seg_of(bi, depth + 1, T) == seg_of(bj, depth + 1, T)) return t;
+  const int p0 = (int)(((long)P * T) >> depth);
+  const int p1 = (int)(((long)(P + 1) * T) >> depth);
+  const int mid = (int)(((long)(2 * P + 1) * T) >> (depth + 1));
+  t.X1 = p0 * DB;
+  t.b1 = (mid - p0) * DB;
+  t.X2 = mid * DB;
+  t.b2 = min((p1 - mid) * DB, m.n - t.X2);
+  t.it = bi - p0;
+  t.jt = bj - mid;
+  t.valid = true;
+  return t;
+}
+
+// first product:  W^T[j][i] = sum_{k <= j} Y22[k][j] * U12[i][k], stored at
+// Y[X2 rows][X1 cols] (the unused lower triangle of Y)
+__global__ __launch_bounds__(NTHREADS) void trtri_w_kernel(const MatDesc* table, int depth) {
   __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
   const MatDesc m = table[blockIdx.y];
-  const int tl = 1 << l;                     // 128-blocks per half
-  const int pair = blockIdx.x >> (2 * l);
-  const int within = blockIdx.x & ((1 << (2 * l)) - 1);
-  const int it = within >> l, jt = within & (tl - 1);
-  const int s1 = pair * 2 * tl, s2 = s1 + tl;   // in 128-blocks
-  if (s2 + jt >= m.T) return;
+  const MergeTile t = merge_tile(m, depth);
+  if (!t.valid) return;
   const int n = m.n;
-  const int X1 = s1 * DB, X2 = s2 * DB;
-  const int b1 = tl * DB;
-  const int b2 = min(b1, n - X2);
-  DenseKM P{m.Y + (size_t)X2 * n + X2, nullptr, n, b2, 0};
-  DenseMK Q{m.U + (size_t)X1 * n + X2, n, b1};
-  EpiStore epi{m.Y + (size_t)X2 * n + X1, n, b2, b1, 1.f, 0.f, false};
-  gemm_tile(P, Q, jt * BM, it * BN, 0, min(b2, (jt + 1) * DB), false, epi, smem);
+  DenseKM P{m.Y + (size_t)t.X2 * n + t.X2, nullptr, n, t.b2, 0};
+  DenseMK Q{m.U + (size_t)t.X1 * n + t.X2, n, t.b1};
+  EpiStore epi{m.Y + (size_t)t.X2 * n + t.X1, n, t.b2, t.b1, 1.f, 0.f, false};
+  gemm_tile(P, Q, t.jt * BM, t.it * BN, 0, min(t.b2, (t.jt + 1) * DB), false, epi, smem);
 }
 
 // second product:  Y12[i][j] = - sum_{k >= i} Y11[i][k] * W^T[j][k]
-__global__ __launch_bounds__(NTHREADS) void trtri_y_kernel(const MatDesc* table, int l) {
+__global__ __launch_bounds__(NTHREADS) void trtri_y_kernel(const MatDesc* table, int depth) {
   __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
   const MatDesc m = table[blockIdx.y];
-  const int tl = 1 << l;
-  const int pair = blockIdx.x >> (2 * l);
-  const int within = blockIdx.x & ((1 << (2 * l)) - 1);
-  const int it = within >> l, jt = within & (tl - 1);
-  const int s1 = pair * 2 * tl, s2 = s1 + tl;
-  if (s2 + jt >= m.T) return;
+  const MergeTile t = merge_tile(m, depth);
+  if (!t.valid) return;
   const int n = m.n;
-  const int X1 = s1 * DB, X2 = s2 * DB;
-  const int b1 = tl * DB;
-  const int b2 = min(b1, n - X2);
-  DenseMK P{m.Y + (size_t)X1 * n + X1, n, b1};
-  DenseMK Q{m.Y + (size_t)X2 * n + X1, n, b2};
-  EpiStore epi{m.Y + (size_t)X1 * n + X2, n, b1, b2, -1.f, 0.f, false};
-  gemm_tile(P, Q, it * BM, jt * BN, it * DB, b1, false, epi, smem);
+  DenseMK P{m.Y + (size_t)t.X1 * n + t.X1, n, t.b1};
+  DenseMK Q{m.Y + (size_t)t.X2 * n + t.X1, n, t.b2};
+  EpiStore epi{m.Y + (size_t)t.X1 * n + t.X2, n, t.b1, t.b2, -1.f, 0.f, false};
+  gemm_tile(P, Q, t.it * BM, t.jt * BN, t.it * DB, t.b1, false, epi, smem);
 }
 
 // dst = Y Y^T over the upper tiles (k >= the later block), mirrored
@@ -459,13 +516,15 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
     hipLaunchKernelGGL(zero_lower_kernel, dim3(Tmax * Tmax, nmat), dim3(256), 0, stream, table);
     return launch_status();
   }
-  for (int l = 0; (1 << l) < Tmax; ++l) {
-    const int na = active((1 << l) + 1);
-    if (na == 0) break;
-    const int npairs = cdiv(Tmax, 2 << l);
-    const dim3 grid(npairs << (2 * l), na);
-    hipLaunchKernelGGL(trtri_w_kernel, grid, dim3(NTHREADS), 0, stream, table, l);
-    hipLaunchKernelGGL(trtri_y_kernel, grid, dim3(NTHREADS), 0, stream, table, l);
+  if (Tmax > 1) {
+    int D = 0;
+    while ((1 << D) < Tmax) ++D;
+    const int na = active(2);
+    const dim3 grid((Tmax - 1) * Tmax / 2, na);
+    for (int depth = D - 1; depth >= 0 && na > 0; --depth) {
+      hipLaunchKernelGGL(trtri_w_kernel, grid, dim3(NTHREADS), 0, stream, table, depth);
+      hipLaunchKernelGGL(trtri_y_kernel, grid, dim3(NTHREADS), 0, stream, table, depth);
+    }
   }
   hipLaunchKernelGGL(lauum_kernel, dim3(Tmax * (Tmax + 1) / 2, nmat), dim3(NTHREADS), 0, stream,
                      table);

@@ -132,9 +132,9 @@ struct EpiStore {
 // raw partial sums of one k-split into a tile-packed workspace
 struct EpiPartial {
   float* ws;      // already offset to this (split, tile)
-  int m0, n0, M, N;
+  int m0, n0, M, N, tn;   // tn = tile width
   __device__ __forceinline__ void store(int row, int col, float v) const {
-    if (row < M && col < N) ws[(row - m0) * BN + (col - n0)] = v;
+    if (row < M && col < N) ws[(row - m0) * tn + (col - n0)] = v;
   }
 };
 

@@ -228,12 +228,14 @@ def test_batchnorm_diag(ops, dev, shape):
 
 # ---- size-independent properties at the benchmark's sizes ---------------------
 
-def test_large_inverse_against_float64_library_inverse(ops, dev):
+def test_large_inverse_at_benchmark_sizes(ops, dev):
     """4608 (largest ResNet-50 factor, batch 32) and 9217 (AlexNet fc6, batch
-    256, rank-deficient before damping): compared on the device with
-    torch.linalg.inv in float64 (a library routine, not the oracle's formula),
-    plus the residual X X^-1 - I, which for a float32 result scales with the
-    condition number (about 7e2 for the second case)."""
+    256, rank-deficient before damping).  The error of the float32 result Y is
+    measured in float64 on the device through one Newton step,
+    Y_true = Y + Y (I - X Y) + O(|I - X Y|^2), and for 4608 also against
+    torch.linalg.inv in float64 (a library routine).  The residual X Y - I of a
+    float32 inverse scales with the condition number (about 7e2 in the second
+    case), so it gets a looser bound."""
     for n, L in [(4608, 1568), (9217, 256)]:
         g = torch.Generator(device='cpu').manual_seed(n)
         x = torch.randn(L, n, generator=g).to(dev)
@@ -243,14 +245,19 @@ def test_large_inverse_against_float64_library_inverse(ops, dev):
         assert info.cpu().tolist() == [0]
         Xd = X.double()
         Xd.diagonal().add_(damp)
-        ref = torch.linalg.inv(Xd)
-        err = ((outs[0].double() - ref).norm() / ref.norm()).item()
-        res = (Xd @ outs[0].double() - torch.eye(n, device=dev, dtype=D)).norm().item() / n ** 0.5
+        Y = outs[0].double()
+        R = torch.eye(n, device=dev, dtype=D) - Xd @ Y
+        err = ((Y @ R).norm() / Y.norm()).item()
+        res = R.norm().item() / n ** 0.5
         print('n=%d rel err %.2e residual %.2e' % (n, err, res))
-        assert err < TOL, (n, err)
         assert res < 1e-3, (n, res)
+        assert err < TOL, (n, err)
+        if n == 4608:
+            ref = torch.linalg.inv(Xd)
+            assert ((Y - ref).norm() / ref.norm()).item() < TOL
+            del ref
         assert torch.equal(outs[0], outs[0].t())
-        del Xd, ref
+        del Xd, Y, R
 
 
 def test_factor_linearity_at_full_size(ops, dev):
