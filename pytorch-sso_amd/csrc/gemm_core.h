@@ -55,6 +55,14 @@ __host__ __device__ inline int tiles128(int d) { return (d + BM - 1) / BM; }
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
+// LDS pointers carry their address space explicitly: through a generic pointer
+// the compiler emits FLAT loads/stores, whose completion is counted together
+// with global loads, and the wait before the MFMAs would then also wait for the
+// prefetch of the next chunk.
+typedef __attribute__((address_space(3))) float lds_f;
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4f lds_f4;
+
 // ---------------------------------------------------------------------------
 // global -> register -> LDS staging of one operand chunk (KC x ROWS elements
 // swept by NT threads)
@@ -67,6 +75,8 @@ struct Stager {
   static constexpr int MSTEP = NT / KC;                 // MK: m rows per sweep
   typename OP::MS ms[NM];
   float regs[CNT];
+  unsigned okbits;     // element i is inside the operand and the k range
+  unsigned onebits;    // element i is the constant 1
 
   __device__ __forceinline__ void init(const OP& op, int m0) {
     const int t = threadIdx.x;
@@ -76,40 +86,60 @@ struct Stager {
 #pragma unroll
       for (int i = 0; i < NM; ++i) ms[i] = op.mstate(m0 + (t / KC) + MSTEP * i);
     }
+    okbits = 0;
+    onebits = 0;
   }
 
+  // Issue the global loads of one chunk.  The loaded values are not touched
+  // here (masking happens in commit), so nothing waits on memory yet.
   __device__ __forceinline__ void fetch(const OP& op, int k0, int kend) {
     const int t = threadIdx.x;
+    unsigned okb = 0, oneb = 0;
     if (OP::layout == KM) {
 #pragma unroll
       for (int i = 0; i < CNT; ++i) {
         const int k = k0 + (t / ROWS) + KSTEP * i;
-        regs[i] = (k < kend) ? op.load(ms[0], op.kstate(k)) : 0.f;
+        const bool kin = k < kend;
+        bool ok;
+        const float* a = op.addr(ms[0], op.kstate(kin ? k : k0), ok);   // k0 is in range
+        regs[i] = *a;
+        okb |= (unsigned)(ok && kin) << i;
+        oneb |= (unsigned)(op.is_one(ms[0]) && kin) << i;
       }
     } else {
       const int k = k0 + (t % KC);
       const bool kin = k < kend;
       const typename OP::KS ks = op.kstate(kin ? k : k0);
 #pragma unroll
-      for (int i = 0; i < CNT; ++i) regs[i] = kin ? op.load(ms[i], ks) : 0.f;
+      for (int i = 0; i < CNT; ++i) {
+        bool ok;
+        const float* a = op.addr(ms[i], ks, ok);
+        regs[i] = *a;
+        okb |= (unsigned)(ok && kin) << i;
+        oneb |= (unsigned)(op.is_one(ms[i]) && kin) << i;
+      }
     }
+    okbits = okb;
+    onebits = oneb;
   }
 
-  __device__ __forceinline__ void commit(float* tile) const {
+  __device__ __forceinline__ void commit(lds_f* tile) const {
     const int t = threadIdx.x;
-    if (OP::layout == KM) {
 #pragma unroll
-      for (int i = 0; i < CNT; ++i) tile[((t / ROWS) + KSTEP * i) * ROWS + (t % ROWS)] = regs[i];
-    } else {
-#pragma unroll
-      for (int i = 0; i < CNT; ++i) tile[((t / KC) + MSTEP * i) * LDS_MK + (t % KC)] = regs[i];
+    for (int i = 0; i < CNT; ++i) {
+      float v = ((okbits >> i) & 1u) ? regs[i] : 0.f;
+      v = ((onebits >> i) & 1u) ? 1.f : v;
+      if (OP::layout == KM)
+        tile[((t / ROWS) + KSTEP * i) * ROWS + (t % ROWS)] = v;
+      else
+        tile[((t / KC) + MSTEP * i) * LDS_MK + (t % KC)] = v;
     }
   }
 };
 
 // fragments of one operand for the 8 MFMA steps of a chunk: f[sub][4j+s]
 template <int LAYOUT, int ROWS>
-__device__ __forceinline__ void load_frags(const float* tile, int base, int r, int h,
+__device__ __forceinline__ void load_frags(const lds_f* tile, int base, int r, int h,
                                            float (&f)[2][8]) {
   if (LAYOUT == KM) {
 #pragma unroll
@@ -124,8 +154,7 @@ __device__ __forceinline__ void load_frags(const float* tile, int base, int r, i
     for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const float4 v =
-            *reinterpret_cast<const float4*>(&tile[(base + 32 * sub + r) * LDS_MK + 8 * j + 4 * h]);
+        const v4f v = *(const lds_f4*)(&tile[(base + 32 * sub + r) * LDS_MK + 8 * j + 4 * h]);
         f[sub][4 * j + 0] = v.x;
         f[sub][4 * j + 1] = v.y;
         f[sub][4 * j + 2] = v.z;
@@ -166,15 +195,15 @@ __device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0
   sp.init(P, m0);
   if (!same) sq.init(Q, n0);
 
-  float* tp[2] = {smem, smem + C::P_FLOATS + C::Q_FLOATS};
-  float* tq[2] = {smem + C::P_FLOATS, smem + 2 * C::P_FLOATS + C::Q_FLOATS};
+  lds_f* const sm = (lds_f*)smem;
+  constexpr int STAGE = C::P_FLOATS + C::Q_FLOATS;
 
   const int nchunks = (kend - kbeg + KC - 1) / KC;
   if (nchunks > 0) {
     sp.fetch(P, kbeg, kend);
     if (!same) sq.fetch(Q, kbeg, kend);
-    sp.commit(tp[0]);
-    if (!same) sq.commit(tq[0]);
+    sp.commit(sm);
+    if (!same) sq.commit(sm + C::P_FLOATS);
   }
   __syncthreads();
 
@@ -186,11 +215,13 @@ __device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0
       if (!same) sq.fetch(Q, kbeg + (c + 1) * KC, kend);
     }
     float fa[2][8], fb[2][8];
-    load_frags<OPP::layout, C::TM>(tp[cur], wm, r, h, fa);
+    const lds_f* const tpc = sm + cur * STAGE;
+    const lds_f* const tqc = tpc + C::P_FLOATS;
+    load_frags<OPP::layout, C::TM>(tpc, wm, r, h, fa);
     if (same)
-      load_frags<OPP::layout, C::TM>(tp[cur], wn, r, h, fb);
+      load_frags<OPP::layout, C::TM>(tpc, wn, r, h, fb);
     else
-      load_frags<OPQ::layout, C::TN>(tq[cur], wn, r, h, fb);
+      load_frags<OPQ::layout, C::TN>(tqc, wn, r, h, fb);
 #pragma unroll
     for (int s = 0; s < 8; ++s)
 #pragma unroll
@@ -199,8 +230,9 @@ __device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0
         for (int b = 0; b < 2; ++b)
           acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a][s], fb[b][s], acc[a][b], 0, 0, 0);
     if (more) {
-      sp.commit(tp[cur ^ 1]);
-      if (!same) sq.commit(tq[cur ^ 1]);
+      lds_f* const tpn = sm + (cur ^ 1) * STAGE;
+      sp.commit(tpn);
+      if (!same) sq.commit(tpn + C::P_FLOATS);
     }
     __syncthreads();
   }

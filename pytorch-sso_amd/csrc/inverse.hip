@@ -108,7 +108,7 @@ __device__ __forceinline__ float bcast(float v, int lane) {
 
 // One wave factors the 32x32 block at (c0, c0) of S in registers (lane j holds
 // column j), inverts the factor, and writes U_qq to S and Y_qq to Yb.
-__device__ __forceinline__ void chol_inv_32(float* S, float* Yb, int c0, int row_base, int* info) {
+__device__ __forceinline__ void chol_inv_32(lds_f* S, lds_f* Yb, int c0, int row_base, int* info) {
   const int lane = threadIdx.x & 63;
   const int j = lane & 31;
   float a[32];
@@ -154,15 +154,15 @@ __device__ __forceinline__ void chol_inv_32(float* S, float* Yb, int c0, int row
 // One wave: acc(32x32) = sum_{k<K} A(k, i) * B(k, j) with operands in LDS,
 //   A(k, i) = a[k*a_ks + i*a_is],  B(k, j) = b[k*b_ks + j*b_js]   (K even).
 // Result element t of lane (r, h): row 8*(t/4) + 4h + t%4, column r.
-__device__ __forceinline__ v16f lds_mma32(const float* a, int a_ks, int a_is, const float* b,
+__device__ __forceinline__ v16f lds_mma32(const lds_f* a, int a_ks, int a_is, const lds_f* b,
                                           int b_ks, int b_js, int K) {
   const int lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
   v16f acc;
 #pragma unroll
   for (int t = 0; t < 16; ++t) acc[t] = 0.f;
-  const float* pa = a + h * a_ks + r * a_is;
-  const float* pb = b + h * b_ks + r * b_js;
+  const lds_f* pa = a + h * a_ks + r * a_is;
+  const lds_f* pb = b + h * b_ks + r * b_js;
 #pragma unroll 4
   for (int k = 0; k < K; k += 2) {
     acc = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[k * a_ks], pb[k * b_ks], acc, 0, 0, 0);
@@ -171,13 +171,13 @@ __device__ __forceinline__ v16f lds_mma32(const float* a, int a_ks, int a_is, co
 }
 
 // store / subtract a 32x32 result block at c[row*ld + col]
-__device__ __forceinline__ void lds_put32(float* c, int ld, const v16f& acc, float scale) {
+__device__ __forceinline__ void lds_put32(lds_f* c, int ld, const v16f& acc, float scale) {
   const int lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
 #pragma unroll
   for (int t = 0; t < 16; ++t) c[(8 * (t >> 2) + 4 * h + (t & 3)) * ld + r] = scale * acc[t];
 }
-__device__ __forceinline__ void lds_sub32(float* c, int ld, const v16f& acc) {
+__device__ __forceinline__ void lds_sub32(lds_f* c, int ld, const v16f& acc) {
   const int lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
 #pragma unroll
@@ -187,7 +187,7 @@ __device__ __forceinline__ void lds_sub32(float* c, int ld, const v16f& acc) {
 // In-LDS off-diagonal inverse block:  Y12 = -Y11 * (U12 * Y22) for the pair
 // X1 = [s1, s1+b), X2 = [s1+b, s1+2b), b = 32 or 64; W is a b x b scratch.
 // 32x32 result blocks are dealt round-robin to the 4 waves.
-__device__ __forceinline__ void tri_pair(const float* S, float* Yb, float* Wt, int s1, int b,
+__device__ __forceinline__ void tri_pair(const lds_f* S, lds_f* Yb, lds_f* Wt, int s1, int b,
                                          int wave_first, int wave_count) {
   const int s2 = s1 + b;
   const int wave = (int)(threadIdx.x >> 6) - wave_first;
@@ -212,9 +212,9 @@ __device__ __forceinline__ void tri_pair(const float* S, float* Yb, float* Wt, i
 
 __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, int p, int* info) {
   extern __shared__ __attribute__((aligned(16))) float dsm[];
-  float* S = dsm;
-  float* Yb = dsm + DB * DLD;
-  float* Wt = dsm + 2 * DB * DLD;
+  lds_f* const S = (lds_f*)dsm;
+  lds_f* const Yb = S + DB * DLD;
+  lds_f* const Wt = S + 2 * DB * DLD;
   const MatDesc m = table[blockIdx.x];
   const int n = m.n;
   const int r0 = p * DB;

@@ -10,28 +10,42 @@ namespace kfac {
 //   extra == 1 : the constant 1 (bias augmentation of a Linear input)
 //   extra == 2 : taken from vec[k] (bias gradient appended to a weight gradient)
 // ---------------------------------------------------------------------------
+// Operand functor contract used by the staging code of the tile engine:
+//   MS mstate(m), KS kstate(k)      per-index precomputation
+//   const float* addr(ms, ks, ok)   ALWAYS a readable address; ok = false when the
+//                                   element lies outside the operand (value -> 0)
+//   bool is_one(ms)                 the element is the constant 1 (bias augmentation)
+// Nothing here branches, and the value is only looked at when the chunk is
+// written to LDS, so the global loads of the next chunk stay in flight while
+// the MFMAs of the current one run.
+
+// Dense row-major matrix read as P(k, m) = p[k*ld + m]  (m contiguous).
+// Optional last column (index M-1) that is not in memory:
+//   extra == 1 : the constant 1 (bias augmentation of a Linear input)
+//   extra == 2 : taken from vec[k] (bias gradient appended to a weight gradient)
 struct DenseKM {
   static constexpr int layout = KM;
   const float* p;
   const float* vec;
   int ld, M, extra;
-  struct MS { int off; int kind; };   // kind: 0 outside, 1 memory, 2 ones, 3 vec
-  struct KS { int off; int k; };
+  struct MS { const float* base; int stride; bool valid; bool one; };
+  struct KS { int k; };
   __device__ __forceinline__ MS mstate(int m) const {
     MS s;
-    s.off = m;
-    if (m >= M) s.kind = 0;
-    else if (extra && m == M - 1) s.kind = extra + 1;
-    else s.kind = 1;
+    s.base = p; s.stride = 0; s.valid = false; s.one = false;
+    if (m < M) {
+      if (extra == 1 && m == M - 1) { s.one = true; }
+      else if (extra == 2 && m == M - 1) { s.base = vec; s.stride = 1; s.valid = true; }
+      else { s.base = p + m; s.stride = ld; s.valid = true; }
+    }
     return s;
   }
-  __device__ __forceinline__ KS kstate(int k) const { return KS{k * ld, k}; }
-  __device__ __forceinline__ float load(const MS& m, const KS& k) const {
-    if (m.kind == 1) return p[k.off + m.off];
-    if (m.kind == 2) return 1.f;
-    if (m.kind == 3) return vec[k.k];
-    return 0.f;
+  __device__ __forceinline__ KS kstate(int k) const { return KS{k}; }
+  __device__ __forceinline__ const float* addr(const MS& m, const KS& k, bool& ok) const {
+    ok = m.valid;
+    return m.base + (unsigned)(k.k * m.stride);
   }
+  __device__ __forceinline__ bool is_one(const MS& m) const { return extra == 1 && m.one; }
 };
 
 // Dense row-major matrix read as P(k, m) = p[m*ld + k]  (k contiguous).
@@ -39,13 +53,17 @@ struct DenseMK {
   static constexpr int layout = MK;
   const float* p;
   int ld, M;
-  struct MS { int off; };             // -1 outside
-  struct KS { int off; };
-  __device__ __forceinline__ MS mstate(int m) const { return MS{m < M ? m * ld : -1}; }
-  __device__ __forceinline__ KS kstate(int k) const { return KS{k}; }
-  __device__ __forceinline__ float load(const MS& m, const KS& k) const {
-    return m.off >= 0 ? p[m.off + k.off] : 0.f;
+  struct MS { const float* row; bool valid; };
+  struct KS { int k; };
+  __device__ __forceinline__ MS mstate(int m) const {
+    return MS{m < M ? p + (size_t)m * ld : p, m < M};
   }
+  __device__ __forceinline__ KS kstate(int k) const { return KS{k}; }
+  __device__ __forceinline__ const float* addr(const MS& m, const KS& k, bool& ok) const {
+    ok = m.valid;
+    return m.row + (m.valid ? (unsigned)k.k : 0u);
+  }
+  __device__ __forceinline__ bool is_one(const MS&) const { return false; }
 };
 
 // Output gradient of a Conv2d, g[n][c][hw], read as P(k=(n,pos), m=c).
@@ -53,16 +71,20 @@ struct ConvG {
   static constexpr int layout = MK;
   const float* p;
   int C, HW;
-  struct MS { int off; };
-  struct KS { int off; };
-  __device__ __forceinline__ MS mstate(int m) const { return MS{m < C ? m * HW : -1}; }
+  struct MS { const float* chan; bool valid; };
+  struct KS { unsigned off; };
+  __device__ __forceinline__ MS mstate(int m) const {
+    return MS{m < C ? p + (size_t)m * HW : p, m < C};
+  }
   __device__ __forceinline__ KS kstate(int k) const {
     const int n = k / HW;
-    return KS{n * C * HW + (k - n * HW)};
+    return KS{(unsigned)(n * C * HW + (k - n * HW))};
   }
-  __device__ __forceinline__ float load(const MS& m, const KS& k) const {
-    return m.off >= 0 ? p[m.off + k.off] : 0.f;
+  __device__ __forceinline__ const float* addr(const MS& m, const KS& k, bool& ok) const {
+    ok = m.valid;
+    return m.chan + (m.valid ? k.off : 0u);
   }
+  __device__ __forceinline__ bool is_one(const MS&) const { return false; }
 };
 
 // Implicit im2col of a Conv2d input x[n][c][H][W]:
@@ -72,12 +94,15 @@ struct ConvA {
   static constexpr int layout = MK;
   const float* p;
   int C, H, W, KH, KW, SH, SW, PH, PW, DH, DW, OH, OW, M, ones;
-  struct MS { int off; int dy; int dx; };   // dy == -2^30: outside; dy == -2^29: ones row
+  // dy = -2^20 marks a row outside the operand or the row of ones: every
+  // bounds test then fails
+  struct MS { int off; int dy; int dx; bool one; };
   struct KS { int off; int y0; int x0; };
   __device__ __forceinline__ MS mstate(int m) const {
     MS s;
-    if (m >= M) { s.off = 0; s.dy = -(1 << 30); s.dx = 0; return s; }
-    if (ones && m == M - 1) { s.off = 0; s.dy = -(1 << 29); s.dx = 0; return s; }
+    s.one = false;
+    if (m >= M) { s.off = 0; s.dy = -(1 << 20); s.dx = 0; return s; }
+    if (ones && m == M - 1) { s.off = 0; s.dy = -(1 << 20); s.dx = 0; s.one = true; return s; }
     const int c = m / (KH * KW);
     const int rem = m - c * KH * KW;
     const int kh = rem / KW;
@@ -98,14 +123,13 @@ struct ConvA {
     s.off = n * C * H * W + s.y0 * W + s.x0;
     return s;
   }
-  __device__ __forceinline__ float load(const MS& m, const KS& k) const {
-    if (m.dy == -(1 << 30)) return 0.f;
-    if (m.dy == -(1 << 29)) return 1.f;
+  __device__ __forceinline__ const float* addr(const MS& m, const KS& k, bool& ok) const {
     const int y = k.y0 + m.dy;
     const int x = k.x0 + m.dx;
-    if ((unsigned)y < (unsigned)H && (unsigned)x < (unsigned)W) return p[k.off + m.off];
-    return 0.f;
+    ok = (unsigned)y < (unsigned)H && (unsigned)x < (unsigned)W;
+    return p + (ok ? (unsigned)(k.off + m.off) : 0u);
   }
+  __device__ __forceinline__ bool is_one(const MS& m) const { return ones && m.one; }
 };
 
 // ---------------------------------------------------------------------------
