@@ -3,7 +3,21 @@
 #include "common.h"
 #include "operands.h"
 
+#include <mutex>
+#include <set>
+
 namespace kfac {
+
+bool enable_large_lds(const void* kernel, int bytes) {
+  static std::mutex mu;
+  static std::set<const void*> done;
+  std::lock_guard<std::mutex> lock(mu);
+  if (done.count(kernel)) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
+    return false;
+  done.insert(kernel);
+  return true;
+}
 
 // Tile configuration and k-split of a symmetric d x d product reduced over K:
 // 64-wide single-wave tiles for small factors (a 128-wide tile would be mostly
@@ -15,7 +29,7 @@ struct SyrkPlan {
   int T;        // tiles per side
   int ntiles;   // upper-triangular tiles
   int splits;
-  int cps;      // 16-deep chunks per split
+  int cps;      // chunks (of the configuration's KC) per split
 };
 
 static SyrkPlan plan_syrk(int d, long K) {
@@ -24,11 +38,13 @@ static SyrkPlan plan_syrk(int d, long K) {
   p.ts = 64 * p.w;
   p.T = cdiv(d, p.ts);
   p.ntiles = p.T * (p.T + 1) / 2;
-  const long nchunks = (K + KC - 1) / KC;
+  const int kc = p.w == 1 ? Cfg<1, 1>::KC : Cfg<2, 2>::KC;
+  const long nchunks = (K + kc - 1) / kc;
   const long target = 2048 / (p.w * p.w);
   long splits = target / p.ntiles;
   if (splits < 1) splits = 1;
-  const long max_splits = nchunks / 8 > 0 ? nchunks / 8 : 1;
+  const long min_chunks = 128 / kc;      // each split at least 128 deep
+  const long max_splits = nchunks / min_chunks > 0 ? nchunks / min_chunks : 1;
   if (splits > max_splits) splits = max_splits;
   long cps = (nchunks + splits - 1) / splits;
   if (cps < 1) cps = 1;
@@ -40,12 +56,13 @@ static SyrkPlan plan_syrk(int d, long K) {
 }
 
 template <class OP, int W>
-__global__ __launch_bounds__(64 * W * W) void syrk_kernel(OP op, int d, int K, int T, int ntiles,
+__global__ __launch_bounds__(64 * W * W, W == 2 ? 2 : 1) void syrk_kernel(OP op, int d, int K, int T, int ntiles,
                                                           int splits, int chunks_per_split,
                                                           float* C, float alpha, float beta,
                                                           float* ws) {
   constexpr int TS = 64 * W;
-  __shared__ __attribute__((aligned(16))) float smem[Cfg<W, W>::SMEM_FLOATS];
+  constexpr int KC = Cfg<W, W>::KC;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
   const int tile = blockIdx.x;
   const int split = blockIdx.y;
   int bi, bj;
@@ -126,8 +143,10 @@ template <class OP, int W>
 static void launch_syrk_cfg(const OP& op, const SyrkPlan& p, int d, int64_t K, float alpha,
                             float beta, float* C, void* workspace, hipStream_t stream) {
   constexpr int TS = 64 * W;
-  hipLaunchKernelGGL((syrk_kernel<OP, W>), dim3(p.ntiles, p.splits), dim3(64 * W * W), 0, stream,
-                     op, d, (int)K, p.T, p.ntiles, p.splits, p.cps, C, alpha, beta,
+  constexpr int lds_bytes = Cfg<W, W>::SMEM_FLOATS * (int)sizeof(float);
+  if (!enable_large_lds((const void*)syrk_kernel<OP, W>, lds_bytes)) return;
+  hipLaunchKernelGGL((syrk_kernel<OP, W>), dim3(p.ntiles, p.splits), dim3(64 * W * W), lds_bytes,
+                     stream, op, d, (int)K, p.T, p.ntiles, p.splits, p.cps, C, alpha, beta,
                      (float*)workspace);
   if (p.splits > 1) {
     hipLaunchKernelGGL((syrk_reduce_kernel<TS>), dim3(p.ntiles, TS * (TS / 64)), dim3(256), 0,
@@ -181,6 +200,7 @@ int kfac_factor_conv_a(const float* x, int n, int c, int H, int W, int kh, int k
   if (!x || !C || n <= 0 || c <= 0 || H <= 0 || W <= 0 || kh <= 0 || kw <= 0 || sh <= 0 ||
       sw <= 0 || ph < 0 || pw < 0 || dh <= 0 || dw <= 0)
     return KFAC_ERR_ARG;
+  if (H >= 16384 || W >= 16384 || kh * dh >= 16384 || kw * dw >= 16384) return KFAC_ERR_ARG;
   if ((int64_t)n * c * H * W >= (int64_t)1 << 31) return KFAC_ERR_ARG;
   const int OH = (H + 2 * ph - dh * (kh - 1) - 1) / sh + 1;
   const int OW = (W + 2 * pw - dw * (kw - 1) - 1) / sw + 1;

@@ -17,9 +17,9 @@
 //   float load(MS, KS): the element, 0 outside the operand's own bounds
 // The layout only chooses how the 256 threads sweep the 16x128 chunk so that
 // global loads coalesce, and how the chunk sits in LDS:
-//   KM chunk -> lds[k][m]   (row length 128), MFMA lanes read ds_read_b32
-//   MK chunk -> lds[m][k+4] (row length 20),  MFMA lanes read ds_read_b128
-// Within a 16-deep chunk the k values are consumed in the order
+//   KM chunk -> lds[k][m]   (row length = tile width), MFMA lanes read ds_read_b32
+//   MK chunk -> lds[m][KC+4],                           MFMA lanes read ds_read_b128
+// Within a 16-deep slice of a chunk the k values are consumed in the order
 //   step (j,s), lane half h  ->  k = 8j + 4h + s
 // for both operands, which is a permutation of the reduction index and so does
 // not change the product.
@@ -30,24 +30,27 @@ namespace kfac {
 
 constexpr int BM = 128;          // tile rows of the default (2x2 waves) configuration
 constexpr int BN = 128;          // tile cols of the default configuration
-constexpr int KC = 16;           // reduction depth per LDS stage
 constexpr int NTHREADS = 256;    // threads of the default configuration
-constexpr int LDS_MK = KC + 4;   // padded row of an MK chunk (bank-conflict free b128)
 
 // A configuration is WM x WN waves, each owning a 64x64 sub-tile:
 //   tile = (64*WM) x (64*WN), threads = 64*WM*WN.
 // 2x2 is the default; 1x1 (one wave, 64x64) serves small factors, where a
 // 128-wide tile would be mostly padding.
+// KC is the reduction depth per LDS stage: 32 for the 2x2 configuration (the
+// 64 MFMAs per wave and stage then cover the latency of the next stage's
+// global loads), 16 for 1x1 (one wave stages the whole chunk by itself).
 template <int WM, int WN>
 struct Cfg {
   static constexpr int TM = 64 * WM;
   static constexpr int TN = 64 * WN;
   static constexpr int NT = 64 * WM * WN;
+  static constexpr int KC = (WM * WN >= 4) ? 32 : 16;
+  static constexpr int LDS_MK = KC + 4;          // padded row of an MK chunk (conflict-free b128)
   static constexpr int P_FLOATS = LDS_MK * TM;   // >= KC*TM and TM*LDS_MK
   static constexpr int Q_FLOATS = LDS_MK * TN;
   static constexpr int SMEM_FLOATS = 2 * (P_FLOATS + Q_FLOATS);
 };
-constexpr int SMEM_FLOATS = Cfg<2, 2>::SMEM_FLOATS;   // 40 KiB
+constexpr int SMEM_FLOATS = Cfg<2, 2>::SMEM_FLOATS;   // 72 KiB
 
 enum { KM = 0, MK = 1 };
 
@@ -67,8 +70,9 @@ typedef __attribute__((address_space(3))) v4f lds_f4;
 // global -> register -> LDS staging of one operand chunk (KC x ROWS elements
 // swept by NT threads)
 // ---------------------------------------------------------------------------
-template <class OP, int ROWS, int NT>
+template <class OP, int ROWS, int NT, int KC>
 struct Stager {
+  static constexpr int LDS_MK = KC + 4;
   static constexpr int CNT = KC * ROWS / NT;            // elements per thread
   static constexpr int NM = (OP::layout == KM) ? 1 : CNT;
   static constexpr int KSTEP = NT / ROWS;               // KM: k rows per sweep
@@ -137,9 +141,10 @@ struct Stager {
   }
 };
 
-// fragments of one operand for the 8 MFMA steps of a chunk: f[sub][4j+s]
-template <int LAYOUT, int ROWS>
-__device__ __forceinline__ void load_frags(const lds_f* tile, int base, int r, int h,
+// fragments of one operand for the 8 MFMA steps of a 16-deep slice starting at
+// k = kofs of the staged chunk: f[sub][4j+s]
+template <int LAYOUT, int ROWS, int LDS_MK>
+__device__ __forceinline__ void load_frags(const lds_f* tile, int base, int r, int h, int kofs,
                                            float (&f)[2][8]) {
   if (LAYOUT == KM) {
 #pragma unroll
@@ -148,13 +153,13 @@ __device__ __forceinline__ void load_frags(const lds_f* tile, int base, int r, i
       for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int s = 0; s < 4; ++s)
-          f[sub][4 * j + s] = tile[(8 * j + 4 * h + s) * ROWS + base + 32 * sub + r];
+          f[sub][4 * j + s] = tile[(kofs + 8 * j + 4 * h + s) * ROWS + base + 32 * sub + r];
   } else {
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const v4f v = *(const lds_f4*)(&tile[(base + 32 * sub + r) * LDS_MK + 8 * j + 4 * h]);
+        const v4f v = *(const lds_f4*)(&tile[(base + 32 * sub + r) * LDS_MK + kofs + 8 * j + 4 * h]);
         f[sub][4 * j + 0] = v.x;
         f[sub][4 * j + 1] = v.y;
         f[sub][4 * j + 2] = v.z;
@@ -190,8 +195,9 @@ __device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
 
-  Stager<OPP, C::TM, C::NT> sp;
-  Stager<OPQ, C::TN, C::NT> sq;
+  constexpr int KC = C::KC;
+  Stager<OPP, C::TM, C::NT, C::KC> sp;
+  Stager<OPQ, C::TN, C::NT, C::KC> sq;
   sp.init(P, m0);
   if (!same) sq.init(Q, n0);
 
@@ -214,21 +220,24 @@ __device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0
       sp.fetch(P, kbeg + (c + 1) * KC, kend);
       if (!same) sq.fetch(Q, kbeg + (c + 1) * KC, kend);
     }
-    float fa[2][8], fb[2][8];
     const lds_f* const tpc = sm + cur * STAGE;
     const lds_f* const tqc = tpc + C::P_FLOATS;
-    load_frags<OPP::layout, C::TM>(tpc, wm, r, h, fa);
-    if (same)
-      load_frags<OPP::layout, C::TM>(tpc, wn, r, h, fb);
-    else
-      load_frags<OPQ::layout, C::TN>(tqc, wn, r, h, fb);
 #pragma unroll
-    for (int s = 0; s < 8; ++s)
+    for (int kofs = 0; kofs < KC; kofs += 16) {
+      float fa[2][8], fb[2][8];
+      load_frags<OPP::layout, C::TM, C::LDS_MK>(tpc, wm, r, h, kofs, fa);
+      if (same)
+        load_frags<OPP::layout, C::TM, C::LDS_MK>(tpc, wn, r, h, kofs, fb);
+      else
+        load_frags<OPQ::layout, C::TN, C::LDS_MK>(tqc, wn, r, h, kofs, fb);
 #pragma unroll
-      for (int a = 0; a < 2; ++a)
+      for (int s = 0; s < 8; ++s)
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a][s], fb[b][s], acc[a][b], 0, 0, 0);
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+          for (int b = 0; b < 2; ++b)
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a][s], fb[b][s], acc[a][b], 0, 0, 0);
+    }
     if (more) {
       lds_f* const tpn = sm + (cur ^ 1) * STAGE;
       sp.commit(tpn);

@@ -102,45 +102,65 @@ constexpr int DLD = DB + 1;      // LDS leading dimension
 constexpr int WLD = 65;
 constexpr int DIAG_SMEM_BYTES = (2 * DB * DLD + 64 * WLD) * (int)sizeof(float);
 
-__device__ __forceinline__ float bcast(float v, int lane) {
-  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
-}
-
-// One wave factors the 32x32 block at (c0, c0) of S in registers (lane j holds
-// column j), inverts the factor, and writes U_qq to S and Y_qq to Yb.
-__device__ __forceinline__ void chol_inv_32(lds_f* S, lds_f* Yb, int c0, int row_base, int* info) {
+// One wave factors the 32x32 block at (c0, c0) of S (lane j holds column j in
+// registers), inverts the factor, and writes U_qq to S and Y_qq to Yb.
+// Each step needs one row of the block in every lane: the lanes write their
+// element of the row to a 32-float LDS buffer and read the whole row back with
+// broadcast ds_read_b128 (no cross-lane register traffic).  `scr` is 16-byte
+// aligned scratch of at least 64 + 32*32 floats.
+__device__ __forceinline__ void chol_inv_32(lds_f* S, lds_f* Yb, lds_f* scr, int c0, int row_base,
+                                            int* info) {
   const int lane = threadIdx.x & 63;
   const int j = lane & 31;
+  lds_f* rowbuf = scr;           // 32 floats
+  lds_f* ubuf = scr + 64;        // 32 x 32, row-major, rows 16-byte aligned
   float a[32];
 #pragma unroll
   for (int i = 0; i < 32; ++i) a[i] = S[(c0 + i) * DLD + c0 + j];
   int bad = 0;
 #pragma unroll
   for (int c = 0; c < 32; ++c) {
-    const float piv = bcast(a[c], c);
+    rowbuf[j] = a[c];            // A[c][j] after the updates of the earlier steps
+    float row[32];
+#pragma unroll
+    for (int g = c / 4; g < 8; ++g) {
+      const v4f v = *(const lds_f4*)(rowbuf + 4 * g);
+      row[4 * g + 0] = v.x;
+      row[4 * g + 1] = v.y;
+      row[4 * g + 2] = v.z;
+      row[4 * g + 3] = v.w;
+    }
+    const float piv = row[c];
     if (!(piv > 0.f) && bad == 0) bad = row_base + c0 + c + 1;
     const float d = sqrtf(piv);
-    const float rd = 1.f / d;
-    float ucj = (j >= c) ? a[c] * rd : 0.f;
-    if (j == c) ucj = d;
-    a[c] = ucj;
+    const float rd = __builtin_amdgcn_rcpf(d);
+    const float f = a[c] * (rd * rd);
 #pragma unroll
-    for (int i = c + 1; i < 32; ++i) {
-      const float uci = bcast(ucj, i);
-      a[i] -= uci * ucj;
-    }
+    for (int i = c + 1; i < 32; ++i) a[i] = fmaf(-row[i], f, a[i]);   // A[i][j] -= U[c][i] U[c][j]
+    a[c] = (j > c) ? a[c] * rd : (j == c ? d : 0.f);
   }
   if (bad != 0 && lane == 0) {
     if (*info == 0) *info = bad;
   }
-  // inverse by back substitution, column j of Y in lane j
+#pragma unroll
+  for (int i = 0; i < 32; ++i) ubuf[i * 32 + j] = (i <= j) ? a[i] : 0.f;
+  // Y = U^-1 by back substitution: column j of Y in lane j, row i of U broadcast
   float y[32];
 #pragma unroll
   for (int i = 31; i >= 0; --i) {
+    float row[32];
+#pragma unroll
+    for (int g = i / 4; g < 8; ++g) {
+      const v4f v = *(const lds_f4*)(ubuf + i * 32 + 4 * g);
+      row[4 * g + 0] = v.x;
+      row[4 * g + 1] = v.y;
+      row[4 * g + 2] = v.z;
+      row[4 * g + 3] = v.w;
+    }
     float s = (j == i) ? 1.f : 0.f;
 #pragma unroll
-    for (int k = i + 1; k < 32; ++k) s -= bcast(a[i], k) * y[k];
-    y[i] = s / bcast(a[i], i);
+    for (int k = i + 1; k < 32; ++k) s = fmaf(-row[k], y[k], s);
+    y[i] = s * __builtin_amdgcn_rcpf(row[i]);
   }
   if (lane < 32) {
 #pragma unroll
@@ -222,24 +242,34 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
   const int t = threadIdx.x;
   const int wave = t >> 6;
 
-  // load the upper triangle; pad with the identity up to 128
-  for (int e = t; e < DB * DB; e += 256) {
-    const int i = e >> 7, j = e & 127;
-    float v = 0.f;
-    if (i < nb && j < nb) {
-      if (j >= i) v = m.U[(size_t)(r0 + i) * n + r0 + j];
-    } else if (i == j) {
-      v = 1.f;
+  // load the upper triangle; pad with the identity up to 128.  16 loads are
+  // issued before the first is used, so the block costs 4 memory round trips
+  // instead of 64.
+  for (int e0 = 0; e0 < DB * DB; e0 += 256 * 16) {
+    float v[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int e = e0 + u * 256 + t;
+      const int i = e >> 7, j = e & 127;
+      const bool in = i < nb && j < nb && j >= i;
+      v[u] = m.U[in ? (size_t)(r0 + i) * n + r0 + j : (size_t)r0 * n + r0];
     }
-    S[i * DLD + j] = v;
-    Yb[i * DLD + j] = 0.f;
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int e = e0 + u * 256 + t;
+      const int i = e >> 7, j = e & 127;
+      const bool in = i < nb && j < nb && j >= i;
+      const bool pad = (i >= nb || j >= nb) && i == j;
+      S[i * DLD + j] = in ? v[u] : (pad ? 1.f : 0.f);
+      Yb[i * DLD + j] = 0.f;
+    }
   }
   __syncthreads();
 
   const int nq = (nb + 31) / 32;
   for (int q = 0; q < nq; ++q) {
     const int c0 = 32 * q;
-    if (t < 64) chol_inv_32(S, Yb, c0, r0, info + m.out);
+    if (t < 64) chol_inv_32(S, Yb, Wt, c0, r0, info + m.out);
     __syncthreads();
     const int rest = nq - q - 1;     // 32-blocks to the right
     if (rest > 0) {
@@ -287,7 +317,7 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
 
 // row panel of the blocked Cholesky: U[p, j] = Ypp^T * A[p, j], j > p
 __global__ __launch_bounds__(NTHREADS) void potrf_panel_kernel(const MatDesc* table, int p) {
-  __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
+  extern __shared__ __attribute__((aligned(16))) float smem[];
   const MatDesc m = table[blockIdx.y];
   const int bj = p + 1 + blockIdx.x;
   if (bj >= m.T) return;
@@ -301,7 +331,7 @@ __global__ __launch_bounds__(NTHREADS) void potrf_panel_kernel(const MatDesc* ta
 
 // trailing update: A[i, j] -= U[p, i]^T U[p, j],  p < i <= j
 __global__ __launch_bounds__(NTHREADS) void potrf_trail_kernel(const MatDesc* table, int p) {
-  __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
+  extern __shared__ __attribute__((aligned(16))) float smem[];
   const MatDesc m = table[blockIdx.y];
   const int Tr = m.T - p - 1;
   if (Tr <= 0) return;
@@ -360,7 +390,7 @@ __device__ __forceinline__ MergeTile merge_tile(const MatDesc& m, int depth) {
 // first product:  W^T[j][i] = sum_{k <= j} Y22[k][j] * U12[i][k], stored at
 // Y[X2 rows][X1 cols] (the unused lower triangle of Y)
 __global__ __launch_bounds__(NTHREADS) void trtri_w_kernel(const MatDesc* table, int depth) {
-  __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
+  extern __shared__ __attribute__((aligned(16))) float smem[];
   const MatDesc m = table[blockIdx.y];
   const MergeTile t = merge_tile(m, depth);
   if (!t.valid) return;
@@ -373,7 +403,7 @@ __global__ __launch_bounds__(NTHREADS) void trtri_w_kernel(const MatDesc* table,
 
 // second product:  Y12[i][j] = - sum_{k >= i} Y11[i][k] * W^T[j][k]
 __global__ __launch_bounds__(NTHREADS) void trtri_y_kernel(const MatDesc* table, int depth) {
-  __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
+  extern __shared__ __attribute__((aligned(16))) float smem[];
   const MatDesc m = table[blockIdx.y];
   const MergeTile t = merge_tile(m, depth);
   if (!t.valid) return;
@@ -386,7 +416,7 @@ __global__ __launch_bounds__(NTHREADS) void trtri_y_kernel(const MatDesc* table,
 
 // dst = Y Y^T over the upper tiles (k >= the later block), mirrored
 __global__ __launch_bounds__(NTHREADS) void lauum_kernel(const MatDesc* table) {
-  __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
+  extern __shared__ __attribute__((aligned(16))) float smem[];
   const MatDesc m = table[blockIdx.y];
   const int ntiles = m.T * (m.T + 1) / 2;
   if ((int)blockIdx.x >= ntiles) return;
@@ -507,9 +537,8 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
     const int nb = active(p + 2);
     if (nb > 0) {
       const int Tr = Tmax - p - 1;
-      hipLaunchKernelGGL(potrf_panel_kernel, dim3(Tr, nb), dim3(NTHREADS), 0, stream, table, p);
-      hipLaunchKernelGGL(potrf_trail_kernel, dim3(Tr * (Tr + 1) / 2, nb), dim3(NTHREADS), 0,
-                         stream, table, p);
+      KFAC_LAUNCH_TILE2(potrf_panel_kernel, dim3(Tr, nb), stream, table, p);
+      KFAC_LAUNCH_TILE2(potrf_trail_kernel, dim3(Tr * (Tr + 1) / 2, nb), stream, table, p);
     }
   }
   if (mode == MODE_CHOLESKY) {
@@ -522,12 +551,11 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
     const int na = active(2);
     const dim3 grid((Tmax - 1) * Tmax / 2, na);
     for (int depth = D - 1; depth >= 0 && na > 0; --depth) {
-      hipLaunchKernelGGL(trtri_w_kernel, grid, dim3(NTHREADS), 0, stream, table, depth);
-      hipLaunchKernelGGL(trtri_y_kernel, grid, dim3(NTHREADS), 0, stream, table, depth);
+      KFAC_LAUNCH_TILE2(trtri_w_kernel, grid, stream, table, depth);
+      KFAC_LAUNCH_TILE2(trtri_y_kernel, grid, stream, table, depth);
     }
   }
-  hipLaunchKernelGGL(lauum_kernel, dim3(Tmax * (Tmax + 1) / 2, nmat), dim3(NTHREADS), 0, stream,
-                     table);
+  KFAC_LAUNCH_TILE2(lauum_kernel, dim3(Tmax * (Tmax + 1) / 2, nmat), stream, table);
   return launch_status();
 }
 

@@ -94,22 +94,25 @@ struct ConvA {
   static constexpr int layout = MK;
   const float* p;
   int C, H, W, KH, KW, SH, SW, PH, PW, DH, DW, OH, OW, M, ones;
-  // dy = -2^20 marks a row outside the operand or the row of ones: every
-  // bounds test then fails
-  struct MS { int off; int dy; int dx; bool one; };
+  // Per row m: the element offset of (c, kh, kw) and the two patch displacements
+  // packed as (dy << 16) | (dx & 0xffff) to keep the 16 row states of a thread in
+  // 32 registers.  dy = -32768 marks a row outside the operand (every bounds test
+  // then fails, image sizes are below 32768); dx = -32768 on top of that marks
+  // the row of ones.
+  struct MS { int off; int dydx; };
   struct KS { int off; int y0; int x0; };
+  static __device__ __forceinline__ int pack(int dy, int dx) { return (dy << 16) | (dx & 0xffff); }
   __device__ __forceinline__ MS mstate(int m) const {
     MS s;
-    s.one = false;
-    if (m >= M) { s.off = 0; s.dy = -(1 << 20); s.dx = 0; return s; }
-    if (ones && m == M - 1) { s.off = 0; s.dy = -(1 << 20); s.dx = 0; s.one = true; return s; }
+    if (m >= M) { s.off = 0; s.dydx = pack(-32768, 0); return s; }
+    if (ones && m == M - 1) { s.off = 0; s.dydx = pack(-32768, -32768); return s; }
     const int c = m / (KH * KW);
     const int rem = m - c * KH * KW;
     const int kh = rem / KW;
     const int kw = rem - kh * KW;
-    s.dy = kh * DH;
-    s.dx = kw * DW;
-    s.off = c * H * W + s.dy * W + s.dx;
+    const int dy = kh * DH, dx = kw * DW;
+    s.dydx = pack(dy, dx);
+    s.off = c * H * W + dy * W + dx;
     return s;
   }
   __device__ __forceinline__ KS kstate(int k) const {
@@ -124,12 +127,14 @@ struct ConvA {
     return s;
   }
   __device__ __forceinline__ const float* addr(const MS& m, const KS& k, bool& ok) const {
-    const int y = k.y0 + m.dy;
-    const int x = k.x0 + m.dx;
+    const int y = k.y0 + (m.dydx >> 16);
+    const int x = k.x0 + (int)(short)(m.dydx & 0xffff);
     ok = (unsigned)y < (unsigned)H && (unsigned)x < (unsigned)W;
     return p + (ok ? (unsigned)(k.off + m.off) : 0u);
   }
-  __device__ __forceinline__ bool is_one(const MS& m) const { return ones && m.one; }
+  __device__ __forceinline__ bool is_one(const MS& m) const {
+    return ones && m.dydx == pack(-32768, -32768);
+  }
 };
 
 // ---------------------------------------------------------------------------

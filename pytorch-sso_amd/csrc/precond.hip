@@ -62,7 +62,7 @@ struct EpiSplit {
 
 template <bool SAMPLE>
 __global__ __launch_bounds__(NTHREADS) void precond_first_kernel(const LayerDesc* table) {
-  __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
+  extern __shared__ __attribute__((aligned(16))) float smem[];
   const LayerDesc m = table[blockIdx.y];
   const int ta = tiles128(m.dA), tg = tiles128(m.dG);
   if ((int)blockIdx.x >= ta * tg) return;
@@ -82,7 +82,7 @@ __global__ __launch_bounds__(NTHREADS) void precond_first_kernel(const LayerDesc
 
 template <bool SAMPLE>
 __global__ __launch_bounds__(NTHREADS) void precond_second_kernel(const LayerDesc* table) {
-  __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
+  extern __shared__ __attribute__((aligned(16))) float smem[];
   const LayerDesc m = table[blockIdx.y];
   const int ta = tiles128(m.dA), tg = tiles128(m.dG);
   if ((int)blockIdx.x >= ta * tg) return;
@@ -142,11 +142,11 @@ static int run_layers(int layers, const int* dG, const int* dA, const float* con
   }
   const dim3 grid(maxtiles, layers);
   if (sample) {
-    hipLaunchKernelGGL(precond_first_kernel<true>, grid, dim3(NTHREADS), 0, stream, table);
-    hipLaunchKernelGGL(precond_second_kernel<true>, grid, dim3(NTHREADS), 0, stream, table);
+    KFAC_LAUNCH_TILE2(precond_first_kernel<true>, grid, stream, table);
+    KFAC_LAUNCH_TILE2(precond_second_kernel<true>, grid, stream, table);
   } else {
-    hipLaunchKernelGGL(precond_first_kernel<false>, grid, dim3(NTHREADS), 0, stream, table);
-    hipLaunchKernelGGL(precond_second_kernel<false>, grid, dim3(NTHREADS), 0, stream, table);
+    KFAC_LAUNCH_TILE2(precond_first_kernel<false>, grid, stream, table);
+    KFAC_LAUNCH_TILE2(precond_second_kernel<false>, grid, stream, table);
   }
   return launch_status();
 }
