@@ -75,7 +75,85 @@ __global__ __launch_bounds__(EW_THREADS) void vec_kernel(const VecDesc* table) {
   }
 }
 
+// y = s0*x + s1*y on float4 (all pointers 16-byte aligned, numel % 4 == 0): the
+// running average of the factors moves the most bytes of all tails
+__global__ __launch_bounds__(EW_THREADS) void axpby4_kernel(const VecDesc* table) {
+  const VecDesc m = table[blockIdx.y];
+  const long n4 = m.numel >> 2;
+  const float4* x = reinterpret_cast<const float4*>(m.a);
+  float4* y = reinterpret_cast<float4*>(m.b);
+  const long stride = (long)gridDim.x * EW_THREADS;
+  for (long i = (long)blockIdx.x * EW_THREADS + threadIdx.x; i < n4; i += stride) {
+    const float4 a = x[i];
+    float4 o;
+    if (m.s1 != 0.f) {
+      const float4 b = y[i];
+      o.x = m.s0 * a.x + m.s1 * b.x;
+      o.y = m.s0 * a.y + m.s1 * b.y;
+      o.z = m.s0 * a.z + m.s1 * b.z;
+      o.w = m.s0 * a.w + m.s1 * b.w;
+    } else {
+      o.x = m.s0 * a.x;
+      o.y = m.s0 * a.y;
+      o.z = m.s0 * a.z;
+      o.w = m.s0 * a.w;
+    }
+    y[i] = o;
+  }
+}
+
 static size_t vec_workspace(int count) { return (size_t)count * sizeof(VecDesc); }
+
+static long upload_table(const std::vector<VecDesc>& descs, VecDesc* table, long per_block,
+                         hipStream_t stream);
+
+// the running average: float4 kernel for the tensors that allow it, scalar for the rest
+static int run_axpby(std::vector<VecDesc>& descs, void* workspace, size_t workspace_bytes,
+                     hipStream_t stream) {
+  const int count = (int)descs.size();
+  if (count == 0) return KFAC_OK;
+  if (!workspace || workspace_bytes < vec_workspace(count)) return KFAC_ERR_WORKSPACE;
+  std::vector<VecDesc> v4, sc;
+  for (const VecDesc& d : descs) {
+    const bool aligned = (((uintptr_t)d.a | (uintptr_t)d.b) & 15) == 0 && (d.numel & 3) == 0;
+    (aligned ? v4 : sc).push_back(d);
+  }
+  VecDesc* table = (VecDesc*)workspace;
+  if (!v4.empty()) {
+    const long maxblocks = upload_table(v4, table, 4L * EW_THREADS * 4, stream);
+    long gx = std::max<long>(64, 8192 / (long)v4.size());
+    gx = std::min(gx, maxblocks);
+    hipLaunchKernelGGL(axpby4_kernel, dim3((unsigned)gx, (unsigned)v4.size()), dim3(EW_THREADS), 0,
+                       stream, table);
+  }
+  if (!sc.empty()) {
+    VecDesc* t2 = table + v4.size();
+    const long maxblocks = upload_table(sc, t2, EW_BLOCK, stream);
+    long gx = std::max<long>(64, 4096 / (long)sc.size());
+    gx = std::min(gx, maxblocks);
+    hipLaunchKernelGGL((vec_kernel<OP_AXPBY>), dim3((unsigned)gx, (unsigned)sc.size()),
+                       dim3(EW_THREADS), 0, stream, t2);
+  }
+  return launch_status();
+}
+
+// copies the descriptors to the device table; returns the block count of the largest tensor
+static long upload_table(const std::vector<VecDesc>& descs, VecDesc* table, long per_block,
+                         hipStream_t stream) {
+  const int count = (int)descs.size();
+  long maxblocks = 1;
+  for (int s0 = 0; s0 < count; s0 += VEC_CHUNK) {
+    VecChunk chunk;
+    const int cnt = std::min(VEC_CHUNK, count - s0);
+    for (int k = 0; k < cnt; ++k) {
+      chunk.d[k] = descs[s0 + k];
+      maxblocks = std::max(maxblocks, (descs[s0 + k].numel + per_block - 1) / per_block);
+    }
+    hipLaunchKernelGGL(vec_setup_kernel, dim3(1), dim3(VEC_CHUNK), 0, stream, chunk, table, s0,
+                       cnt);
+  }
+  return maxblocks;
+}
 
 template <int OP>
 static int run_vec(std::vector<VecDesc>& descs, void* workspace, size_t workspace_bytes,
@@ -104,28 +182,43 @@ static int run_vec(std::vector<VecDesc>& descs, void* workspace, size_t workspac
 
 // ---- BatchNorm diagonal curvature ----------------------------------------
 
-// out[row] = sum_i ((x[row][i] - shift[c]) / scale[c])^2, row = (n, c), c = row % C
+// out[row] = sum_i ((x[row][i] - shift[c]) / scale[c])^2, row = (n, c), c = row % C.
+// One wave per row when rows are short (a 256-thread workgroup then covers 4
+// rows), one workgroup per row otherwise; lanes stride the row so that loads
+// coalesce.
+template <int ROWS_PER_BLOCK>
 __global__ __launch_bounds__(256) void rowsq_kernel(const float* x, const float* scale,
-                                                    const float* shift, int C, int len,
+                                                    const float* shift, long rows, int C, int len,
                                                     float* out) {
+  constexpr int TPR = 256 / ROWS_PER_BLOCK;       // threads per row
   __shared__ float red[256];
-  const long row = blockIdx.x;
-  const int c = (int)(row % C);
-  const float sh = shift ? shift[c] : 0.f;
-  const float rs = scale ? 1.f / scale[c] : 1.f;
-  const float* p = x + row * (long)len;
+  const int sub = threadIdx.x / TPR;
+  const int lane = threadIdx.x - sub * TPR;
+  const long row = (long)blockIdx.x * ROWS_PER_BLOCK + sub;
   float s = 0.f;
-  for (int i = threadIdx.x; i < len; i += 256) {
-    const float v = (p[i] - sh) * rs;
-    s += v * v;
+  if (row < rows) {
+    const int c = (int)(row % C);
+    const float sh = shift ? shift[c] : 0.f;
+    const float rs = scale ? 1.f / scale[c] : 1.f;
+    const float* p = x + row * (long)len;
+    int i = lane;
+    for (; i + 3 * TPR < len; i += 4 * TPR) {       // 4 loads in flight per thread
+      const float v0 = (p[i] - sh) * rs, v1 = (p[i + TPR] - sh) * rs;
+      const float v2 = (p[i + 2 * TPR] - sh) * rs, v3 = (p[i + 3 * TPR] - sh) * rs;
+      s += v0 * v0 + v1 * v1 + v2 * v2 + v3 * v3;
+    }
+    for (; i < len; i += TPR) {
+      const float v = (p[i] - sh) * rs;
+      s += v * v;
+    }
   }
   red[threadIdx.x] = s;
   __syncthreads();
-  for (int w = 128; w > 0; w >>= 1) {
-    if (threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+  for (int w = TPR / 2; w > 0; w >>= 1) {
+    if (lane < w) red[threadIdx.x] += red[threadIdx.x + w];
     __syncthreads();
   }
-  if (threadIdx.x == 0) out[row] = red[0];
+  if (lane == 0 && row < rows) out[row] = red[threadIdx.x];
 }
 
 // w_curv[c] = alpha * sum_n sx[n][c] * sg[n][c] ; b_curv[c] = alpha * sum_n sg[n][c]
@@ -159,7 +252,7 @@ int kfac_axpby_batched(int count, const int64_t* numel, const float* const* x, f
     if (numel[i] <= 0 || !x[i] || !y[i]) return KFAC_ERR_ARG;
     d[i] = VecDesc{(float*)x[i], y[i], nullptr, (long)numel[i], a, b, 0.f, 0.f};
   }
-  return run_vec<OP_AXPBY>(d, workspace, workspace_bytes, (hipStream_t)stream);
+  return run_axpby(d, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 int kfac_diag_inverse_batched(int count, const int64_t* numel, const float* const* ema,
@@ -207,8 +300,12 @@ int kfac_rowsq_sum(const float* x, int64_t rows, int channels, int len, const fl
                    const float* shift, float* out, void* stream) {
   if (!x || !out || rows <= 0 || channels <= 0 || len <= 0 || rows >= (int64_t)1 << 31)
     return KFAC_ERR_ARG;
-  hipLaunchKernelGGL(rowsq_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, x,
-                     scale, shift, channels, len, out);
+  if (len <= 256)
+    hipLaunchKernelGGL(rowsq_kernel<4>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                       (hipStream_t)stream, x, scale, shift, (long)rows, channels, len, out);
+  else
+    hipLaunchKernelGGL(rowsq_kernel<1>, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, x,
+                       scale, shift, (long)rows, channels, len, out);
   return launch_status();
 }
 

@@ -56,7 +56,7 @@ static SyrkPlan plan_syrk(int d, long K) {
 }
 
 template <class OP, int W>
-__global__ __launch_bounds__(64 * W * W, W == 2 ? 2 : 1) void syrk_kernel(OP op, int d, int K, int T, int ntiles,
+__global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void syrk_kernel(OP op, int d, int K, int T, int ntiles,
                                                           int splits, int chunks_per_split,
                                                           float* C, float alpha, float beta,
                                                           float* ws) {

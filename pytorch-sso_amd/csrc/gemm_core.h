@@ -44,7 +44,7 @@ struct Cfg {
   static constexpr int TM = 64 * WM;
   static constexpr int TN = 64 * WN;
   static constexpr int NT = 64 * WM * WN;
-  static constexpr int KC = (WM * WN >= 4) ? 32 : 16;
+  static constexpr int KC = 16;
   static constexpr int LDS_MK = KC + 4;          // padded row of an MK chunk (conflict-free b128)
   static constexpr int P_FLOATS = LDS_MK * TM;   // >= KC*TM and TM*LDS_MK
   static constexpr int Q_FLOATS = LDS_MK * TN;
@@ -222,26 +222,47 @@ __device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0
     }
     const lds_f* const tpc = sm + cur * STAGE;
     const lds_f* const tqc = tpc + C::P_FLOATS;
+    lds_f* const tpn = sm + (cur ^ 1) * STAGE;
+    // The chunk is consumed in 16-deep slices.  The LDS writes of the NEXT chunk
+    // are issued before the last slice, so that they (and the wait for the
+    // global loads that feed them) sit in the shadow of MFMAs instead of in
+    // front of the barrier.
 #pragma unroll
-    for (int kofs = 0; kofs < KC; kofs += 16) {
+    for (int sl = 0; sl < KC / 16; ++sl) {
       float fa[2][8], fb[2][8];
-      load_frags<OPP::layout, C::TM, C::LDS_MK>(tpc, wm, r, h, kofs, fa);
+      load_frags<OPP::layout, C::TM, C::LDS_MK>(tpc, wm, r, h, 16 * sl, fa);
       if (same)
-        load_frags<OPP::layout, C::TM, C::LDS_MK>(tpc, wn, r, h, kofs, fb);
+        load_frags<OPP::layout, C::TM, C::LDS_MK>(tpc, wn, r, h, 16 * sl, fb);
       else
-        load_frags<OPQ::layout, C::TN, C::LDS_MK>(tqc, wn, r, h, kofs, fb);
+        load_frags<OPQ::layout, C::TN, C::LDS_MK>(tqc, wn, r, h, 16 * sl, fb);
+      if (sl == KC / 16 - 1) {
 #pragma unroll
-      for (int s = 0; s < 8; ++s)
+        for (int s = 0; s < 4; ++s)
 #pragma unroll
-        for (int a = 0; a < 2; ++a)
+          for (int a = 0; a < 2; ++a)
 #pragma unroll
-          for (int b = 0; b < 2; ++b)
-            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a][s], fb[b][s], acc[a][b], 0, 0, 0);
-    }
-    if (more) {
-      lds_f* const tpn = sm + (cur ^ 1) * STAGE;
-      sp.commit(tpn);
-      if (!same) sq.commit(tpn + C::P_FLOATS);
+            for (int b = 0; b < 2; ++b)
+              acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a][s], fb[b][s], acc[a][b], 0, 0, 0);
+        if (more) {
+          sp.commit(tpn);
+          if (!same) sq.commit(tpn + C::P_FLOATS);
+        }
+#pragma unroll
+        for (int s = 4; s < 8; ++s)
+#pragma unroll
+          for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+              acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a][s], fb[b][s], acc[a][b], 0, 0, 0);
+      } else {
+#pragma unroll
+        for (int s = 0; s < 8; ++s)
+#pragma unroll
+          for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+              acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a][s], fb[b][s], acc[a][b], 0, 0, 0);
+      }
     }
     __syncthreads();
   }

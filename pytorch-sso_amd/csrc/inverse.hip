@@ -329,22 +329,41 @@ __global__ __launch_bounds__(NTHREADS) void potrf_panel_kernel(const MatDesc* ta
   gemm_tile(P, Q, 0, bj * BN, 0, DB, false, epi, smem);
 }
 
-// trailing update: A[i, j] -= U[p, i]^T U[p, j],  p < i <= j
-__global__ __launch_bounds__(NTHREADS) void potrf_trail_kernel(const MatDesc* table, int p) {
+// trailing update with the block rows [kb0, kb0 + nk) of U:
+//   A[i, j] -= sum_k U[k, i]^T U[k, j]   for block rows row_lo <= i < row_hi, j >= i.
+// The Cholesky runs in outer panels of OUTER_BLOCKS diagonal blocks: inside an
+// outer panel each step updates only the remaining rows of that panel (nk = 1),
+// and the rows beyond it receive the whole panel at once (nk = OUTER_BLOCKS),
+// which cuts the read-modify-write passes over the trailing matrix by that factor.
+constexpr int OUTER_BLOCKS = 4;
+
+__global__ __launch_bounds__(NTHREADS) void potrf_trail_kernel(const MatDesc* table, int kb0,
+                                                               int nk, int row_lo, int row_hi) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   const MatDesc m = table[blockIdx.y];
-  const int Tr = m.T - p - 1;
-  if (Tr <= 0) return;
-  const int ntiles = Tr * (Tr + 1) / 2;
-  if ((int)blockIdx.x >= ntiles) return;
+  const int T = m.T;
+  const int hi = min(row_hi, T);
+  if (row_lo >= hi) return;
   int bi, bj;
-  upper_tile(blockIdx.x, Tr, bi, bj);
-  bi += p + 1;
-  bj += p + 1;
+  if (row_hi >= T) {
+    // all remaining rows: walk the upper triangle of the (T - row_lo)^2 block grid
+    const int Tr = T - row_lo;
+    if ((int)blockIdx.x >= Tr * (Tr + 1) / 2) return;
+    upper_tile(blockIdx.x, Tr, bi, bj);
+    bi += row_lo;
+    bj += row_lo;
+  } else {
+    // a few rows: rectangular walk, tiles left of the diagonal exit
+    const int width = T - row_lo;
+    const int rr = blockIdx.x / width;
+    bi = row_lo + rr;
+    bj = row_lo + (blockIdx.x - rr * width);
+    if (bi >= hi || bj < bi) return;
+  }
   const int n = m.n;
-  DenseKM P{m.U + (size_t)p * DB * n, nullptr, n, n, 0};
+  DenseKM P{m.U + (size_t)kb0 * DB * n, nullptr, n, n, 0};
   EpiStore epi{m.U, n, n, n, -1.f, 1.f, false};
-  gemm_tile(P, P, bi * BM, bj * BN, 0, DB, bi == bj, epi, smem);
+  gemm_tile(P, P, bi * BM, bj * BN, 0, nk * DB, bi == bj, epi, smem);
 }
 
 // ---- Y = U^-1 by balanced recursive halving over the 128-blocks ---------------
@@ -530,15 +549,27 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
   hipLaunchKernelGGL(inv_copy_damp_kernel, dim3(Tmax * (Tmax + 1) / 2, nmat), dim3(256), 0, stream,
                      table, info);
 
-  for (int p = 0; p < Tmax; ++p) {
-    const int na = active(p + 1);
-    hipLaunchKernelGGL(potrf_diag_kernel, dim3(na), dim3(256), DIAG_SMEM_BYTES, stream, table, p,
-                       info);
-    const int nb = active(p + 2);
-    if (nb > 0) {
-      const int Tr = Tmax - p - 1;
-      KFAC_LAUNCH_TILE2(potrf_panel_kernel, dim3(Tr, nb), stream, table, p);
-      KFAC_LAUNCH_TILE2(potrf_trail_kernel, dim3(Tr * (Tr + 1) / 2, nb), stream, table, p);
+  for (int P0 = 0; P0 < Tmax; P0 += OUTER_BLOCKS) {
+    const int Pend = std::min(P0 + OUTER_BLOCKS, Tmax);
+    for (int p = P0; p < Pend; ++p) {
+      const int na = active(p + 1);
+      hipLaunchKernelGGL(potrf_diag_kernel, dim3(na), dim3(256), DIAG_SMEM_BYTES, stream, table,
+                         p, info);
+      const int nb = active(p + 2);
+      if (nb == 0) continue;
+      KFAC_LAUNCH_TILE2(potrf_panel_kernel, dim3(Tmax - p - 1, nb), stream, table, p);
+      if (p + 1 < Pend) {
+        // rows (p, Pend) of the outer panel, all columns to the right
+        const int rows = Pend - p - 1, width = Tmax - p - 1;
+        KFAC_LAUNCH_TILE2(potrf_trail_kernel, dim3(rows * width, nb), stream, table, p, 1, p + 1,
+                          Pend);
+      }
+    }
+    const int nc = active(Pend + 1);
+    if (Pend < Tmax && nc > 0) {
+      const int Tr = Tmax - Pend;
+      KFAC_LAUNCH_TILE2(potrf_trail_kernel, dim3(Tr * (Tr + 1) / 2, nc), stream, table, P0,
+                        Pend - P0, Pend, Tmax);
     }
   }
   if (mode == MODE_CHOLESKY) {

@@ -114,11 +114,16 @@ static int run_layers(int layers, const int* dG, const int* dA, const float* con
   char* tbase = (char*)workspace + align256((size_t)layers * sizeof(LayerDesc));
   size_t off = 0;
   int maxtiles = 0;
+  // longest tiles first: the table (= grid.y) is ordered by the reduction length of
+  // the second, larger product so that the tail of the launch is made of short tiles
+  std::vector<int> order(layers);
+  for (int l = 0; l < layers; ++l) order[l] = l;
+  std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return dA[a] > dA[b]; });
   for (int s0 = 0; s0 < layers; s0 += LAYER_CHUNK) {
     LayerChunk chunk;
     const int cnt = std::min(LAYER_CHUNK, layers - s0);
     for (int k = 0; k < cnt; ++k) {
-      const int l = s0 + k;
+      const int l = order[s0 + k];
       LayerDesc& d = chunk.d[k];
       d.L = L[l];
       d.R = R[l];
