@@ -15,6 +15,9 @@
  *    tells the caller how much to bring;
  *  - the return value is 0 on success or one of the KFAC_ERR_* codes; nothing
  *    throws and nothing keeps a caller pointer after returning;
+ *  - sizes: any single matrix (factor, inverse, gradient viewed as 2-D) is at most
+ *    1 GiB (16384 x 16384 fp32); layer inputs of any size are accepted (the factor
+ *    builders consume them in slices of at most 1 GiB along the batch dimension);
  *  - entry points are re-entrant: they may be called from any host thread
  *    (the backward hooks of the host code run on autograd's worker thread).
  */
@@ -29,7 +32,7 @@ extern "C" {
 #endif
 
 #define KFAC_OK 0
-#define KFAC_ERR_ARG 1        /* null pointer, non-positive size, size above 2^31 elements */
+#define KFAC_ERR_ARG 1        /* null pointer, non-positive size, matrix above 16384 x 16384 */
 #define KFAC_ERR_WORKSPACE 2  /* workspace_bytes smaller than the query says */
 #define KFAC_ERR_LAUNCH 3     /* the HIP runtime refused a launch */
 

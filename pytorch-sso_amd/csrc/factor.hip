@@ -183,15 +183,29 @@ size_t kfac_factor_workspace_bytes(int d, int64_t K) {
   return p.splits > 1 ? (size_t)p.splits * p.ntiles * p.ts * p.ts * sizeof(float) : 0;
 }
 
+// Operand offsets are 30-bit byte offsets: an input larger than 1 GiB is consumed
+// in slices along its leading dimension, each slice accumulating into C.
+static int64_t slice_len(int64_t total, int64_t elems_per_unit) {
+  const int64_t max_units = (MAX_OPERAND_BYTES / 4) / elems_per_unit;
+  return max_units < 1 ? 0 : (total < max_units ? total : max_units);
+}
+
 int kfac_factor_linear(const float* x, int64_t rows, int f, int64_t ldx, int add_bias,
                        float alpha, float beta, float* C, void* workspace,
                        size_t workspace_bytes, void* stream) {
   if (!x || !C || rows <= 0 || f <= 0 || ldx < f) return KFAC_ERR_ARG;
-  if (rows * ldx >= (int64_t)1 << 31) return KFAC_ERR_ARG;
   const int d = f + (add_bias ? 1 : 0);
-  DenseKM op{x, nullptr, (int)ldx, d, add_bias ? 1 : 0};
-  return launch_syrk(op, d, rows, alpha, beta, C, workspace, workspace_bytes,
-                     (hipStream_t)stream);
+  if ((int64_t)d * d * 4 > MAX_OPERAND_BYTES) return KFAC_ERR_ARG;
+  const int64_t step = slice_len(rows, ldx);
+  if (step == 0) return KFAC_ERR_ARG;
+  for (int64_t r0 = 0; r0 < rows; r0 += step) {
+    const int64_t cnt = rows - r0 < step ? rows - r0 : step;
+    DenseKM op{x + r0 * ldx, nullptr, (int)ldx, d, add_bias ? 1 : 0};
+    const int st = launch_syrk(op, d, cnt, alpha, r0 == 0 ? beta : 1.f, C, workspace,
+                               workspace_bytes, (hipStream_t)stream);
+    if (st != KFAC_OK) return st;
+  }
+  return KFAC_OK;
 }
 
 int kfac_factor_conv_a(const float* x, int n, int c, int H, int W, int kh, int kw, int sh, int sw,
@@ -201,24 +215,40 @@ int kfac_factor_conv_a(const float* x, int n, int c, int H, int W, int kh, int k
       sw <= 0 || ph < 0 || pw < 0 || dh <= 0 || dw <= 0)
     return KFAC_ERR_ARG;
   if (H >= 16384 || W >= 16384 || kh * dh >= 16384 || kw * dw >= 16384) return KFAC_ERR_ARG;
-  if ((int64_t)n * c * H * W >= (int64_t)1 << 31) return KFAC_ERR_ARG;
   const int OH = (H + 2 * ph - dh * (kh - 1) - 1) / sh + 1;
   const int OW = (W + 2 * pw - dw * (kw - 1) - 1) / sw + 1;
   if (OH <= 0 || OW <= 0) return KFAC_ERR_ARG;
-  const int64_t K = (int64_t)n * OH * OW;
-  if (K >= (int64_t)1 << 31) return KFAC_ERR_ARG;
-  const int d = c * kh * kw + (add_bias ? 1 : 0);
-  ConvA op{x, c, H, W, kh, kw, sh, sw, ph, pw, dh, dw, OH, OW, d, add_bias ? 1 : 0};
-  return launch_syrk(op, d, K, alpha, beta, C, workspace, workspace_bytes, (hipStream_t)stream);
+  const int64_t dd = (int64_t)c * kh * kw + (add_bias ? 1 : 0);
+  if (dd * dd * 4 > MAX_OPERAND_BYTES) return KFAC_ERR_ARG;
+  const int d = (int)dd;
+  const int64_t image = (int64_t)c * H * W;
+  const int64_t step = slice_len(n, image);   // (offsets into the padding are never used)
+  if (step == 0) return KFAC_ERR_ARG;
+  for (int64_t n0 = 0; n0 < n; n0 += step) {
+    const int cnt = (int)(n - n0 < step ? n - n0 : step);
+    ConvA op{x + n0 * image, c, H, W, kh, kw, sh, sw, ph, pw, dh, dw, OH, OW, d, add_bias ? 1 : 0};
+    const int st = launch_syrk(op, d, (int64_t)cnt * OH * OW, alpha, n0 == 0 ? beta : 1.f, C,
+                               workspace, workspace_bytes, (hipStream_t)stream);
+    if (st != KFAC_OK) return st;
+  }
+  return KFAC_OK;
 }
 
 int kfac_factor_conv_g(const float* g, int n, int c, int h, int w, float alpha, float beta,
                        float* C, void* workspace, size_t workspace_bytes, void* stream) {
   if (!g || !C || n <= 0 || c <= 0 || h <= 0 || w <= 0) return KFAC_ERR_ARG;
-  if ((int64_t)n * c * h * w >= (int64_t)1 << 31) return KFAC_ERR_ARG;
-  ConvG op{g, c, h * w};
-  return launch_syrk(op, c, (int64_t)n * h * w, alpha, beta, C, workspace, workspace_bytes,
-                     (hipStream_t)stream);
+  if ((int64_t)c * c * 4 > MAX_OPERAND_BYTES) return KFAC_ERR_ARG;
+  const int64_t image = (int64_t)c * h * w;
+  const int64_t step = slice_len(n, image);
+  if (step == 0) return KFAC_ERR_ARG;
+  for (int64_t n0 = 0; n0 < n; n0 += step) {
+    const int cnt = (int)(n - n0 < step ? n - n0 : step);
+    ConvG op{g + n0 * image, c, h * w};
+    const int st = launch_syrk(op, c, (int64_t)cnt * h * w, alpha, n0 == 0 ? beta : 1.f, C,
+                               workspace, workspace_bytes, (hipStream_t)stream);
+    if (st != KFAC_OK) return st;
+  }
+  return KFAC_OK;
 }
 
 }  // extern "C"

@@ -66,6 +66,19 @@ typedef __attribute__((address_space(3))) float lds_f;
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4f lds_f4;
 
+// ---- raw buffer addressing (see the operand contract in operands.h) ----------
+constexpr unsigned INV_M = 0x80000000u;
+constexpr unsigned INV_K = 0x40000000u;
+constexpr long MAX_OPERAND_BYTES = 1L << 30;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const float* p) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p), 0, (int)MAX_OPERAND_BYTES,
+                                           0x00020000);
+}
+__device__ __forceinline__ float buffer_load(__amdgpu_buffer_rsrc_t r, unsigned off) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, 0));
+}
+
 // ---------------------------------------------------------------------------
 // global -> register -> LDS staging of one operand chunk (KC x ROWS elements
 // swept by NT threads)
@@ -79,8 +92,7 @@ struct Stager {
   static constexpr int MSTEP = NT / KC;                 // MK: m rows per sweep
   typename OP::MS ms[NM];
   float regs[CNT];
-  unsigned okbits;     // element i is inside the operand and the k range
-  unsigned onebits;    // element i is the constant 1
+  unsigned onebits;    // element i is the constant 1 (and inside the k range)
 
   __device__ __forceinline__ void init(const OP& op, int m0) {
     const int t = threadIdx.x;
@@ -90,40 +102,38 @@ struct Stager {
 #pragma unroll
       for (int i = 0; i < NM; ++i) ms[i] = op.mstate(m0 + (t / KC) + MSTEP * i);
     }
-    okbits = 0;
     onebits = 0;
   }
 
-  // Issue the global loads of one chunk.  The loaded values are not touched
-  // here (masking happens in commit), so nothing waits on memory yet.
+  // Issue the buffer loads of one chunk.  Elements outside the operand or the
+  // k range come back as 0 from the hardware's range check; the loaded values
+  // are not touched until commit, so nothing here waits on memory.
   __device__ __forceinline__ void fetch(const OP& op, int k0, int kend) {
     const int t = threadIdx.x;
-    unsigned okb = 0, oneb = 0;
+    const __amdgpu_buffer_rsrc_t rs = op.rsrc();
+    unsigned oneb = 0;
     if (OP::layout == KM) {
 #pragma unroll
       for (int i = 0; i < CNT; ++i) {
         const int k = k0 + (t / ROWS) + KSTEP * i;
         const bool kin = k < kend;
-        bool ok;
-        const float* a = op.addr(ms[0], op.kstate(kin ? k : k0), ok);   // k0 is in range
-        regs[i] = *a;
-        okb |= (unsigned)(ok && kin) << i;
+        const typename OP::KS ks = op.kstate(k, kin);
+        regs[i] = buffer_load(rs, op.off(ms[0], ks));
+        if constexpr (OP::has_second) {
+          if (op.second()) regs[i] += buffer_load(op.rsrc2(), op.off2(ms[0], ks));
+        }
         oneb |= (unsigned)(op.is_one(ms[0]) && kin) << i;
       }
     } else {
       const int k = k0 + (t % KC);
       const bool kin = k < kend;
-      const typename OP::KS ks = op.kstate(kin ? k : k0);
+      const typename OP::KS ks = op.kstate(k, kin);
 #pragma unroll
       for (int i = 0; i < CNT; ++i) {
-        bool ok;
-        const float* a = op.addr(ms[i], ks, ok);
-        regs[i] = *a;
-        okb |= (unsigned)(ok && kin) << i;
+        regs[i] = buffer_load(rs, op.off(ms[i], ks));
         oneb |= (unsigned)(op.is_one(ms[i]) && kin) << i;
       }
     }
-    okbits = okb;
     onebits = oneb;
   }
 
@@ -131,8 +141,7 @@ struct Stager {
     const int t = threadIdx.x;
 #pragma unroll
     for (int i = 0; i < CNT; ++i) {
-      float v = ((okbits >> i) & 1u) ? regs[i] : 0.f;
-      v = ((onebits >> i) & 1u) ? 1.f : v;
+      const float v = ((onebits >> i) & 1u) ? 1.f : regs[i];
       if (OP::layout == KM)
         tile[((t / ROWS) + KSTEP * i) * ROWS + (t % ROWS)] = v;
       else

@@ -610,7 +610,7 @@ int kfac_damped_inverse_batched(int count, const int* dims, const float* const* 
   if (count < 0 || (count > 0 && (!dims || !src || !dst || !info))) return KFAC_ERR_ARG;
   std::vector<HostMat> mats(count);
   for (int i = 0; i < count; ++i) {
-    if (dims[i] <= 0 || dims[i] > 46340 || !src[i] || !dst[i] || src[i] == dst[i])
+    if (dims[i] <= 0 || dims[i] > 16384 || !src[i] || !dst[i] || src[i] == dst[i])
       return KFAC_ERR_ARG;
     mats[i] = HostMat{src[i], dst[i], dims[i], damp ? damp[i] : 0.f, -1, 0, i};
   }
@@ -626,7 +626,7 @@ int kfac_pi_damped_inverse_batched(int layers, const int* dA, const int* dG,
     return KFAC_ERR_ARG;
   std::vector<HostMat> mats(2 * layers);
   for (int l = 0; l < layers; ++l) {
-    if (dA[l] <= 0 || dG[l] <= 0 || dA[l] > 46340 || dG[l] > 46340 || !A[l] || !G[l] ||
+    if (dA[l] <= 0 || dG[l] <= 0 || dA[l] > 16384 || dG[l] > 16384 || !A[l] || !G[l] ||
         !Ainv[l] || !Ginv[l] || A[l] == Ainv[l] || G[l] == Ginv[l] || !(damping[l] >= 0.f))
       return KFAC_ERR_ARG;
     const float r = sqrtf(damping[l]);
@@ -642,7 +642,7 @@ int kfac_cholesky_upper_batched(int count, const int* dims, const float* const* 
   if (count < 0 || (count > 0 && (!dims || !src || !dst || !info))) return KFAC_ERR_ARG;
   std::vector<HostMat> mats(count);
   for (int i = 0; i < count; ++i) {
-    if (dims[i] <= 0 || dims[i] > 46340 || !src[i] || !dst[i] || src[i] == dst[i])
+    if (dims[i] <= 0 || dims[i] > 16384 || !src[i] || !dst[i] || src[i] == dst[i])
       return KFAC_ERR_ARG;
     mats[i] = HostMat{src[i], dst[i], dims[i], 0.f, -1, 0, i};
   }

@@ -10,80 +10,99 @@ namespace kfac {
 //   extra == 1 : the constant 1 (bias augmentation of a Linear input)
 //   extra == 2 : taken from vec[k] (bias gradient appended to a weight gradient)
 // ---------------------------------------------------------------------------
-// Operand functor contract used by the staging code of the tile engine:
-//   MS mstate(m), KS kstate(k)      per-index precomputation
-//   const float* addr(ms, ks, ok)   ALWAYS a readable address; ok = false when the
-//                                   element lies outside the operand (value -> 0)
-//   bool is_one(ms)                 the element is the constant 1 (bias augmentation)
-// Nothing here branches, and the value is only looked at when the chunk is
-// written to LDS, so the global loads of the next chunk stay in flight while
-// the MFMAs of the current one run.
-
-// Dense row-major matrix read as P(k, m) = p[k*ld + m]  (m contiguous).
+// Operand functor contract used by the staging code of the tile engine.
+// Elements are read with raw buffer loads (buffer_load_dword ... offen): the
+// functor supplies a buffer resource over its tensor and a 32-bit BYTE offset
+// per element, and an element outside the operand gets an offset beyond the
+// buffer, for which the hardware returns 0 without touching memory.  So there
+// is no branch, no 64-bit address arithmetic and no masking of loaded values.
+//   rsrc()                    buffer resource (uniform) over [p, p + 1 GiB); valid
+//                             offsets lie inside the tensor by construction
+//   MS mstate(m), KS kstate(k, valid)   per-index precomputation
+//   unsigned off(ms, ks)      byte offset; >= num_records when outside
+//   bool is_one(ms)           the element is the constant 1 (bias augmentation)
+// Offsets of valid elements are below 2^30 (tensors are limited to 1 GiB per
+// call; the entry points split larger ones); an invalid row adds 2^31 and an
+// invalid k adds 2^30, so every sum with an invalid part lands in [2^30, 2^32).
+// Dense row-major matrix read as P(k, m) = p[k*ld + m]  (m contiguous), K rows.
 // Optional last column (index M-1) that is not in memory:
 //   extra == 1 : the constant 1 (bias augmentation of a Linear input)
-//   extra == 2 : taken from vec[k] (bias gradient appended to a weight gradient)
+//   extra == 2 : taken from vec[k] (bias gradient appended to a weight gradient);
+//                read through a second resource and added (one of the two loads
+//                of an element is always out of range, i.e. 0)
 struct DenseKM {
   static constexpr int layout = KM;
+  static constexpr bool has_second = true;
   const float* p;
   const float* vec;
   int ld, M, extra;
-  struct MS { const float* base; int stride; bool valid; bool one; };
-  struct KS { int k; };
+  struct MS { unsigned off; unsigned off2; bool one; };
+  struct KS { unsigned off; unsigned off2; };
+  __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc() const {
+    return make_rsrc(p);
+  }
+  __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc2() const {
+    return make_rsrc(extra == 2 ? vec : p);
+  }
+  __device__ __forceinline__ bool second() const { return extra == 2; }
   __device__ __forceinline__ MS mstate(int m) const {
     MS s;
-    s.base = p; s.stride = 0; s.valid = false; s.one = false;
+    s.off = INV_M; s.off2 = INV_M; s.one = false;
     if (m < M) {
-      if (extra == 1 && m == M - 1) { s.one = true; }
-      else if (extra == 2 && m == M - 1) { s.base = vec; s.stride = 1; s.valid = true; }
-      else { s.base = p + m; s.stride = ld; s.valid = true; }
+      if (extra == 1 && m == M - 1) s.one = true;
+      else if (extra == 2 && m == M - 1) s.off2 = 0;
+      else s.off = (unsigned)m * 4u;
     }
     return s;
   }
-  __device__ __forceinline__ KS kstate(int k) const { return KS{k}; }
-  __device__ __forceinline__ const float* addr(const MS& m, const KS& k, bool& ok) const {
-    ok = m.valid;
-    return m.base + (unsigned)(k.k * m.stride);
+  __device__ __forceinline__ KS kstate(int k, bool valid) const {
+    return KS{valid ? (unsigned)(k * ld) * 4u : INV_K, valid ? (unsigned)k * 4u : INV_K};
   }
+  __device__ __forceinline__ unsigned off(const MS& m, const KS& k) const { return m.off + k.off; }
+  __device__ __forceinline__ unsigned off2(const MS& m, const KS& k) const { return m.off2 + k.off2; }
   __device__ __forceinline__ bool is_one(const MS& m) const { return extra == 1 && m.one; }
 };
 
-// Dense row-major matrix read as P(k, m) = p[m*ld + k]  (k contiguous).
+// Dense row-major matrix read as P(k, m) = p[m*ld + k]  (k contiguous), M rows.
 struct DenseMK {
   static constexpr int layout = MK;
+  static constexpr bool has_second = false;
   const float* p;
   int ld, M;
-  struct MS { const float* row; bool valid; };
-  struct KS { int k; };
+  struct MS { unsigned off; };
+  struct KS { unsigned off; };
+  __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc() const {
+    return make_rsrc(p);
+  }
   __device__ __forceinline__ MS mstate(int m) const {
-    return MS{m < M ? p + (size_t)m * ld : p, m < M};
+    return MS{m < M ? (unsigned)(m * ld) * 4u : INV_M};
   }
-  __device__ __forceinline__ KS kstate(int k) const { return KS{k}; }
-  __device__ __forceinline__ const float* addr(const MS& m, const KS& k, bool& ok) const {
-    ok = m.valid;
-    return m.row + (m.valid ? (unsigned)k.k : 0u);
+  __device__ __forceinline__ KS kstate(int k, bool valid) const {
+    return KS{valid ? (unsigned)k * 4u : INV_K};
   }
+  __device__ __forceinline__ unsigned off(const MS& m, const KS& k) const { return m.off + k.off; }
   __device__ __forceinline__ bool is_one(const MS&) const { return false; }
 };
 
 // Output gradient of a Conv2d, g[n][c][hw], read as P(k=(n,pos), m=c).
 struct ConvG {
   static constexpr int layout = MK;
+  static constexpr bool has_second = false;
   const float* p;
   int C, HW;
-  struct MS { const float* chan; bool valid; };
+  struct MS { unsigned off; };
   struct KS { unsigned off; };
+  __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc() const {
+    return make_rsrc(p);
+  }
   __device__ __forceinline__ MS mstate(int m) const {
-    return MS{m < C ? p + (size_t)m * HW : p, m < C};
+    return MS{m < C ? (unsigned)(m * HW) * 4u : INV_M};
   }
-  __device__ __forceinline__ KS kstate(int k) const {
+  __device__ __forceinline__ KS kstate(int k, bool valid) const {
     const int n = k / HW;
-    return KS{(unsigned)(n * C * HW + (k - n * HW))};
+    return KS{valid ? (unsigned)(n * C * HW + (k - n * HW)) * 4u : INV_K};
   }
-  __device__ __forceinline__ const float* addr(const MS& m, const KS& k, bool& ok) const {
-    ok = m.valid;
-    return m.chan + (m.valid ? k.off : 0u);
-  }
+  __device__ __forceinline__ unsigned off(const MS& m, const KS& k) const { return m.off + k.off; }
   __device__ __forceinline__ bool is_one(const MS&) const { return false; }
 };
 
@@ -92,16 +111,20 @@ struct ConvG {
 // (0 in the padding), plus an optional trailing row of ones (m == M-1).
 struct ConvA {
   static constexpr int layout = MK;
+  static constexpr bool has_second = false;
   const float* p;
   int C, H, W, KH, KW, SH, SW, PH, PW, DH, DW, OH, OW, M, ones;
-  // Per row m: the element offset of (c, kh, kw) and the two patch displacements
-  // packed as (dy << 16) | (dx & 0xffff) to keep the 16 row states of a thread in
-  // 32 registers.  dy = -32768 marks a row outside the operand (every bounds test
-  // then fails, image sizes are below 32768); dx = -32768 on top of that marks
-  // the row of ones.
+  // Per row m: the byte offset of (c, kh, kw) and the two patch displacements
+  // packed as (dy << 16) | (dx & 0xffff), so that the 8 row states of a thread
+  // take 16 registers.  dy = -32768 marks a row outside the operand (every bounds
+  // test then fails; image sizes are below 16384); dx = -32768 on top of that
+  // marks the row of ones.  An invalid k gets y0 = -2^20, failing the same test.
   struct MS { int off; int dydx; };
   struct KS { int off; int y0; int x0; };
   static __device__ __forceinline__ int pack(int dy, int dx) { return (dy << 16) | (dx & 0xffff); }
+  __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc() const {
+    return make_rsrc(p);
+  }
   __device__ __forceinline__ MS mstate(int m) const {
     MS s;
     if (m >= M) { s.off = 0; s.dydx = pack(-32768, 0); return s; }
@@ -112,25 +135,25 @@ struct ConvA {
     const int kw = rem - kh * KW;
     const int dy = kh * DH, dx = kw * DW;
     s.dydx = pack(dy, dx);
-    s.off = c * H * W + dy * W + dx;
+    s.off = (c * H * W + dy * W + dx) * 4;
     return s;
   }
-  __device__ __forceinline__ KS kstate(int k) const {
+  __device__ __forceinline__ KS kstate(int k, bool valid) const {
     const int n = k / (OH * OW);
     const int rem = k - n * OH * OW;
     const int oh = rem / OW;
     const int ow = rem - oh * OW;
     KS s;
-    s.y0 = oh * SH - PH;
+    s.y0 = valid ? oh * SH - PH : -(1 << 20);
     s.x0 = ow * SW - PW;
-    s.off = n * C * H * W + s.y0 * W + s.x0;
+    s.off = (n * C * H * W + s.y0 * W + s.x0) * 4;
     return s;
   }
-  __device__ __forceinline__ const float* addr(const MS& m, const KS& k, bool& ok) const {
+  __device__ __forceinline__ unsigned off(const MS& m, const KS& k) const {
     const int y = k.y0 + (m.dydx >> 16);
     const int x = k.x0 + (int)(short)(m.dydx & 0xffff);
-    ok = (unsigned)y < (unsigned)H && (unsigned)x < (unsigned)W;
-    return p + (ok ? (unsigned)(k.off + m.off) : 0u);
+    const bool ok = (unsigned)y < (unsigned)H && (unsigned)x < (unsigned)W;
+    return ok ? (unsigned)(k.off + m.off) : INV_M;
   }
   __device__ __forceinline__ bool is_one(const MS& m) const {
     return ones && m.dydx == pack(-32768, -32768);

@@ -176,8 +176,8 @@ int kfac_precondition_batched(int layers, const int* dG, const int* dA,
   std::vector<int> hb(layers);
   for (int l = 0; l < layers; ++l) {
     if (dG[l] <= 0 || dA[l] <= 0 || !Ginv[l] || !Ainv[l] || !gradW[l]) return KFAC_ERR_ARG;
-    if ((int64_t)dA[l] * dA[l] >= (int64_t)1 << 31 || (int64_t)dG[l] * dG[l] >= (int64_t)1 << 31 ||
-        (int64_t)dA[l] * dG[l] >= (int64_t)1 << 31)
+    if ((int64_t)dA[l] * dA[l] > (int64_t)1 << 28 || (int64_t)dG[l] * dG[l] > (int64_t)1 << 28 ||
+        (int64_t)dA[l] * dG[l] > (int64_t)1 << 28)
       return KFAC_ERR_ARG;
     hb[l] = gradb[l] != nullptr;
     if (hb[l] && dA[l] < 2) return KFAC_ERR_ARG;
@@ -199,8 +199,8 @@ int kfac_sample_batched(int layers, const int* dG, const int* dA, const float* c
   for (int l = 0; l < layers; ++l) {
     if (dG[l] <= 0 || dA[l] <= 0 || !U_G[l] || !U_A[l] || !noise[l] || !meanW[l] || !paramW[l])
       return KFAC_ERR_ARG;
-    if ((int64_t)dA[l] * dA[l] >= (int64_t)1 << 31 || (int64_t)dG[l] * dG[l] >= (int64_t)1 << 31 ||
-        (int64_t)dA[l] * dG[l] >= (int64_t)1 << 31)
+    if ((int64_t)dA[l] * dA[l] > (int64_t)1 << 28 || (int64_t)dG[l] * dG[l] > (int64_t)1 << 28 ||
+        (int64_t)dA[l] * dG[l] > (int64_t)1 << 28)
       return KFAC_ERR_ARG;
     hb[l] = paramb[l] != nullptr;
     if (hb[l] && (!meanb[l] || dA[l] < 2)) return KFAC_ERR_ARG;
