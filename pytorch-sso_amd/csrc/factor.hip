@@ -63,8 +63,11 @@ __global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void syrk_kernel(OP op,
   constexpr int TS = 64 * W;
   constexpr int KC = Cfg<W, W>::KC;
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  const int tile = blockIdx.x;
-  const int split = blockIdx.y;
+  // work item = (split, tile), tile fastest: the tiles of one split read the
+  // same rows of the input, so they are kept on one XCD
+  const int item = xcd_remap(blockIdx.y * ntiles + blockIdx.x, ntiles * splits);
+  const int tile = item % ntiles;
+  const int split = item / ntiles;
   int bi, bj;
   upper_tile(tile, T, bi, bj);
   const int kbeg = split * chunks_per_split * KC;

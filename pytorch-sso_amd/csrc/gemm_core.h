@@ -297,6 +297,16 @@ __device__ __forceinline__ void gemm_tile(const OPP& P, const OPQ& Q, int m0, in
   gemm_tile_cfg<2, 2>(P, Q, m0, n0, kbeg, kend, same, epi, smem);
 }
 
+// Workgroups are handed to the 8 XCDs round-robin in dispatch order, and each
+// XCD has its own L2.  This maps the dispatch index `id` of a 1-D problem of
+// `total` work items so that every XCD walks a CONTIGUOUS range of items:
+// neighbouring tiles, which share operand panels, then hit the same L2.
+__device__ __forceinline__ int xcd_remap(int id, int total) {
+  const int x = id & 7, q = total >> 3, r = total & 7;
+  const int base = x < r ? x * (q + 1) : r * (q + 1) + (x - r) * q;
+  return base + (id >> 3);
+}
+
 // tile index t (0-based, row-major over the upper triangle incl. diagonal of a
 // T x T block grid) -> (bi, bj), bi <= bj
 __device__ __forceinline__ void upper_tile(int t, int T, int& bi, int& bj) {

@@ -132,8 +132,9 @@ __device__ __forceinline__ void chol_inv_32(lds_f* S, lds_f* Yb, lds_f* scr, int
     }
     const float piv = row[c];
     if (!(piv > 0.f) && bad == 0) bad = row_base + c0 + c + 1;
-    const float d = sqrtf(piv);
-    const float rd = __builtin_amdgcn_rcpf(d);
+    // 1/sqrt in one instruction: the next step's pivot row waits on this chain
+    const float rd = __builtin_amdgcn_rsqf(piv);
+    const float d = piv * rd;
     const float f = a[c] * (rd * rd);
 #pragma unroll
     for (int i = c + 1; i < 32; ++i) a[i] = fmaf(-row[i], f, a[i]);   // A[i][j] -= U[c][i] U[c][j]
@@ -157,9 +158,16 @@ __device__ __forceinline__ void chol_inv_32(lds_f* S, lds_f* Yb, lds_f* scr, int
       row[4 * g + 2] = v.z;
       row[4 * g + 3] = v.w;
     }
-    float s = (j == i) ? 1.f : 0.f;
+    // y[i+1] was finished last: it enters the sum last, so that only one FMA and
+    // one multiply separate consecutive rows; two partial sums shorten the rest
+    float s0 = (j == i) ? 1.f : 0.f, s1 = 0.f;
 #pragma unroll
-    for (int k = i + 1; k < 32; ++k) s = fmaf(-row[k], y[k], s);
+    for (int k = 31; k > i + 1; k -= 2) {
+      s0 = fmaf(-row[k], y[k], s0);
+      if (k - 1 > i + 1) s1 = fmaf(-row[k - 1], y[k - 1], s1);
+    }
+    float s = s0 + s1;
+    if (i + 1 < 32) s = fmaf(-row[i + 1], y[i + 1], s);
     y[i] = s * __builtin_amdgcn_rcpf(row[i]);
   }
   if (lane < 32) {
