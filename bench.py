@@ -1,7 +1,7 @@
 """K-FAC step benchmark on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50|alexnet_fc|convnet|mlp]
-                    [--no-cpu-baseline]
+                    [--no-cpu-baseline] [--copy-calibration]
 
 A "step" is one pass of the K-FAC hot path over one batch of synthetic input,
 driven through the public torchsso API: for every layer the two Kronecker
@@ -181,8 +181,10 @@ class LayerSet(object):
         return n
 
     # -- the three phases of a step -----------------------------------------
-    def build_factors(self):
+    def build_factors(self, kinds=('conv', 'linear', 'bn')):
         for s, m, c, xin, g in zip(self.specs, self.model, self.curvs, self.inputs, self.gouts):
+            if s['kind'] not in kinds:
+                continue
             if s['kind'] == 'bn':
                 # forward hook: sum_hw xhat^2 from the layer output; backward hook: the rest
                 c.forward_postprocess(m, (xin,), xin)
@@ -202,27 +204,31 @@ class LayerSet(object):
         self.opt.step()
 
     def timed_phases(self, iters):
-        """Average ms of factor build / EMA+inversion / precondition+update."""
+        """Average ms of: Kronecker factor build (the syrk kernels only) / BatchNorm
+        diagonal curvature / EMA / inversion / precondition+update, bracketed by HIP
+        events on the stream the kernels are launched on (torch's current stream)."""
         torch = self.torch
         from torchsso.curv import curvature as _curv
         ev = lambda: torch.cuda.Event(enable_timing=True)
-        acc = [0., 0., 0., 0.]
+        acc = [0.] * 5
         groups = self.opt.param_groups
         for _ in range(iters):
             self.restore_grads()
-            e = [ev() for _ in range(5)]
+            e = [ev() for _ in range(6)]
             e[0].record()
-            self.build_factors()
+            self.build_factors(('conv', 'linear'))
             e[1].record()
-            _curv.update_ema_all(self.curvs)
+            self.build_factors(('bn',))
             e[2].record()
-            _curv.update_inv_all(self.curvs)
+            _curv.update_ema_all(self.curvs)
             e[3].record()
+            _curv.update_inv_all(self.curvs)
+            e[4].record()
             _curv.precondition_all([(g['curv'], g['params']) for g in groups])
             self.opt._fused_update(groups, 'params')
-            e[4].record()
+            e[5].record()
             torch.cuda.synchronize()
-            for i in range(4):
+            for i in range(5):
                 acc[i] += e[i].elapsed_time(e[i + 1])
         return [a / iters for a in acc]
 
@@ -341,6 +347,9 @@ def main():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--workload', default='resnet50', choices=sorted(WORKLOADS))
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--copy-calibration', action='store_true',
+                    help='also run a plain 1 GiB device copy (reference for rocprofv3 --pmc '
+                         'FETCH_SIZE / WRITE_SIZE readings)')
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
         print('bench.py measures the one-GPU share of the K-FAC step; --gpus must be 1 '
@@ -359,7 +368,14 @@ def main():
         print('no HIP device visible', file=sys.stderr)
         sys.exit(1)
     ms, ev_ms, phases, resident, not_spd = run_gpu(args, specs, batch)
-    f_ms, ema_ms, inv_ms, pre_ms = phases
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device='cuda:0').normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    f_ms, bn_ms, ema_ms, inv_ms, pre_ms = phases
     total_flops = work['factor'] + work['inverse'] + work['precondition']
 
     out = {
@@ -374,7 +390,8 @@ def main():
                    'inputs_resident_GB': round(resident / 1e9, 3)},
         'tflops': round(total_flops / (ms * 1e-3) / 1e12, 2),
         'algorithmic_gflop': {k: round(v / 1e9, 1) for k, v in work.items() if not k.endswith('bytes')},
-        'phases_ms': {'factor': round(f_ms, 4), 'ema': round(ema_ms, 4),
+        'phases_ms': {'factor': round(f_ms, 4), 'batchnorm_diag': round(bn_ms, 4),
+                      'ema': round(ema_ms, 4),
                       'invert': round(inv_ms, 4), 'precondition_update': round(pre_ms, 4)},
         'phases_tflops': {'factor': round(work['factor'] / f_ms / 1e9, 2),
                           'invert': round(work['inverse'] / inv_ms / 1e9, 2),

@@ -357,7 +357,7 @@ __global__ __launch_bounds__(NTHREADS) void potrf_trail_kernel(const MatDesc* ta
     // all remaining rows: walk the upper triangle of the (T - row_lo)^2 block grid
     const int Tr = T - row_lo;
     if ((int)blockIdx.x >= Tr * (Tr + 1) / 2) return;
-    upper_tile(blockIdx.x, Tr, bi, bj);
+    upper_tile(xcd_remap(blockIdx.x, Tr * (Tr + 1) / 2), Tr, bi, bj);
     bi += row_lo;
     bj += row_lo;
   } else {
@@ -396,7 +396,7 @@ __device__ __forceinline__ MergeTile merge_tile(const MatDesc& m, int depth) {
   const int T = m.T;
   if (T < 2 || (int)blockIdx.x >= (T - 1) * T / 2) return t;
   int bi, bj;
-  upper_tile(blockIdx.x, T - 1, bi, bj);
+  upper_tile(xcd_remap(blockIdx.x, (T - 1) * T / 2), T - 1, bi, bj);
   bj += 1;
   const int P = seg_of(bi, depth, T);
   if (seg_of(bj, depth, T) != P) return t;
@@ -448,7 +448,7 @@ __global__ __launch_bounds__(NTHREADS) void lauum_kernel(const MatDesc* table) {
   const int ntiles = m.T * (m.T + 1) / 2;
   if ((int)blockIdx.x >= ntiles) return;
   int bi, bj;
-  upper_tile(blockIdx.x, m.T, bi, bj);
+  upper_tile(xcd_remap(blockIdx.x, ntiles), m.T, bi, bj);   // a tile row per L2
   const int n = m.n;
   DenseMK P{m.Y, n, n};
   EpiStore epi{m.U, n, n, n, 1.f, 0.f, bi != bj};

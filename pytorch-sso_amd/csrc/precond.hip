@@ -66,7 +66,8 @@ __global__ __launch_bounds__(NTHREADS) void precond_first_kernel(const LayerDesc
   const LayerDesc m = table[blockIdx.y];
   const int ta = tiles128(m.dA), tg = tiles128(m.dG);
   if ((int)blockIdx.x >= ta * tg) return;
-  const int bi = blockIdx.x / tg, bj = blockIdx.x - bi * tg;   // bi over dA, bj over dG
+  const int item = xcd_remap(blockIdx.x, ta * tg);
+  const int bi = item / tg, bj = item - bi * tg;   // bi over dA, bj over dG
   EpiStore epi{m.Tt, m.dG, m.dA, m.dG, 1.f, 0.f, false};
   if (SAMPLE) {
     // noise E is a plain dG x dA matrix; U_G is upper triangular: L(k, i) = U_G[i][k], k >= i
@@ -86,7 +87,8 @@ __global__ __launch_bounds__(NTHREADS) void precond_second_kernel(const LayerDes
   const LayerDesc m = table[blockIdx.y];
   const int ta = tiles128(m.dA), tg = tiles128(m.dG);
   if ((int)blockIdx.x >= ta * tg) return;
-  const int bi = blockIdx.x / ta, bj = blockIdx.x - bi * ta;   // bi over dG, bj over dA
+  const int item = xcd_remap(blockIdx.x, ta * tg);
+  const int bi = item / ta, bj = item - bi * ta;   // bi over dG, bj over dA
   DenseKM P{m.Tt, nullptr, m.dG, m.dG, 0};
   DenseKM Q{m.R, nullptr, m.dA, m.dA, 0};
   EpiSplit epi{m.outW, m.outb, m.meanW, m.meanb, m.dG, m.dA, m.dAw, m.scale};
