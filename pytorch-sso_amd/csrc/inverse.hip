@@ -314,11 +314,24 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
   }
   if (nq > 2) tri_pair(S, Yb, Wt, 0, 64, 0, 4);
 
-  for (int e = t; e < DB * DB; e += 256) {
-    const int i = e >> 7, j = e & 127;
-    if (i < nb && j < nb) {
-      m.U[(size_t)(r0 + i) * n + r0 + j] = S[i * DLD + j];
-      m.Y[(size_t)(r0 + i) * n + r0 + j] = Yb[i * DLD + j];
+  // write U_pp and Y_pp back, 16 LDS reads in flight per thread
+  for (int e0 = 0; e0 < DB * DB; e0 += 256 * 16) {
+    float u[16], y[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const int e = e0 + k * 256 + t;
+      const int i = e >> 7, j = e & 127;
+      u[k] = S[i * DLD + j];
+      y[k] = Yb[i * DLD + j];
+    }
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const int e = e0 + k * 256 + t;
+      const int i = e >> 7, j = e & 127;
+      if (i < nb && j < nb) {
+        m.U[(size_t)(r0 + i) * n + r0 + j] = u[k];
+        m.Y[(size_t)(r0 + i) * n + r0 + j] = y[k];
+      }
     }
   }
 }
