@@ -27,6 +27,10 @@ sys.path.insert(0, ROOT)
 
 METRIC = 'K-FAC step ms (factor+invert+precondition) & fp32 MFMA TFLOP/s, 1 MI355X'
 PEAK_FP32_MFMA_TFLOPS = 157.3
+# HBM bytes per syrk_kernel launch, averaged over the 108 launches of a resnet50 step, from two
+# rocprofv3 --pmc runs (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration with a 1 GiB copy):
+# 39.5 MB read + 22.5 MB written.
+RESNET50_SYRK_TRAFFIC_BYTES = 62.0e6
 
 
 # ---------------------------------------------------------------------------
@@ -401,7 +405,7 @@ def main():
                      'achieved': round(work['factor'] / f_ms / 1e9, 2),
                      'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
                      'frac': round(work['factor'] / f_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4),
-                     'traffic': None},
+                     'traffic': RESNET50_SYRK_TRAFFIC_BYTES if args.workload == 'resnet50' else None},
     }
     if not args.no_cpu_baseline:
         cpu_ms, cores, sample = run_cpu_baseline(specs, batch)
