@@ -183,6 +183,20 @@ int kfac_sgd_update_batched(int count, const int64_t* numel, float* const* param
                             const float* lr, const float* momentum, const float* weight_decay,
                             void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- Fisher weighting ---------------------------------------------------- */
+
+/* out[r][i] = x[r][i] * (use_sqrt ? sqrt(w[r]) : w[r]) for `rows` rows of `len`
+ * contiguous elements (out may equal x).  The true-Fisher curvatures weigh each
+ * sample's output gradient by a probability: G = sum_n prob[n] g_n g_n^T
+ * (torchsso/curv/fisher/linear.py:47-54, fisher/conv.py:61-70 of the reference,
+ * pg = g * prob then einsum(pg, g)).  With use_sqrt the weighted gradient
+ * sqrt(prob) * g can go through the symmetric factor kernels unchanged, and the
+ * sum over classes / MC samples (Fisher.accumulate_cov, fisher/__init__.py:24-28)
+ * is their beta = 1 epilogue.  Without it: prob * (sum_hw g^2) of
+ * fisher/batchnorm.py:18-21. */
+int kfac_scale_rows(const float* x, const float* w, int64_t rows, int64_t len, int use_sqrt,
+                    float* out, void* stream);
+
 /* ---- BatchNorm diagonal curvature -------------------------------------- */
 
 /* out[row] = sum_i ((x[row*len + i] - shift[c]) / scale[c])^2, c = row % channels;

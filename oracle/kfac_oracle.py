@@ -22,6 +22,8 @@ which retypes the formula):
                        2x2 by hand
   precondition         Kronecker identity via torch.kron
   bn_diag              per-sample gradient identity through autograd
+  fisher_*             prob == 1 reduces to the Cov factor; the exact sum over classes at the
+                       logits layer equals mean_n(diag(p_n) - p_n p_n^T) (closed form)
   cholesky_upper       U^T U == X, U upper, diag > 0
   sample               injected-noise Kronecker identity
   kfac_step / vi_step  golden vectors written by the reference itself
@@ -108,6 +110,38 @@ def bn_diag(xhat, g, bias=True, dtype=torch.float32, scale_by_batch=True):
     if scale_by_batch:
         out = [o * float(n ** 2) for o in out]
     return out
+
+
+def fisher_linear_g(g, prob, dtype=torch.float32, scale_by_batch=True):
+    """One weighted pass of KronFisherLinear: G = (prob * g)^T g / n, then *= n^2
+    (torchsso/curv/fisher/linear.py:47-54; curvature.py:154-155).  The passes of one
+    step are summed (Fisher.accumulate_cov, fisher/__init__.py:24-28)."""
+    g = g.to(dtype)
+    n = g.shape[0]
+    G = ((g * prob.to(dtype).reshape(n, 1)).t() @ g) / n
+    return G * float(n ** 2) if scale_by_batch else G
+
+
+def fisher_conv_g(g, prob, dtype=torch.float32, scale_by_batch=True):
+    """One weighted pass of KronFisherConv2d (torchsso/curv/fisher/conv.py:61-70)."""
+    g = g.to(dtype)
+    n, c, h, w = g.shape
+    pm = (g * prob.to(dtype).reshape(n, 1, 1, 1)).transpose(0, 1).reshape(c, -1)
+    m = g.transpose(0, 1).reshape(c, -1)
+    G = (pm @ m.t()) / (n * h * w)
+    return G * float(n ** 2) if scale_by_batch else G
+
+
+def fisher_bn_diag(xhat, g, prob, bias=True, dtype=torch.float32, scale_by_batch=True):
+    """One weighted pass of DiagFisherBatchNorm2d (torchsso/curv/fisher/batchnorm.py:11-30)."""
+    xhat, g = xhat.to(dtype), g.to(dtype)
+    n = g.shape[0]
+    gg = (g * prob.to(dtype).reshape(n, 1, 1, 1) * g).sum(dim=(2, 3))
+    in_in = (xhat * xhat).sum(dim=(2, 3))
+    out = [(in_in * gg).mean(dim=0)]
+    if bias:
+        out.append(gg.mean(dim=0))
+    return [o * float(n ** 2) for o in out] if scale_by_batch else out
 
 
 def bn_restore_input(out, weight, bias):

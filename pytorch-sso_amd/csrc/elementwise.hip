@@ -221,6 +221,17 @@ __global__ __launch_bounds__(256) void rowsq_kernel(const float* x, const float*
   if (lane == 0 && row < rows) out[row] = red[threadIdx.x];
 }
 
+// out[r][i] = x[r][i] * (use_sqrt ? sqrt(w[r]) : w[r]),  rows of length len
+__global__ __launch_bounds__(256) void scale_rows_kernel(const float* x, const float* w, long rows,
+                                                         long len, int use_sqrt, float* out) {
+  const long total = rows * len;
+  const long stride = (long)gridDim.x * 256;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+    const float s = w[i / len];
+    out[i] = x[i] * (use_sqrt ? sqrtf(s) : s);
+  }
+}
+
 // w_curv[c] = alpha * sum_n sx[n][c] * sg[n][c] ; b_curv[c] = alpha * sum_n sg[n][c]
 __global__ void bn_combine_kernel(const float* sx, const float* sg, int N, int C, float alpha,
                                   float* w_curv, float* b_curv) {
@@ -306,6 +317,17 @@ int kfac_rowsq_sum(const float* x, int64_t rows, int channels, int len, const fl
   else
     hipLaunchKernelGGL(rowsq_kernel<1>, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, x,
                        scale, shift, (long)rows, channels, len, out);
+  return launch_status();
+}
+
+int kfac_scale_rows(const float* x, const float* w, int64_t rows, int64_t len, int use_sqrt,
+                    float* out, void* stream) {
+  if (!x || !w || !out || rows <= 0 || len <= 0) return KFAC_ERR_ARG;
+  const long total = (long)rows * len;
+  long blocks = (total + 1023) / 1024;
+  if (blocks > 8192) blocks = 8192;
+  hipLaunchKernelGGL(scale_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     x, w, (long)rows, (long)len, use_sqrt, out);
   return launch_status();
 }
 

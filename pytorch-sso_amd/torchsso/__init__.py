@@ -13,6 +13,9 @@ from torchsso.curv.cov.linear import CovLinear, KronCovLinear  # NOQA
 from torchsso.curv.cov.conv import CovConv2d, KronCovConv2d  # NOQA
 from torchsso.curv.cov.batchnorm import CovBatchNorm1d, DiagCovBatchNorm1d, CovBatchNorm2d, DiagCovBatchNorm2d  # NOQA
 
+from torchsso.curv.fisher import Fisher, get_closure_for_fisher  # NOQA
+from torchsso.curv.fisher import KronFisherLinear, KronFisherConv2d, DiagFisherBatchNorm2d  # NOQA
+
 from torchsso import optim  # NOQA
 
 __version__ = '0.1.0'

@@ -63,6 +63,7 @@ _SIGNATURES = {
                                                c_ptr, c_size, c_ptr]),
     'kfac_sgd_update_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
                                         c_ptr, c_size, c_ptr]),
+    'kfac_scale_rows': (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_int, c_ptr, c_ptr]),
     'kfac_rowsq_sum': (c_int, [c_ptr, c_i64, c_int, c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     'kfac_bn_diag_combine': (c_int, [c_ptr, c_ptr, c_int, c_int, c_f32, c_ptr, c_ptr, c_ptr]),
 }

@@ -328,3 +328,18 @@ def bn_diag_combine(sx, sg, alpha, bias):
                                   _hip.stream_ptr(sx.device))
     _hip.check(st, 'kfac_bn_diag_combine')
     return w, b
+
+
+def scale_rows(x, w, use_sqrt):
+    """x[r] * (sqrt(w[r]) if use_sqrt else w[r]) for every row r = index along dim 0 (new tensor)."""
+    lib = _hip.load()
+    x = x.contiguous()
+    rows = x.shape[0]
+    if w.numel() != rows:
+        raise _hip.KfacHipError('scale_rows: %d weights for %d rows' % (w.numel(), rows))
+    out = torch.empty_like(x)
+    st = lib.kfac_scale_rows(_hip.dev_ptr(x, 'input'), _hip.dev_ptr(w.contiguous(), 'weights'), rows,
+                             x.numel() // rows, int(bool(use_sqrt)), out.data_ptr(),
+                             _hip.stream_ptr(x.device))
+    _hip.check(st, 'kfac_scale_rows')
+    return out

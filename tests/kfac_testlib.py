@@ -251,3 +251,11 @@ class OracleOps(object):
         w = alpha * (sx * sg).sum(dim=0)
         b = alpha * sg.sum(dim=0) if bias else None
         return w, b
+
+
+def _oracle_scale_rows(self, x, w, use_sqrt):
+    s = w.reshape((-1,) + (1,) * (x.dim() - 1))
+    return x * (s.sqrt() if use_sqrt else s)
+
+
+OracleOps.scale_rows = _oracle_scale_rows

@@ -223,3 +223,68 @@ def test_config5_noisy_kfac_step_runs_and_samples():
                         g['std_scale'], torch.float64)
         assert O.rel_fro(g['params'][0].data, w) < TOL
         assert O.rel_fro(g['params'][1].data, b) < TOL
+
+
+def test_fisher_closure_on_gpu_matches_closed_form():
+    """Exact Fisher through SecondOrderOptimizer(curv_type='Fisher'): the G factor of
+    the logits layer equals mean_n(diag(p_n) - p_n p_n^T); a conv + BatchNorm front
+    end exercises the weighted conv G and BatchNorm kernels against the oracle."""
+    import torchsso
+    dev = torch.device('cuda:0')
+    torch.manual_seed(2)
+
+    class Net(nn.Module):
+        num_classes = 5
+
+        def __init__(self):
+            super().__init__()
+            self.c1 = nn.Conv2d(3, 6, 3, padding=1)
+            self.bn = nn.BatchNorm2d(6)
+            self.fc = nn.Linear(6 * 4 * 4, 5)
+
+        def forward(self, x):
+            return self.fc(F.relu(self.bn(self.c1(x))).flatten(1))
+
+    model = Net().to(dev)
+    x = torch.randn(12, 3, 4, 4, device=dev)
+    y = torch.randint(0, 5, (12,), device=dev)
+    opt = torchsso.optim.SecondOrderOptimizer(
+        model, 'Fisher', {'Conv2d': 'Kron', 'Linear': 'Kron', 'BatchNorm2d': 'Diag'},
+        {'damping': 1e-3, 'ema_decay': 1.}, lr=0.0)
+    names = [type(g['curv']).__name__ for g in opt.param_groups]
+    assert names == ['KronFisherConv2d', 'DiagFisherBatchNorm2d', 'KronFisherLinear']
+    seen = {}
+
+    def closure():
+        ret = torchsso.get_closure_for_fisher(opt, model, x, y)()
+        seen['G'] = [[d.clone() for d in g['curv'].data] for g in opt.param_groups]
+        return ret
+    loss, out = opt.step(closure=closure)
+    p = torch.softmax(out.detach().double(), 1).cpu()
+    closed = sum(torch.diag(p[i]) - torch.outer(p[i], p[i]) for i in range(12)) / 12
+    assert O.rel_fro(seen['G'][2][1], closed) < TOL
+    # conv G and BatchNorm data against the oracle, from per-class output gradients
+    with torch.no_grad():
+        pass
+    model2 = Net().to(dev)
+    model2.load_state_dict(model.state_dict())
+    feats = {}
+    h1 = model2.c1.register_forward_hook(lambda m, i, o: feats.__setitem__('c1', o))
+    h2 = model2.bn.register_forward_hook(lambda m, i, o: feats.__setitem__('bn', o))
+    out2 = model2(x)
+    Gc = torch.zeros(6, 6, dtype=torch.float64)
+    bnw = torch.zeros(6, dtype=torch.float64)
+    bnb = torch.zeros(6, dtype=torch.float64)
+    xhat = O.bn_restore_input(feats['bn'].detach().double().cpu(), model2.bn.weight.detach().double().cpu(),
+                              model2.bn.bias.detach().double().cpu())
+    for k in range(5):
+        gc, gb = torch.autograd.grad(F.cross_entropy(out2, torch.full_like(y, k)),
+                                     [feats['c1'], feats['bn']], retain_graph=True)
+        Gc += O.fisher_conv_g(gc.cpu(), p[:, k], torch.float64)
+        d = O.fisher_bn_diag(xhat, gb.cpu(), p[:, k], True, torch.float64)
+        bnw += d[0]
+        bnb += d[1]
+    h1.remove()
+    h2.remove()
+    assert O.rel_fro(seen['G'][0][1], Gc) < TOL
+    assert O.rel_fro(seen['G'][1][0], bnw) < TOL and O.rel_fro(seen['G'][1][1], bnb) < TOL

@@ -273,3 +273,46 @@ def test_factor_linearity_at_full_size(ops, dev):
     u = torch.nn.functional.unfold(x[:1].double(), 3, padding=1)[0]
     one = ops.factor_conv_a(x[:1].contiguous(), (3, 3), (1, 1), (1, 1), (1, 1), False, 1.0)
     assert O.rel_fro(one, u @ u.t()) < TOL
+
+
+# ---- Fisher weighting ---------------------------------------------------------------
+
+def test_fisher_weighted_factors(ops, dev):
+    torch.manual_seed(7)
+    n, f = 96, 130
+    g = torch.randn(n, f) * 1e-2
+    passes = [torch.rand(n) for _ in range(3)]
+    acc = None
+    ref = torch.zeros(f, f, dtype=D)
+    for k, prob in enumerate(passes):
+        pg = ops.scale_rows(g.to(dev), prob.to(dev), True)
+        acc = ops.factor_linear(pg, False, float(n), out=acc, beta=0. if k == 0 else 1.)
+        ref += O.fisher_linear_g(g, prob, D)
+    assert O.rel_fro(acc, ref) < TOL
+    g4 = torch.randn(8, 70, 5, 6) * 1e-2
+    prob = torch.rand(8)
+    pg = ops.scale_rows(g4.to(dev), prob.to(dev), True)
+    G = ops.factor_conv_g(pg, 8.0 / 30)
+    assert O.rel_fro(G, O.fisher_conv_g(g4, prob, D)) < TOL
+    # BatchNorm: prob * sum_hw g^2
+    out = torch.randn(8, 70, 5, 6)
+    w, b = torch.rand(70) + 0.5, torch.randn(70)
+    sx = ops.rowsq_sum(out.to(dev), 70, w.to(dev), b.to(dev))
+    sg = ops.scale_rows(ops.rowsq_sum(g4.to(dev), 70), prob.to(dev), False)
+    wc, bc = ops.bn_diag_combine(sx, sg, 8.0, True)
+    ref = O.fisher_bn_diag(O.bn_restore_input(out.double(), w.double(), b.double()), g4, prob, True, D)
+    assert O.rel_fro(wc, ref[0]) < TOL and O.rel_fro(bc, ref[1]) < TOL
+
+
+def test_factor_input_above_one_gib_is_consumed_in_slices(ops, dev):
+    """1.2 GB of rows: the entry point walks them in slices of at most 1 GiB that
+    accumulate into the factor; checked by linearity against two half-size calls."""
+    rows, f = 300000, 1024
+    g = torch.Generator(device='cpu').manual_seed(3)
+    x = torch.randn(rows, f, generator=g).to(dev)
+    full = ops.factor_linear(x, True, 1.0 / rows)
+    half = rows // 2
+    a = ops.factor_linear(x[:half].contiguous(), True, 1.0 / rows)
+    b = ops.factor_linear(x[half:].contiguous(), True, 1.0 / rows)
+    assert O.rel_fro(full, a.double() + b.double()) < 1e-5
+    assert abs(full[-1, -1].item() - 1.0) < 1e-5

@@ -178,3 +178,52 @@ def test_product_has_no_cpu_path():
     acc = torchsso.utils.TensorAccumulator()
     with pytest.raises(AssertionError):
         acc.update([1.0, 2.0])
+
+
+def test_fisher_closure_exact_and_mc(oracle_ops):
+    """Exact Fisher: the G factor of the logits layer equals mean_n(diag(p) - p p^T);
+    every layer (also the first) gets a G factor; gradients are those of the true
+    loss.  MC Fisher with many samples approaches the exact one."""
+    torch.manual_seed(5)
+
+    class Net(nn.Module):
+        num_classes = 4
+
+        def __init__(self):
+            super().__init__()
+            self.l1 = nn.Linear(6, 5)
+            self.l2 = nn.Linear(5, 4)
+
+        def forward(self, x):
+            return self.l2(F.relu(self.l1(x)))
+
+    model = Net()
+    x, y = torch.randn(10, 6), torch.randint(0, 4, (10,))
+    import copy
+    plain = copy.deepcopy(model)      # no curvature hooks on this one
+    opt = torchsso.optim.SecondOrderOptimizer(model, 'Fisher', {'Linear': 'Kron'},
+                                              {'damping': 1e-3, 'ema_decay': 1.}, lr=0.0)
+    assert type(opt.param_groups[0]['curv']).__name__ == 'KronFisherLinear'
+    ref_grads = torch.autograd.grad(F.cross_entropy(plain(x), y), list(plain.parameters()))
+    p = torch.softmax(plain(x), 1).detach()
+    closed = sum(torch.diag(p[i]) - torch.outer(p[i], p[i]) for i in range(10)) / 10
+    raw = {}
+
+    def closure():
+        ret = torchsso.get_closure_for_fisher(opt, model, x, y)()
+        raw['g'] = [q.grad.clone() for q in model.parameters()]
+        raw['G'] = [g['curv'].G.clone() for g in opt.param_groups]
+        return ret
+    opt.step(closure=closure)
+    for got, ref in zip(raw['g'], ref_grads):
+        assert torch.allclose(got, ref, atol=1e-6)
+    assert torch.allclose(raw['G'][1], closed, atol=1e-5)
+    assert raw['G'][0].abs().sum() > 0 and all(q.requires_grad for q in model.parameters())
+    exact_first = raw['G'][0]
+    torch.manual_seed(0)
+    mc = torchsso.get_closure_for_fisher(opt, model, x, y, approx_type='mc', num_mc=4000)
+    mc()
+    assert torch.allclose(opt.param_groups[1]['curv'].G, closed, atol=0.02)
+    assert (opt.param_groups[0]['curv'].G - exact_first).norm() / exact_first.norm() < 0.15
+    with pytest.raises(ValueError):
+        torchsso.get_closure_for_fisher(opt, model, x, y, approx_type='bogus')()

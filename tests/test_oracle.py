@@ -292,3 +292,28 @@ def test_oracle_vi_accumulation_matches_reference():
     hist = T.oracle_kfac_run(model, torch.from_numpy(gold['x']), torch.from_numpy(gold['y']), 2,
                              lr=0.05, damping=1e-3, ema_decay=0.95, momentum=0.9, num_mc_samples=3)
     T.compare_with_golden(hist, gold, 2e-4)
+
+
+# ---- Fisher weighting ---------------------------------------------------------
+
+def test_fisher_factors_reduce_to_cov_and_match_the_presoftmax_closed_form():
+    torch.manual_seed(12)
+    n, c = 6, 4
+    g = torch.randn(n, c, dtype=D)
+    ones = torch.ones(n, dtype=D)
+    assert torch.allclose(O.fisher_linear_g(g, ones, D), O.factor_linear_g(g, D), atol=1e-12)
+    g4 = torch.randn(n, c, 3, 3, dtype=D)
+    assert torch.allclose(O.fisher_conv_g(g4, ones, D), O.factor_conv_g(g4, D), atol=1e-12)
+    xh = torch.randn(n, c, 3, 3, dtype=D)
+    a, b = O.fisher_bn_diag(xh, g4, ones, True, D), O.bn_diag(xh, g4, True, D)
+    assert all(torch.allclose(u, v, atol=1e-12) for u, v in zip(a, b))
+    # exact Fisher at the logits: sum over classes of p_c * grad_c grad_c^T, with
+    # grad_c = (p - e_c)/n the gradient of the mean cross entropy for label c
+    logits = torch.randn(n, c, dtype=D)
+    p = torch.softmax(logits, 1)
+    G = torch.zeros(c, c, dtype=D)
+    for k in range(c):
+        grad_k = (p - torch.eye(c, dtype=D)[k]) / n
+        G += O.fisher_linear_g(grad_k, p[:, k], D)
+    closed = sum(torch.diag(p[i]) - torch.outer(p[i], p[i]) for i in range(n)) / n
+    assert torch.allclose(G, closed, atol=1e-12)
