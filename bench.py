@@ -157,7 +157,7 @@ class LayerSet(object):
             {'damping': 1e-3, 'ema_decay': 0.95}, lr=1e-3, momentum=0.9)
         self.curvs = [g['curv'] for g in self.opt.param_groups]
         # synthetic layer inputs / output gradients / raw parameter gradients
-        self.inputs, self.gouts, self.raw_grads = [], [], []
+        self.inputs, self.gouts = [], []
         for s, m in zip(specs, self.model):
             if s['kind'] == 'conv':
                 xin = torch.randn(batch, s['cin'], s['hin'], s['hin'], device=device)
@@ -173,10 +173,18 @@ class LayerSet(object):
                 g = torch.randn(batch, s['c'], s['h'], s['h'], device=device) * 1e-2
             self.inputs.append(xin)
             self.gouts.append(g)
-            self.raw_grads.append([torch.randn_like(p) * 1e-2 for p in m.parameters()])
-        for m, raws in zip(self.model, self.raw_grads):
-            for p, r in zip(m.parameters(), raws):
-                p.grad = r.clone()
+        # raw parameter gradients: every p.grad is a 256-byte aligned view into one
+        # flat buffer, so that handing the step fresh gradients (what a backward pass
+        # would do) is one device copy
+        params = [p for m in self.model for p in m.parameters()]
+        offs, total = [], 0
+        for p in params:
+            offs.append(total)
+            total += (p.numel() + 63) // 64 * 64
+        self.flat_raw = torch.randn(total, device=device) * 1e-2
+        self.flat_grad = self.flat_raw.clone()
+        for p, o in zip(params, offs):
+            p.grad = self.flat_grad[o:o + p.numel()].view_as(p)
 
     def bytes_resident(self):
         n = 0
@@ -198,9 +206,7 @@ class LayerSet(object):
                 c.update_in_backward(g)
 
     def restore_grads(self):
-        for m, raws in zip(self.model, self.raw_grads):
-            for p, r in zip(m.parameters(), raws):
-                p.grad.copy_(r)
+        self.flat_grad.copy_(self.flat_raw)
 
     def step(self):
         self.restore_grads()

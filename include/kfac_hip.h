@@ -57,9 +57,18 @@ int kfac_factor_linear(const float* x, int64_t rows, int f, int64_t ldx, int add
                        float alpha, float beta, float* C,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* Scratch needed by kfac_factor_conv_a for this geometry (it may exceed
+ * kfac_factor_workspace_bytes of the same factor). */
+size_t kfac_factor_conv_a_workspace_bytes(int n, int c, int H, int W, int kh, int kw,
+                                          int sh, int sw, int ph, int pw, int dh, int dw,
+                                          int add_bias);
+
 /* C = alpha * M M^T + beta * C with M = im2col(x) as [c*kh*kw (+1), n*oh*ow],
- * row order (c, kh, kw), ones ROW last; the patches are gathered tile by tile
- * into LDS and never written to memory.  x is [n, c, H, W].
+ * row order (c, kh, kw), ones ROW last; M is never written to memory.
+ * x is [n, c, H, W].  Two kernels, same result: in general the patches are
+ * gathered tile by tile into LDS; for a stride-1, bias-free layer with 2..9
+ * kernel taps the blocks of C that share a tap displacement are built from one
+ * spatial correlation of the input with itself (3.4x fewer flops for 3x3).
  * Replaces F.unfold + transpose/reshape + cat + einsum('ik,jk->ij') + div(n) in
  * torchsso/curv/cov/conv.py:47-67 (alpha = 1/n).  groups are ignored, as there. */
 int kfac_factor_conv_a(const float* x, int n, int c, int H, int W,

@@ -22,6 +22,16 @@ bool enable_large_lds(const void* kernel, int bytes);
                          __VA_ARGS__);                                                       \
   } while (0)
 
+// A factor of a stride-1, bias-free Conv2d by spatial correlations
+// (factor_conv_taps.hip).  conv_a_taps returns -1 when the geometry is not
+// covered; the caller then uses the im2col kernel.
+bool conv_a_taps_applicable(int c, int kh, int kw, int sh, int sw, int add_bias);
+size_t conv_a_taps_workspace(int n, int c, int H, int W, int kh, int kw, int ph, int pw, int dh,
+                             int dw);
+int conv_a_taps(const float* x, int n, int c, int H, int W, int kh, int kw, int ph, int pw, int dh,
+                int dw, float alpha, float beta, float* A, void* workspace, size_t workspace_bytes,
+                hipStream_t stream);
+
 inline int launch_status() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? KFAC_OK : KFAC_ERR_LAUNCH;

@@ -193,6 +193,30 @@ static int64_t slice_len(int64_t total, int64_t elems_per_unit) {
   return max_units < 1 ? 0 : (total < max_units ? total : max_units);
 }
 
+size_t kfac_factor_conv_a_workspace_bytes(int n, int c, int H, int W, int kh, int kw, int sh,
+                                          int sw, int ph, int pw, int dh, int dw, int add_bias) {
+  if (n <= 0 || c <= 0 || H <= 0 || W <= 0 || kh <= 0 || kw <= 0 || sh <= 0 || sw <= 0 ||
+      ph < 0 || pw < 0 || dh <= 0 || dw <= 0)
+    return 0;
+  const int OH = (H + 2 * ph - dh * (kh - 1) - 1) / sh + 1;
+  const int OW = (W + 2 * pw - dw * (kw - 1) - 1) / sw + 1;
+  if (OH <= 0 || OW <= 0) return 0;
+  const int64_t image = (int64_t)c * H * W;
+  const int64_t step = slice_len(n, image);
+  if (step == 0) return 0;
+  const int d = c * kh * kw + (add_bias ? 1 : 0);
+  size_t need = kfac_factor_workspace_bytes(d, step * OH * OW);
+  if (conv_a_taps_applicable(c, kh, kw, sh, sw, add_bias)) {
+    const size_t t = conv_a_taps_workspace((int)step, c, H, W, kh, kw, ph, pw, dh, dw);
+    if (t > need) need = t;
+    if (n % step) {
+      const size_t t2 = conv_a_taps_workspace((int)(n % step), c, H, W, kh, kw, ph, pw, dh, dw);
+      if (t2 > need) need = t2;
+    }
+  }
+  return need;
+}
+
 int kfac_factor_linear(const float* x, int64_t rows, int f, int64_t ldx, int add_bias,
                        float alpha, float beta, float* C, void* workspace,
                        size_t workspace_bytes, void* stream) {
@@ -229,9 +253,24 @@ int kfac_factor_conv_a(const float* x, int n, int c, int H, int W, int kh, int k
   if (step == 0) return KFAC_ERR_ARG;
   for (int64_t n0 = 0; n0 < n; n0 += step) {
     const int cnt = (int)(n - n0 < step ? n - n0 : step);
+    const float bslice = n0 == 0 ? beta : 1.f;
+    if (kh == 1 && kw == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && !add_bias) {
+      // a pointwise convolution: M is the input itself, viewed as [c, n*H*W]
+      ConvG op{x + n0 * image, c, H * W};
+      const int st = launch_syrk(op, d, (int64_t)cnt * H * W, alpha, bslice, C, workspace,
+                                 workspace_bytes, (hipStream_t)stream);
+      if (st != KFAC_OK) return st;
+      continue;
+    }
+    if (conv_a_taps_applicable(c, kh, kw, sh, sw, add_bias)) {
+      const int st = conv_a_taps(x + n0 * image, cnt, c, H, W, kh, kw, ph, pw, dh, dw, alpha,
+                                 bslice, C, workspace, workspace_bytes, (hipStream_t)stream);
+      if (st == KFAC_OK) continue;
+      if (st != -1) return st;
+    }
     ConvA op{x + n0 * image, c, H, W, kh, kw, sh, sw, ph, pw, dh, dw, OH, OW, d, add_bias ? 1 : 0};
-    const int st = launch_syrk(op, d, (int64_t)cnt * OH * OW, alpha, n0 == 0 ? beta : 1.f, C,
-                               workspace, workspace_bytes, (hipStream_t)stream);
+    const int st = launch_syrk(op, d, (int64_t)cnt * OH * OW, alpha, bslice, C, workspace,
+                               workspace_bytes, (hipStream_t)stream);
     if (st != KFAC_OK) return st;
   }
   return KFAC_OK;

@@ -1,0 +1,353 @@
+// A factor of a stride-1 Conv2d by spatial correlations.
+//
+// With M = im2col(x), the block of A = M M^T that couples kernel tap t = (kh, kw)
+// with tap t' = (kh', kw') is
+//     A[(c,t),(c',t')] = sum_{n,oh,ow} x~[n,c,oh+oy_t,ow+ox_t] * x~[n,c',oh+oy_t',ow+ox_t']
+// (x~ = zero-padded input, o = tap*dilation - padding).  For stride 1 this is the
+// spatial cross-correlation of channel c with channel c' at displacement
+// delta = o_t' - o_t, summed over a rectangular window of positions that depends
+// on (t, t') only through a few boundary rows and columns.  All blocks with the
+// same displacement therefore share one product over the interior, and differ by
+// thin edge strips.  For a 3x3 kernel the 45 block products of the upper triangle
+// collapse to 13 interior products (one per displacement of the half plane) plus
+// strips of one row or column: about 3.4x fewer flops than the im2col product,
+// with no bounds check anywhere (every piece lies inside the image).
+//
+//  1. host: per axis, the windows of all tap pairs are cut into disjoint pieces
+//     (plan_axis); a job = (displacement, piece_y, piece_x);
+//  2. corr_kernel: R_job[c][c'] = sum over the job's rectangle, on the MFMA tile
+//     engine, k-split across workgroups, partial sums into the workspace;
+//  3. block_sum_kernel: B[(t,t')][c][c'] = sum over the block's jobs and their
+//     k-splits, in a fixed order (t <= t');
+//  4. interleave_kernel: A[(c,t),(c',t')] = alpha * B + beta * A_old, with the
+//     blocks below the diagonal taken transposed; an 8x8-channel region of A goes
+//     through LDS so that both the reads of B and the writes of A are row-contiguous.
+#include <limits.h>
+#include <string.h>
+
+#include <algorithm>
+#include <vector>
+
+#include "common.h"
+#include "operands.h"
+
+namespace kfac {
+
+// x[n][c][u0 + ry + dy][v0 + rx + dx] for k = (n, ry, rx) inside a hh x ww rectangle
+struct ShiftX {
+  static constexpr int layout = MK;
+  static constexpr bool has_second = false;
+  const float* p;
+  int C, H, W, u0, v0, hh, ww;     // u0, v0 already include the displacement
+  struct MS { unsigned off; };
+  struct KS { unsigned off; };
+  __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc() const { return make_rsrc(p); }
+  __device__ __forceinline__ MS mstate(int m) const {
+    return MS{m < C ? (unsigned)(m * H * W) * 4u : INV_M};
+  }
+  __device__ __forceinline__ KS kstate(int k, bool valid) const {
+    const int area = hh * ww;
+    const int n = k / area;
+    const int rem = k - n * area;
+    const int ry = rem / ww;
+    const int rx = rem - ry * ww;
+    return KS{valid ? (unsigned)(n * C * H * W + (u0 + ry) * W + v0 + rx) * 4u : INV_K};
+  }
+  __device__ __forceinline__ unsigned off(const MS& m, const KS& k) const { return m.off + k.off; }
+  __device__ __forceinline__ bool is_one(const MS&) const { return false; }
+};
+
+struct JobDesc {
+  short u0, v0, hh, ww;    // rectangle of the first factor
+  short dy, dx;            // displacement of the second factor
+  short splits, pad;       // k-splits
+  int K;                   // n * hh * ww
+  int cps;                 // chunks per split
+  int tiles0;              // (unused by the kernels) first work item, kept for the host
+  int part0;               // index (in C*C units) of its first partial in the workspace
+};
+
+constexpr int MAX_JOBS = 64;
+constexpr int MAX_TAPS = 9;
+constexpr int MAX_PAIRS = MAX_TAPS * (MAX_TAPS + 1) / 2;
+constexpr int MAX_PAIR_JOBS = 512;     // pool shared by all pairs
+constexpr int CT = 8;                  // channels per side of an interleave region
+
+// The whole plan travels as a kernel argument (below the 4 KiB limit).
+struct TapPlanDev {
+  JobDesc jobs[MAX_JOBS];
+  int item0[MAX_JOBS];     // first work item of each job; INT_MAX past the last job
+  int njobs;
+  int npairs;
+  unsigned char pair_t[MAX_PAIRS + 3];       // t * 16 + t'
+  unsigned char pair_of[MAX_TAPS * MAX_TAPS + 3];   // [t * T + t'] -> pair (t <= t')
+  short pair_first[MAX_PAIRS + 1];           // into pair_jobs
+  short pair_jobs[MAX_PAIR_JOBS];
+};
+static_assert(sizeof(TapPlanDev) <= 3800, "plan must fit the kernel argument buffer");
+template <int W>
+__global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void corr_kernel(
+    const float* x, int C, int H, int Wd, const TapPlanDev plan, int tiles_side, float* ws) {
+  constexpr int TS = 64 * W;
+  constexpr int KC = Cfg<W, W>::KC;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  // work item -> (job, split, tile)
+  const int item = blockIdx.x;
+  int j = -1;
+#pragma unroll
+  for (int q = 0; q < MAX_JOBS; ++q) j += plan.item0[q] <= item ? 1 : 0;
+  const JobDesc jd = plan.jobs[j];
+  const int ntiles = tiles_side * tiles_side;
+  const int local = item - plan.item0[j];
+  const int split = local / ntiles;
+  const int tile = local - split * ntiles;
+  const int bi = tile / tiles_side, bj = tile - bi * tiles_side;
+  const int kbeg = split * jd.cps * KC;
+  int kend = kbeg + jd.cps * KC;
+  if (kend > jd.K) kend = jd.K;
+  ShiftX P{x, C, H, Wd, jd.u0, jd.v0, jd.hh, jd.ww};
+  ShiftX Q{x, C, H, Wd, jd.u0 + jd.dy, jd.v0 + jd.dx, jd.hh, jd.ww};
+  EpiStore epi{ws + (size_t)(jd.part0 + split) * C * C, C, C, C, 1.f, 0.f, false};
+  gemm_tile_cfg<W, W>(P, Q, bi * TS, bj * TS, kbeg, kend, false, epi, smem);
+}
+
+// B[pair][c][c'] = sum over the pair's jobs and their k-splits, in a fixed order
+__global__ __launch_bounds__(256) void block_sum_kernel(const TapPlanDev plan, const float* ws,
+                                                        int CC, float* B) {
+  const int pair = blockIdx.y;
+  const int jb = plan.pair_first[pair], je = plan.pair_first[pair + 1];
+  const int e = (blockIdx.x * 256 + threadIdx.x) * 4;
+  if (e >= CC) return;        // CC is a multiple of 4 (channel counts are >= 16 and even)
+  float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int q = jb; q < je; ++q) {
+    const JobDesc jd = plan.jobs[plan.pair_jobs[q]];
+    const float* part = ws + (size_t)jd.part0 * CC + e;
+    for (int sp = 0; sp < jd.splits; ++sp) {
+      const float4 v = *reinterpret_cast<const float4*>(part + (size_t)sp * CC);
+      s.x += v.x;
+      s.y += v.y;
+      s.z += v.z;
+      s.w += v.w;
+    }
+  }
+  *reinterpret_cast<float4*>(B + (size_t)pair * CC + e) = s;
+}
+
+// One workgroup writes the region of A that couples channels [8I, 8I+8) with
+// channels [8J, 8J+8), all taps: (8T)^2 elements, staged in LDS.
+__global__ __launch_bounds__(256) void interleave_kernel(const TapPlanDev plan, const float* B,
+                                                         int C, int T, float alpha, float beta,
+                                                         float* A) {
+  __shared__ float region[CT * MAX_TAPS][CT * MAX_TAPS + 1];
+  const int I = blockIdx.y, J = blockIdx.x;
+  const int d = C * T;
+  const size_t CC = (size_t)C * C;
+  const int total = T * T * CT * CT;
+  for (int e = threadIdx.x; e < total; e += 256) {
+    const int tt = e / (CT * CT);
+    const int ij = e - tt * (CT * CT);
+    const int t = tt / T, t2 = tt - t * T;
+    float v = 0.f;
+    if (t <= t2) {
+      // B[(t,t2)][c][c2], read along c2
+      const int i = ij / CT, j = ij - i * CT;
+      const int c = I * CT + i, c2 = J * CT + j;
+      if (c < C && c2 < C) v = B[plan.pair_of[t * T + t2] * CC + (size_t)c * C + c2];
+      region[i * T + t][j * T + t2] = v;
+    } else {
+      // transposed block: B[(t2,t)][c2][c], read along c
+      const int j = ij / CT, i = ij - j * CT;
+      const int c = I * CT + i, c2 = J * CT + j;
+      if (c < C && c2 < C) v = B[plan.pair_of[t2 * T + t] * CC + (size_t)c2 * C + c];
+      region[i * T + t][j * T + t2] = v;
+    }
+  }
+  __syncthreads();
+  const int side = CT * T;
+  const int rows = min(side, d - I * side), cols = min(side, d - J * side);
+  for (int e = threadIdx.x; e < side * side; e += 256) {
+    const int r = e / side, q = e - r * side;
+    if (r < rows && q < cols) {
+      const size_t idx = (size_t)(I * side + r) * d + J * side + q;
+      float o = alpha * region[r][q];
+      if (beta != 0.f) o += beta * A[idx];
+      A[idx] = o;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host-side planning
+// ---------------------------------------------------------------------------
+struct AxisPiece {
+  int delta, lo, hi;      // first-factor coordinates [lo, hi)
+};
+
+struct AxisPlan {
+  std::vector<AxisPiece> pieces;
+  // for tap pair (a, a'): indices of the pieces that make up its window
+  std::vector<std::vector<int>> pair_pieces;   // [a * K + a']
+};
+
+static AxisPlan plan_axis(int size, int out, int K, int dil, int pad) {
+  AxisPlan ap;
+  ap.pair_pieces.resize((size_t)K * K);
+  struct Win { int a, b, delta, lo, hi; };
+  std::vector<Win> wins;
+  for (int a = 0; a < K; ++a)
+    for (int b = 0; b < K; ++b) {
+      const int oa = a * dil - pad, ob = b * dil - pad;
+      const int lo = std::max(0, std::max(-oa, -ob));
+      const int hi = std::min(out, std::min(size - oa, size - ob));
+      if (hi > lo) wins.push_back(Win{a, b, ob - oa, lo + oa, hi + oa});
+    }
+  // per displacement: cut at every window boundary
+  std::vector<int> deltas;
+  for (auto& w : wins) deltas.push_back(w.delta);
+  std::sort(deltas.begin(), deltas.end());
+  deltas.erase(std::unique(deltas.begin(), deltas.end()), deltas.end());
+  for (int dl : deltas) {
+    std::vector<int> cuts;
+    for (auto& w : wins)
+      if (w.delta == dl) { cuts.push_back(w.lo); cuts.push_back(w.hi); }
+    std::sort(cuts.begin(), cuts.end());
+    cuts.erase(std::unique(cuts.begin(), cuts.end()), cuts.end());
+    for (size_t i = 0; i + 1 < cuts.size(); ++i) {
+      const int lo = cuts[i], hi = cuts[i + 1];
+      std::vector<const Win*> users;
+      for (auto& w : wins)
+        if (w.delta == dl && w.lo <= lo && hi <= w.hi) users.push_back(&w);
+      if (users.empty()) continue;
+      const int idx = (int)ap.pieces.size();
+      ap.pieces.push_back(AxisPiece{dl, lo, hi});
+      for (auto* w : users) ap.pair_pieces[(size_t)w->a * K + w->b].push_back(idx);
+    }
+  }
+  return ap;
+}
+
+struct TapPlanHost {
+  TapPlanDev dev;
+  int tiles_side, w, items;
+  size_t partial_floats, sum_offset;
+  bool ok;
+};
+
+static TapPlanHost plan_taps(int n, int c, int H, int Wd, int kh, int kw, int ph, int pw, int dh,
+                             int dw) {
+  TapPlanHost hp;
+  hp.ok = false;
+  const int T = kh * kw;
+  if (T < 2 || T > MAX_TAPS) return hp;
+  const int OH = H + 2 * ph - dh * (kh - 1), OW = Wd + 2 * pw - dw * (kw - 1);
+  if (OH <= 0 || OW <= 0) return hp;
+  const AxisPlan ay = plan_axis(H, OH, kh, dh, ph), ax = plan_axis(Wd, OW, kw, dw, pw);
+  TapPlanDev& pd = hp.dev;
+  memset(&pd, 0, sizeof(pd));
+  std::vector<long> job_key;
+  int npj = 0;
+  pd.pair_first[0] = 0;
+  for (int t = 0; t < T; ++t)
+    for (int t2 = t; t2 < T; ++t2) {
+      const int a = t / kw, b = t % kw, a2 = t2 / kw, b2 = t2 % kw;
+      pd.pair_t[pd.npairs] = (unsigned char)(t * 16 + t2);
+      pd.pair_of[t * T + t2] = (unsigned char)pd.npairs;
+      for (int py : ay.pair_pieces[(size_t)a * kh + a2])
+        for (int px : ax.pair_pieces[(size_t)b * kw + b2]) {
+          const long key = (long)py * 4096 + px;
+          int j = 0;
+          while (j < (int)job_key.size() && job_key[j] != key) ++j;
+          if (j == (int)job_key.size()) {
+            if (pd.njobs >= MAX_JOBS) return hp;
+            job_key.push_back(key);
+            JobDesc& jd = pd.jobs[pd.njobs++];
+            jd.u0 = (short)ay.pieces[py].lo;
+            jd.hh = (short)(ay.pieces[py].hi - ay.pieces[py].lo);
+            jd.dy = (short)ay.pieces[py].delta;
+            jd.v0 = (short)ax.pieces[px].lo;
+            jd.ww = (short)(ax.pieces[px].hi - ax.pieces[px].lo);
+            jd.dx = (short)ax.pieces[px].delta;
+            jd.K = n * (int)jd.hh * (int)jd.ww;
+          }
+          if (npj >= MAX_PAIR_JOBS) return hp;
+          pd.pair_jobs[npj++] = (short)j;
+        }
+      ++pd.npairs;
+      pd.pair_first[pd.npairs] = (short)npj;
+    }
+  // tiles and k-splits: work items in proportion to each job's length
+  hp.w = c <= 64 ? 1 : 2;
+  const int ts = 64 * hp.w;
+  hp.tiles_side = cdiv(c, ts);
+  const int ntiles = hp.tiles_side * hp.tiles_side;
+  const int kc = hp.w == 1 ? Cfg<1, 1>::KC : Cfg<2, 2>::KC;
+  double total = 0;
+  for (int j = 0; j < pd.njobs; ++j) total += (double)pd.jobs[j].K;
+  const double target_items = hp.w == 1 ? 3072.0 : 1024.0;
+  int item = 0, part = 0;
+  for (int j = 0; j < pd.njobs; ++j) {
+    JobDesc& jd = pd.jobs[j];
+    const long nchunks = ((long)jd.K + kc - 1) / kc;
+    long splits = (long)(target_items * ((double)jd.K / total) / ntiles + 0.5);
+    const long max_splits = std::max<long>(1, nchunks / (128 / kc));
+    splits = std::max<long>(1, std::min(std::min(splits, max_splits), 4096L));
+    long cps = (nchunks + splits - 1) / splits;
+    splits = (nchunks + cps - 1) / cps;
+    jd.splits = (short)splits;
+    jd.cps = (int)cps;
+    jd.tiles0 = item;
+    pd.item0[j] = item;
+    jd.part0 = part;
+    item += (int)splits * ntiles;
+    part += (int)splits;
+  }
+  for (int j = pd.njobs; j < MAX_JOBS; ++j) pd.item0[j] = INT_MAX;
+  hp.items = item;
+  hp.partial_floats = (size_t)(part + pd.npairs) * c * c;     // partials, then the block sums
+  hp.sum_offset = (size_t)part * c * c;
+  hp.ok = true;
+  return hp;
+}
+
+bool conv_a_taps_applicable(int c, int kh, int kw, int sh, int sw, int add_bias) {
+  return sh == 1 && sw == 1 && !add_bias && kh * kw >= 2 && kh * kw <= MAX_TAPS && c >= 16 &&
+         c % 2 == 0;
+}
+
+size_t conv_a_taps_workspace(int n, int c, int H, int W, int kh, int kw, int ph, int pw, int dh,
+                             int dw) {
+  const TapPlanHost hp = plan_taps(n, c, H, W, kh, kw, ph, pw, dh, dw);
+  return hp.ok ? hp.partial_floats * sizeof(float) : 0;
+}
+
+// returns KFAC_OK, an error, or -1 when the geometry is not covered (the caller
+// then uses the im2col kernel)
+int conv_a_taps(const float* x, int n, int c, int H, int W, int kh, int kw, int ph, int pw, int dh,
+                int dw, float alpha, float beta, float* A, void* workspace, size_t workspace_bytes,
+                hipStream_t stream) {
+  const TapPlanHost hp = plan_taps(n, c, H, W, kh, kw, ph, pw, dh, dw);
+  if (!hp.ok) return -1;
+  if (!workspace || workspace_bytes < hp.partial_floats * sizeof(float)) return KFAC_ERR_WORKSPACE;
+  float* ws = (float*)workspace;
+  float* B = ws + hp.sum_offset;
+  const int T = kh * kw;
+  if (hp.w == 1) {
+    constexpr int lds = Cfg<1, 1>::SMEM_FLOATS * (int)sizeof(float);
+    if (!enable_large_lds((const void*)corr_kernel<1>, lds)) return KFAC_ERR_LAUNCH;
+    hipLaunchKernelGGL(corr_kernel<1>, dim3(hp.items), dim3(64), lds, stream, x, c, H, W, hp.dev,
+                       hp.tiles_side, ws);
+  } else {
+    constexpr int lds = Cfg<2, 2>::SMEM_FLOATS * (int)sizeof(float);
+    if (!enable_large_lds((const void*)corr_kernel<2>, lds)) return KFAC_ERR_LAUNCH;
+    hipLaunchKernelGGL(corr_kernel<2>, dim3(hp.items), dim3(256), lds, stream, x, c, H, W, hp.dev,
+                       hp.tiles_side, ws);
+  }
+  hipLaunchKernelGGL(block_sum_kernel, dim3(cdiv(c * c / 4, 256), hp.dev.npairs), dim3(256), 0,
+                     stream, hp.dev, ws, c * c, B);
+  const int regions = cdiv(c, CT);
+  hipLaunchKernelGGL(interleave_kernel, dim3(regions, regions), dim3(256), 0, stream, hp.dev, B, c,
+                     T, alpha, beta, A);
+  return launch_status();
+}
+
+}  // namespace kfac

@@ -59,7 +59,8 @@ def factor_conv_a(x, kernel_size, stride, padding, dilation, add_bias, alpha, ou
         raise _hip.KfacHipError('conv geometry gives an empty output')
     d = c * kh * kw + (1 if add_bias else 0)
     out = _out_square(out, d, x, beta)
-    ws, ws_bytes = _hip.workspace(x.device, lib.kfac_factor_workspace_bytes(d, n * oh * ow))
+    ws, ws_bytes = _hip.workspace(x.device, lib.kfac_factor_conv_a_workspace_bytes(
+        n, c, H, W, kh, kw, sh, sw, ph, pw, dh, dw, int(bool(add_bias))))
     st = lib.kfac_factor_conv_a(_hip.dev_ptr(x, 'input'), n, c, H, W, kh, kw, sh, sw, ph, pw,
                                 dh, dw, int(bool(add_bias)), float(alpha), float(beta),
                                 _hip.dev_ptr(out, 'factor'),

@@ -65,6 +65,11 @@ def test_factor_linear_fused_running_average(ops, dev):
     ((2, 3, 30, 30), (7, 7), (2, 2), (3, 3), (1, 1), False),
     ((1, 1, 1, 1), (1, 1), (1, 1), (0, 0), (1, 1), True),
     ((16, 32, 28, 28), (3, 3), (2, 2), (1, 1), (1, 1), False),
+    # pointwise without bias (read like an output gradient), with padding, with stride
+    ((4, 48, 8, 8), (1, 1), (1, 1), (0, 0), (1, 1), False),
+    ((3, 300, 7, 7), (1, 1), (1, 1), (0, 0), (1, 1), False),
+    ((3, 20, 7, 7), (1, 1), (1, 1), (1, 1), (1, 1), False),
+    ((3, 20, 8, 8), (1, 1), (2, 2), (0, 0), (1, 1), False),
 ])
 def test_factor_conv_a(ops, dev, shape, k, s, p, d, bias):
     torch.manual_seed(sum(shape))
@@ -74,6 +79,38 @@ def test_factor_conv_a(ops, dev, shape, k, s, p, d, bias):
     assert out.shape == ref.shape
     assert O.rel_fro(out, ref) < TOL
     assert torch.equal(out, out.t())
+
+
+# stride 1, no bias, 2..9 taps, an even channel count >= 16: the A factor is assembled
+# from spatial correlations of the input instead of the im2col product (and falls
+# back to it when the geometry needs too many pieces, e.g. 3x3 without padding)
+@pytest.mark.parametrize('shape,k,p,d', [
+    ((3, 16, 7, 9), (3, 3), (1, 1), (1, 1)),
+    ((2, 130, 9, 8), (3, 3), (2, 2), (2, 2)),
+    ((2, 18, 6, 7), (2, 3), (1, 0), (1, 2)),
+    ((2, 16, 5, 5), (3, 3), (2, 1), (1, 1)),
+    ((2, 32, 3, 3), (3, 3), (1, 1), (1, 1)),
+    ((2, 16, 2, 2), (3, 3), (1, 1), (1, 1)),
+    ((2, 20, 10, 10), (1, 5), (0, 2), (1, 1)),
+    ((2, 16, 6, 6), (3, 3), (3, 3), (1, 1)),
+    ((2, 16, 7, 7), (3, 3), (0, 0), (1, 1)),
+    ((4, 256, 14, 14), (3, 3), (1, 1), (1, 1)),
+    ((2, 512, 7, 7), (3, 3), (1, 1), (1, 1)),
+    ((5, 66, 28, 28), (3, 3), (1, 1), (1, 1)),
+])
+def test_factor_conv_a_by_correlations(ops, dev, shape, k, p, d):
+    torch.manual_seed(sum(shape) + k[1])
+    x = torch.randn(*shape)
+    ref = O.factor_conv_a(x, k, (1, 1), p, d, False, D)
+    out = ops.factor_conv_a(x.to(dev), k, (1, 1), p, d, False, 1.0 / shape[0])
+    assert out.shape == ref.shape
+    assert O.rel_fro(out, ref) < TOL
+    assert torch.equal(out, out.t())
+    # running-average epilogue on the same path
+    old = spd(ref.shape[0])
+    out = ops.factor_conv_a(x.to(dev), k, (1, 1), p, d, False, 0.9 / shape[0],
+                            out=old.to(dev).clone(), beta=0.1)
+    assert O.rel_fro(out, 0.9 * ref + 0.1 * old.double()) < TOL
 
 
 @pytest.mark.parametrize('shape', [(1, 1, 1, 1), (2, 3, 4, 4), (8, 64, 7, 7), (4, 130, 14, 14),
