@@ -182,6 +182,43 @@ int kfac_diag_precondition_batched(int count, const int64_t* numel, const float*
                                    float* const* grad,
                                    void* workspace, size_t workspace_bytes, void* stream);
 
+/* Diagonal covariance of a Linear layer: W[i][j] = alpha * sum_b g[b][i]^2 a[b][j]^2
+ * ([fout, fin]) and, with add_bias, bvec[i] = alpha * sum_b g[b][i]^2.
+ * g is [n, fout], a is [n, fin].  Replaces the two element-wise squares, the
+ * einsum('ki,kj->ij') and the mean of torchsso/curv/cov/linear.py:28-45 with
+ * the n^2 rescale of curvature.py:154-158 folded in (alpha = n). */
+int kfac_diag_cov_linear(const float* g, const float* a, int n, int fout, int fin, int add_bias,
+                         float alpha, float* W, float* bvec, void* stream);
+
+/* Diagonal covariance of a Conv2d weight:
+ *   out[i][j] = alpha * sum_b (sum_k g[b][i][k] * M_b[j][k])^2     ([cout, c*kh*kw])
+ * with M_b = im2col of sample b, i.e. the batch sum of the squared per-sample
+ * weight gradients.  g is [n, cout, OH, OW], x is [n, c, H, W].
+ * Replaces F.unfold + einsum('bik,bjk->bij') + mul + mean of
+ * torchsso/curv/cov/conv.py:15-36 (alpha = n after the n^2 rescale); neither the
+ * unfolded input nor the per-sample gradients are written to memory. */
+size_t kfac_diag_cov_conv2d_workspace_bytes(int n, int cout, int c, int kh, int kw);
+int kfac_diag_cov_conv2d(const float* g, const float* x, int n, int cout, int c, int H, int W,
+                         int kh, int kw, int sh, int sw, int ph, int pw, int dh, int dw,
+                         float alpha, float* out,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+/* y[i] = sqrt(x[i])   std of a diagonal curvature, curvature.py:240-241. */
+int kfac_sqrt_batched(int count, const int64_t* numel, const float* const* x, float* const* y,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
+/* y[i] = max(x[i], y[i])   running maximum of the average, curvature.py:189-191. */
+int kfac_max_batched(int count, const int64_t* numel, const float* const* x, float* const* y,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* param = mean + std_scale * noise * std, element-wise; noise_to_param[i] holds the
+ * standard-normal noise on entry and the sampled parameter on return.
+ * DiagCurvature.sample_params, curvature.py:243-246 (std_scale is a HOST array). */
+int kfac_diag_sample_batched(int count, const int64_t* numel, const float* const* mean,
+                             const float* const* std_dev, float* const* noise_to_param,
+                             const float* std_scale,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
 /* g += weight_decay*p ; if momentum: buf = momentum*buf + g, g = buf ; p -= lr*g
  * with g written back, per tensor i with its own lr/momentum/weight_decay
  * (HOST arrays).  The preconditioned-gradient tail of

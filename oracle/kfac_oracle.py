@@ -22,6 +22,10 @@ which retypes the formula):
                        2x2 by hand
   precondition         Kronecker identity via torch.kron
   bn_diag              per-sample gradient identity through autograd
+  diag_cov_linear/conv per-sample gradients taken one sample at a time through autograd
+                       (the bias entry of diag_cov_conv2d, a sum of squares where the
+                       per-sample gradient would give the square of a sum, is pinned
+                       by brute-force loops instead)
   fisher_*             prob == 1 reduces to the Cov factor; the exact sum over classes at the
                        logits layer equals mean_n(diag(p_n) - p_n p_n^T) (closed form)
   cholesky_upper       U^T U == X, U upper, diag > 0
@@ -110,6 +114,47 @@ def bn_diag(xhat, g, bias=True, dtype=torch.float32, scale_by_batch=True):
     if scale_by_batch:
         out = [o * float(n ** 2) for o in out]
     return out
+
+
+def diag_cov_linear(a, g, bias=True, prob=None, dtype=torch.float32, scale_by_batch=True):
+    """Diagonal covariance of a Linear layer: W = (g^2)^T (a^2) / n, b = mean_n g^2
+    (torchsso/curv/cov/linear.py:28-45), times n^2 (curvature.py:154-158).  With
+    `prob`, one weighted pass of DiagFisherLinear: g^2 is replaced by prob * g^2
+    (fisher/linear.py:11-33)."""
+    a, g = a.to(dtype), g.to(dtype)
+    n = a.shape[0]
+    gg = g * g
+    if prob is not None:
+        gg = gg * prob.to(dtype).reshape(n, 1)
+    out = [(gg.t() @ (a * a)) / n]
+    if bias:
+        out.append(gg.mean(dim=0))
+    return [o * float(n ** 2) for o in out] if scale_by_batch else out
+
+
+def diag_cov_conv2d(x, g, kernel_size, stride=(1, 1), padding=(0, 0), dilation=(1, 1), bias=True,
+                    prob=None, dtype=torch.float32, scale_by_batch=True):
+    """Diagonal covariance of a Conv2d layer: the batch mean of the squared
+    per-sample weight gradients g_b M_b^T (M_b = unfold of sample b), shaped like
+    the weight; the bias entry is mean_n sum_hw g^2 -- the sum of the squares,
+    as the reference computes it (torchsso/curv/cov/conv.py:15-42), times n^2
+    (curvature.py:154-158).  With `prob`, one weighted pass of DiagFisherConv2d
+    (fisher/conv.py:12-45)."""
+    x, g = x.to(dtype), g.to(dtype)
+    n, c_out, h, w = g.shape
+    kh, kw = kernel_size
+    m = F.unfold(x, kernel_size=kernel_size, stride=stride, padding=padding, dilation=dilation)
+    g2d = g.reshape(n, c_out, -1)
+    grad_in = torch.bmm(g2d, m.transpose(1, 2))                    # n x c_out x (c kh kw)
+    sq = grad_in * grad_in
+    gg = (g2d * g2d).sum(dim=2)                                    # n x c_out
+    if prob is not None:
+        sq = sq * prob.to(dtype).reshape(n, 1, 1)
+        gg = gg * prob.to(dtype).reshape(n, 1)
+    out = [sq.mean(dim=0).reshape(c_out, -1, kh, kw)]
+    if bias:
+        out.append(gg.mean(dim=0))
+    return [o * float(n ** 2) for o in out] if scale_by_batch else out
 
 
 def fisher_linear_g(g, prob, dtype=torch.float32, scale_by_batch=True):

@@ -26,7 +26,7 @@ __global__ void vec_setup_kernel(VecChunk chunk, VecDesc* table, int offset, int
   if (i < count) table[offset + i] = chunk.d[i];
 }
 
-enum { OP_AXPBY = 0, OP_DIAG_INV = 1, OP_MUL = 2, OP_SGD = 3 };
+enum { OP_AXPBY = 0, OP_DIAG_INV = 1, OP_MUL = 2, OP_SGD = 3, OP_SQRT = 4, OP_MAX = 5, OP_ADDCMUL = 6 };
 
 constexpr int EW_THREADS = 256;
 constexpr int EW_PER_THREAD = 4;
@@ -47,6 +47,13 @@ __device__ __forceinline__ void apply(const VecDesc& m, long i) {
   } else if (OP == OP_MUL) {
     // b *= a
     m.b[i] = m.b[i] * m.a[i];
+  } else if (OP == OP_SQRT) {
+    m.b[i] = sqrtf(m.a[i]);
+  } else if (OP == OP_MAX) {
+    m.b[i] = fmaxf(m.a[i], m.b[i]);
+  } else if (OP == OP_ADDCMUL) {
+    // b = a + s0 * b * c     (a = mean, b = noise in / parameter out, c = std)
+    m.b[i] = fmaf(m.s0 * m.b[i], m.c[i], m.a[i]);
   } else {
     // a = param, b = grad, c = momentum buffer; s0 = lr, s1 = momentum, s2 = weight decay
     float g = m.b[i];
@@ -289,6 +296,43 @@ int kfac_diag_precondition_batched(int count, const int64_t* numel, const float*
     d[i] = VecDesc{(float*)inv[i], grad[i], nullptr, (long)numel[i], 0.f, 0.f, 0.f, 0.f};
   }
   return run_vec<OP_MUL>(d, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int kfac_sqrt_batched(int count, const int64_t* numel, const float* const* x, float* const* y,
+                       void* workspace, size_t workspace_bytes, void* stream) {
+  if (count < 0 || (count > 0 && (!numel || !x || !y))) return KFAC_ERR_ARG;
+  std::vector<VecDesc> d(count);
+  for (int i = 0; i < count; ++i) {
+    if (numel[i] <= 0 || !x[i] || !y[i]) return KFAC_ERR_ARG;
+    d[i] = VecDesc{(float*)x[i], y[i], nullptr, (long)numel[i], 0.f, 0.f, 0.f, 0.f};
+  }
+  return run_vec<OP_SQRT>(d, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int kfac_max_batched(int count, const int64_t* numel, const float* const* x, float* const* y,
+                     void* workspace, size_t workspace_bytes, void* stream) {
+  if (count < 0 || (count > 0 && (!numel || !x || !y))) return KFAC_ERR_ARG;
+  std::vector<VecDesc> d(count);
+  for (int i = 0; i < count; ++i) {
+    if (numel[i] <= 0 || !x[i] || !y[i]) return KFAC_ERR_ARG;
+    d[i] = VecDesc{(float*)x[i], y[i], nullptr, (long)numel[i], 0.f, 0.f, 0.f, 0.f};
+  }
+  return run_vec<OP_MAX>(d, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int kfac_diag_sample_batched(int count, const int64_t* numel, const float* const* mean,
+                             const float* const* std_dev, float* const* noise_to_param,
+                             const float* std_scale, void* workspace, size_t workspace_bytes,
+                             void* stream) {
+  if (count < 0 || (count > 0 && (!numel || !mean || !std_dev || !noise_to_param || !std_scale)))
+    return KFAC_ERR_ARG;
+  std::vector<VecDesc> d(count);
+  for (int i = 0; i < count; ++i) {
+    if (numel[i] <= 0 || !mean[i] || !std_dev[i] || !noise_to_param[i]) return KFAC_ERR_ARG;
+    d[i] = VecDesc{(float*)mean[i], noise_to_param[i], (float*)std_dev[i], (long)numel[i],
+                   std_scale[i], 0.f, 0.f, 0.f};
+  }
+  return run_vec<OP_ADDCMUL>(d, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 int kfac_sgd_update_batched(int count, const int64_t* numel, float* const* param,

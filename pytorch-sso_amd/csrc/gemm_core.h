@@ -24,6 +24,7 @@
 // for both operands, which is a permutation of the reduction index and so does
 // not change the product.
 #pragma once
+#include <type_traits>
 #include <hip/hip_runtime.h>
 
 namespace kfac {
@@ -83,6 +84,13 @@ __device__ __forceinline__ float buffer_load(__amdgpu_buffer_rsrc_t r, unsigned 
 // global -> register -> LDS staging of one operand chunk (KC x ROWS elements
 // swept by NT threads)
 // ---------------------------------------------------------------------------
+// An operand type with `static constexpr bool square = true` has its elements
+// squared on the way into LDS (diagonal curvature: sums of squared gradients).
+template <class T, class = void>
+struct squares_elements : std::false_type {};
+template <class T>
+struct squares_elements<T, std::void_t<decltype(T::square)>> : std::bool_constant<T::square> {};
+
 template <class OP, int ROWS, int NT, int KC>
 struct Stager {
   static constexpr int LDS_MK = KC + 4;
@@ -141,7 +149,8 @@ struct Stager {
     const int t = threadIdx.x;
 #pragma unroll
     for (int i = 0; i < CNT; ++i) {
-      const float v = ((onebits >> i) & 1u) ? 1.f : regs[i];
+      float v = ((onebits >> i) & 1u) ? 1.f : regs[i];
+      if (squares_elements<OP>::value) v *= v;
       if (OP::layout == KM)
         tile[((t / ROWS) + KSTEP * i) * ROWS + (t % ROWS)] = v;
       else
@@ -183,6 +192,25 @@ __device__ __forceinline__ void load_frags(const lds_f* tile, int base, int r, i
 // EPI::store(row, col, value) receives every element of the tile (global
 // coordinates row = m0 + ..., col = n0 + ...).
 // ---------------------------------------------------------------------------
+// An epilogue with `static constexpr bool indexed = true` receives the running
+// index (a*2 + b)*16 + i of each accumulator instead of its position in C.
+template <class T, class = void>
+struct indexed_epilogue : std::false_type {};
+template <class T>
+struct indexed_epilogue<T, std::void_t<decltype(T::indexed)>> : std::bool_constant<T::indexed> {};
+
+// Position in C of accumulator element i of block (a, b) of the calling thread;
+// the epilogue visits (a, b, i) in lexicographic order, 64 elements per thread.
+template <int WM, int WN>
+__device__ __forceinline__ void acc_coords(int m0, int n0, int a, int b, int i, int& row,
+                                           int& col) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  row = m0 + (wave / WN) * 64 + 32 * a + 8 * (i >> 2) + 4 * h + (i & 3);
+  col = n0 + (wave % WN) * 64 + 32 * b + r;
+}
+
 template <int WM, int WN, class OPP, class OPQ, class EPI>
 __device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0, int n0,
                                               int kbeg, int kend, bool same, EPI& epi,
@@ -276,17 +304,18 @@ __device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0
     __syncthreads();
   }
 
-  // accumulator element i of lane (r, h) in block (a, b):
-  //   row = 32a + 8*(i/4) + 4h + i%4 ,  col = 32b + r
 #pragma unroll
   for (int a = 0; a < 2; ++a)
 #pragma unroll
     for (int b = 0; b < 2; ++b)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int row = m0 + wm + 32 * a + 8 * (i >> 2) + 4 * h + (i & 3);
-        const int col = n0 + wn + 32 * b + r;
-        epi.store(row, col, acc[a][b][i]);
+        int row, col;
+        acc_coords<WM, WN>(m0, n0, a, b, i, row, col);
+        if constexpr (indexed_epilogue<EPI>::value)
+          epi.store_at((a * 2 + b) * 16 + i, acc[a][b][i]);     // index known at compile time
+        else
+          epi.store(row, col, acc[a][b][i]);
       }
 }
 

@@ -9,12 +9,13 @@ from torchsso import _hip, _ops  # NOQA
 from torchsso import utils  # NOQA
 
 from torchsso.curv.curvature import Curvature, DiagCurvature, KronCurvature  # NOQA
-from torchsso.curv.cov.linear import CovLinear, KronCovLinear  # NOQA
-from torchsso.curv.cov.conv import CovConv2d, KronCovConv2d  # NOQA
+from torchsso.curv.cov.linear import CovLinear, DiagCovLinear, KronCovLinear  # NOQA
+from torchsso.curv.cov.conv import CovConv2d, DiagCovConv2d, KronCovConv2d  # NOQA
 from torchsso.curv.cov.batchnorm import CovBatchNorm1d, DiagCovBatchNorm1d, CovBatchNorm2d, DiagCovBatchNorm2d  # NOQA
 
 from torchsso.curv.fisher import Fisher, get_closure_for_fisher  # NOQA
 from torchsso.curv.fisher import KronFisherLinear, KronFisherConv2d, DiagFisherBatchNorm2d  # NOQA
+from torchsso.curv.fisher import DiagFisherLinear, DiagFisherConv2d  # NOQA
 
 from torchsso import optim  # NOQA
 

@@ -21,8 +21,7 @@ c_f32 = ctypes.c_float
 c_ptr = ctypes.c_void_p
 c_size = ctypes.c_size_t
 
-ERRORS = {1: 'invalid argument', 2: 'workspace too small', 3: 'HIP launch failed',
-          4: 'size above the static scratch limit'}
+ERRORS = {1: 'invalid argument', 2: 'workspace too small', 3: 'HIP launch failed'}
 
 
 class KfacHipError(RuntimeError):
@@ -60,6 +59,15 @@ _SIGNATURES = {
                                    c_ptr, c_size, c_ptr]),
     'kfac_diag_inverse_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_int,
                                           c_ptr, c_size, c_ptr]),
+    'kfac_sqrt_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_size, c_ptr]),
+    'kfac_max_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_size, c_ptr]),
+    'kfac_diag_sample_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
+                                         c_ptr, c_size, c_ptr]),
+    'kfac_diag_cov_linear': (c_int, [c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_f32,
+                                     c_ptr, c_ptr, c_ptr]),
+    'kfac_diag_cov_conv2d_workspace_bytes': (c_size, [c_int] * 5),
+    'kfac_diag_cov_conv2d': (c_int, [c_ptr, c_ptr] + [c_int] * 13 + [c_f32, c_ptr,
+                                                                   c_ptr, c_size, c_ptr]),
     'kfac_diag_precondition_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr,
                                                c_ptr, c_size, c_ptr]),
     'kfac_sgd_update_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,

@@ -282,6 +282,90 @@ def diag_precondition_batched(invs, grads):
     _hip.check(st, 'kfac_diag_precondition_batched')
 
 
+def sqrt_batched(xs, ys):
+    """ys[i] = sqrt(xs[i])."""
+    lib = _hip.load()
+    if len(xs) == 0:
+        return
+    _check_same_numel(xs, ys, 'sqrt')
+    dev, numel, ws, ws_bytes = _vec_args(lib, xs)
+    st = lib.kfac_sqrt_batched(len(xs), numel, _hip.ptr_array(xs, 'x'), _hip.ptr_array(ys, 'y'),
+                               _ws_ptr(ws), ws_bytes, _hip.stream_ptr(dev))
+    _hip.check(st, 'kfac_sqrt_batched')
+
+
+def max_batched(xs, ys):
+    """ys[i] = max(xs[i], ys[i]) in place."""
+    lib = _hip.load()
+    if len(xs) == 0:
+        return
+    _check_same_numel(xs, ys, 'max')
+    dev, numel, ws, ws_bytes = _vec_args(lib, xs)
+    st = lib.kfac_max_batched(len(xs), numel, _hip.ptr_array(xs, 'x'), _hip.ptr_array(ys, 'y'),
+                              _ws_ptr(ws), ws_bytes, _hip.stream_ptr(dev))
+    _hip.check(st, 'kfac_max_batched')
+
+
+def diag_sample_batched(means, stds, noise_to_params, std_scales):
+    """noise_to_params[i] = means[i] + std_scales[i] * noise_to_params[i] * stds[i] in place."""
+    lib = _hip.load()
+    if len(means) == 0:
+        return
+    _check_same_numel(means, stds, 'diag sample (std)')
+    _check_same_numel(means, noise_to_params, 'diag sample (param)')
+    dev, numel, ws, ws_bytes = _vec_args(lib, means)
+    st = lib.kfac_diag_sample_batched(len(means), numel, _hip.ptr_array(means, 'mean'),
+                                      _hip.ptr_array(stds, 'std'),
+                                      _hip.ptr_array(noise_to_params, 'param'),
+                                      _hip.f32_array(std_scales), _ws_ptr(ws), ws_bytes,
+                                      _hip.stream_ptr(dev))
+    _hip.check(st, 'kfac_diag_sample_batched')
+
+
+def diag_cov_linear(g, a, add_bias, alpha):
+    """(W, b): W[i][j] = alpha * sum_k g[k,i]^2 a[k,j]^2 ; b[i] = alpha * sum_k g[k,i]^2 (or None)."""
+    lib = _hip.load()
+    if g.dim() != 2 or a.dim() != 2 or g.shape[0] != a.shape[0]:
+        raise _hip.KfacHipError('diag_cov_linear: g %s vs a %s' % (tuple(g.shape), tuple(a.shape)))
+    g, a = g.contiguous(), a.contiguous()
+    n, fout = g.shape
+    fin = a.shape[1]
+    W = torch.empty((fout, fin), dtype=torch.float32, device=g.device)
+    b = torch.empty(fout, dtype=torch.float32, device=g.device) if add_bias else None
+    st = lib.kfac_diag_cov_linear(_hip.dev_ptr(g, 'output gradient'), _hip.dev_ptr(a, 'input'), n,
+                                  fout, fin, int(bool(add_bias)), float(alpha), W.data_ptr(),
+                                  None if b is None else b.data_ptr(), _hip.stream_ptr(g.device))
+    _hip.check(st, 'kfac_diag_cov_linear')
+    return W, b
+
+
+def diag_cov_conv2d(g, x, kernel_size, stride, padding, dilation, alpha):
+    """[cout, c*kh*kw] tensor alpha * sum_b (g_b M_b^T)^2 of squared per-sample weight gradients."""
+    lib = _hip.load()
+    if g.dim() != 4 or x.dim() != 4 or g.shape[0] != x.shape[0]:
+        raise _hip.KfacHipError('diag_cov_conv2d: g %s vs x %s' % (tuple(g.shape), tuple(x.shape)))
+    g, x = g.contiguous(), x.contiguous()
+    n, c, H, W = x.shape
+    cout = g.shape[1]
+    kh, kw = _pair(kernel_size)
+    sh, sw = _pair(stride)
+    ph, pw = _pair(padding)
+    dh, dw = _pair(dilation)
+    oh = (H + 2 * ph - dh * (kh - 1) - 1) // sh + 1
+    ow = (W + 2 * pw - dw * (kw - 1) - 1) // sw + 1
+    if (oh, ow) != tuple(g.shape[2:]):
+        raise _hip.KfacHipError('diag_cov_conv2d: output gradient is %s, geometry gives %s'
+                                % (tuple(g.shape[2:]), (oh, ow)))
+    out = torch.empty((cout, c * kh * kw), dtype=torch.float32, device=g.device)
+    ws, ws_bytes = _hip.workspace(g.device,
+                                  lib.kfac_diag_cov_conv2d_workspace_bytes(n, cout, c, kh, kw))
+    st = lib.kfac_diag_cov_conv2d(_hip.dev_ptr(g, 'output gradient'), _hip.dev_ptr(x, 'input'), n,
+                                  cout, c, H, W, kh, kw, sh, sw, ph, pw, dh, dw, float(alpha),
+                                  out.data_ptr(), _ws_ptr(ws), ws_bytes, _hip.stream_ptr(g.device))
+    _hip.check(st, 'kfac_diag_cov_conv2d')
+    return out
+
+
 def sgd_update_batched(params, grads, bufs, lrs, momenta, weight_decays):
     """g += wd*p; buf = m*buf + g, g = buf (if m); p -= lr*g  for every tensor."""
     lib = _hip.load()

@@ -3,9 +3,11 @@
 KronCovLinear mirrors torchsso/curv/cov/linear.py:48-114 of the reference; the
 factors come from the HIP factor kernel, with the bias column (LAST) synthesised
 in the kernel and the 1/n and n^2 scalings folded into its scale factor.
+DiagCovLinear mirrors cov/linear.py:28-45: one product of the squared output
+gradient with the squared input, the operands squared inside the kernel.
 """
 from torchsso import _ops
-from torchsso.curv.curvature import Curvature, KronCurvature
+from torchsso.curv.curvature import Curvature, DiagCurvature, KronCurvature
 
 
 class CovLinear(Curvature):
@@ -17,6 +19,23 @@ class CovLinear(Curvature):
 
     def precondition_grad(self, params):
         pass
+
+
+class DiagCovLinear(DiagCurvature):
+
+    def _diag_data(self, grad_output):
+        # W[i][j] = mean_b g[b][i]^2 a[b][j]^2, b[i] = mean_b g[b][i]^2, both * n^2
+        # (reference: linear.py:30-45, curvature.py:154-158)
+        data_input = getattr(self._module, 'data_input', None)
+        assert data_input is not None
+        n = data_input.shape[0]
+        a = data_input.reshape(n, -1)
+        g = grad_output.reshape(n, -1)
+        w, b = _ops.diag_cov_linear(g, a, self.bias, float(n))
+        return [w] if b is None else [w, b]
+
+    def update_in_backward(self, grad_output):
+        self._data = self._diag_data(grad_output)
 
 
 class KronCovLinear(KronCurvature):

@@ -286,10 +286,12 @@ def update_ema_all(curvs):
             c._l2_reg_ema = c._l2_reg * beta + c._l2_reg_ema * (1 - beta)
     for beta, (xs, ys) in by_beta.items():
         _ops.axpby_batched(xs, ys, beta, 1 - beta)
+    xs, ys = [], []
     for c in curvs:
         if c.use_max_ema:
-            for e, e_max in zip(c.ema, c.ema_max):
-                torch.max(e, e_max, out=e_max)
+            xs.extend(c.ema)
+            ys.extend(c.ema_max)
+    _ops.max_batched(xs, ys)
 
 
 def update_inv_all(curvs):
@@ -338,11 +340,16 @@ def update_std_all(curvs):
         outs.extend(c.std)
     if mats:
         _ops.cholesky_upper_batched(mats, outs)
+    xs, ys = [], []
     for c in curvs:
         if c.kind == 'diag':
-            c.std = [i.sqrt() for i in c.inv]
+            if c.std is None or any(s.shape != i.shape for s, i in zip(c.std, c.inv)):
+                c.std = [torch.empty_like(i) for i in c.inv]
+            xs.extend(c.inv)
+            ys.extend(c.std)
         elif c.kind == 'full':
             raise NotImplementedError
+    _ops.sqrt_batched(xs, ys)
 
 
 def step_all(curvs, update_std=False, update_inv=True):
@@ -403,6 +410,7 @@ def sample_all(items):
     the generator (cov/linear.py:92-93, cov/conv.py:100-101,
     curvature.py:243-246); the products run batched afterwards."""
     by_scale = {}
+    d_mean, d_std, d_param, d_scale = [], [], [], []
     for c, params, mean, std_scale in items:
         if c.kind == 'kron':
             A_ic, G_ic = c.std
@@ -420,10 +428,18 @@ def sample_all(items):
             lst.append((G_ic, A_ic, noise, mean[0].contiguous(), mb, w, pb))
         elif c.kind == 'diag':
             for p, m, std in zip(params, mean, c.std):
-                noise = torch.randn_like(m)
-                p.data.copy_(torch.addcmul(m, noise, std, value=std_scale))
+                if not p.data.is_contiguous():
+                    p.data = p.data.contiguous()
+                # the noise is drawn straight into the parameter (same generator
+                # consumption as randn_like(m)) and turned into the sample in place
+                p.data.normal_()
+                d_mean.append(m.contiguous())
+                d_std.append(std)
+                d_param.append(p.data)
+                d_scale.append(float(std_scale))
         else:
             raise NotImplementedError
+    _ops.diag_sample_batched(d_mean, d_std, d_param, d_scale)
     for std_scale, lst in by_scale.items():
         _ops.sample_batched([x[0] for x in lst], [x[1] for x in lst], [x[2] for x in lst],
                             [x[3] for x in lst], [x[4] for x in lst], [x[5] for x in lst],

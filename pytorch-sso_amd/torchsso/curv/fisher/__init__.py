@@ -14,8 +14,8 @@ import torch.nn.functional as F
 
 from torchsso import _ops
 from torchsso.curv.cov.batchnorm import DiagCovBatchNorm2d
-from torchsso.curv.cov.conv import KronCovConv2d
-from torchsso.curv.cov.linear import KronCovLinear
+from torchsso.curv.cov.conv import DiagCovConv2d, KronCovConv2d
+from torchsso.curv.cov.linear import DiagCovLinear, KronCovLinear
 
 
 class Fisher(object):
@@ -42,6 +42,41 @@ class Fisher(object):
 
     def update_as_presoftmax(self, prob):
         raise NotImplementedError('This method supports only torchsso.KronFisherLinear.')
+
+
+class _DiagFisher(Fisher):
+    """Diagonal Fisher of a Linear / Conv2d layer: the per-sample gradients are
+    weighted by sqrt(prob) through the output gradient, so their squares carry
+    prob (reference: fisher/linear.py:5-35, fisher/conv.py:6-47)."""
+
+    def update_in_backward(self, grad_output):
+        if self.do_backward:
+            assert self.prob is not None
+            n = grad_output.shape[0]
+            pg = _ops.scale_rows(grad_output, self.prob.reshape(n), True)
+            data = self._diag_data(pg)
+            if self._acc is None:
+                self._acc = data
+            else:
+                _ops.axpby_batched([d.reshape(-1) for d in data],
+                                   [a.reshape(-1) for a in self._acc], 1., 1.)
+            self._data = self._acc
+        else:
+            self._data = self.finalize()
+
+
+class DiagFisherLinear(_DiagFisher, DiagCovLinear):
+
+    def __init__(self, *args, **kwargs):
+        DiagCovLinear.__init__(self, *args, **kwargs)
+        Fisher.__init__(self)
+
+
+class DiagFisherConv2d(_DiagFisher, DiagCovConv2d):
+
+    def __init__(self, *args, **kwargs):
+        DiagCovConv2d.__init__(self, *args, **kwargs)
+        Fisher.__init__(self)
 
 
 class KronFisherLinear(KronCovLinear, Fisher):

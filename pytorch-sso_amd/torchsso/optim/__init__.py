@@ -1,2 +1,2 @@
 from torchsso.optim.secondorder import SecondOrderOptimizer  # NOQA
-from torchsso.optim.vi import VIOptimizer  # NOQA
+from torchsso.optim.vi import VIOptimizer, VOGN  # NOQA

@@ -20,9 +20,15 @@ not installed; empty placeholder modules are put in sys.modules before the
 import so that the single-process classes load.  No reference file is modified
 or copied; only inputs and outputs (arrays) are saved.
 
-VIOptimizer's posterior sampling cannot be produced this way: the reference's
-`torchsso.utils.cholesky` exists for CuPy only (utils/cholesky_cupy.py:9-14).
-The VI case below therefore uses prior_variance=0 (no sampling, std_scale=0).
+VIOptimizer's posterior sampling with Kronecker curvature cannot be produced
+this way: the reference's `torchsso.utils.cholesky` exists for CuPy only
+(utils/cholesky_cupy.py:9-14).  The Kronecker VI case below therefore uses
+prior_variance=0 (no sampling, std_scale=0).  With diagonal curvature (VOGN) the
+std is an element-wise square root, so that case samples, and pins the order in
+which the generator is consumed (valid for CPU tensors only: a GPU generator
+yields other numbers).
+
+    python tests/golden/make_reference_vectors.py [case ...]     (default: all)
 """
 import os
 import sys
@@ -74,6 +80,8 @@ def snapshot(optimizer, out, tag):
 
 
 def run_case(torchsso, torch, nn, F, name, model, x, y, opt_cls, opt_args, steps):
+    if len(sys.argv) > 1 and name not in sys.argv[1:]:
+        return
     out = {'x': x.numpy().copy(), 'y': y.numpy().copy()}
     for k, v in model.state_dict().items():
         out['init.' + k] = v.numpy().copy()
@@ -134,6 +142,24 @@ def main():
              dict(dataset_size=100, curv_type='Cov', curv_shapes={'Linear': 'Kron'},
                   curv_kwargs={'damping': 1e-3, 'ema_decay': 0.95},
                   lr=0.05, momentum=0.9, num_mc_samples=3, prior_variance=0), steps=2)
+
+    # 4. VOGN: diagonal curvature for Conv2d / BatchNorm2d / Linear, with sampling
+    torch.manual_seed(0)
+    x = torch.randn(6, 2, 8, 8)
+    y = torch.randint(0, 5, (6,))
+    run_case(torchsso, torch, nn, F, 'ref_convnet_vogn', build_convnet(torch, nn), x, y,
+             torchsso.optim.VOGN,
+             dict(dataset_size=60, lr=0.01, num_mc_samples=2, warmup_kl_weighting_steps=None,
+                  curv_kwargs={'ema_decay': 0.1, 'damping': 1e-3}), steps=3)
+
+    # 5. the same without sampling (prior_variance=0), for runs on a GPU generator
+    torch.manual_seed(0)
+    x = torch.randn(6, 2, 8, 8)
+    y = torch.randint(0, 5, (6,))
+    run_case(torchsso, torch, nn, F, 'ref_convnet_vogn_nosample', build_convnet(torch, nn), x, y,
+             torchsso.optim.VOGN,
+             dict(dataset_size=60, lr=0.01, num_mc_samples=2, warmup_kl_weighting_steps=None,
+                  prior_variance=0, curv_kwargs={'ema_decay': 0.1, 'damping': 1e-3}), steps=3)
 
 
 if __name__ == '__main__':

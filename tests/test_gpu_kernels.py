@@ -312,6 +312,62 @@ def test_factor_linearity_at_full_size(ops, dev):
     assert O.rel_fro(one, u @ u.t()) < TOL
 
 
+# ---- diagonal covariance of Linear / Conv2d (VOGN) ------------------------------------
+
+@pytest.mark.parametrize('n,fin,fout,bias', [(1, 1, 1, True), (7, 5, 3, False), (128, 784, 1000, True),
+                                            (33, 130, 257, True), (256, 300, 10, False)])
+def test_diag_cov_linear(ops, dev, n, fin, fout, bias):
+    torch.manual_seed(n + fin)
+    a, g = torch.randn(n, fin), torch.randn(n, fout) * 1e-2
+    w, b = ops.diag_cov_linear(g.to(dev), a.to(dev), bias, float(n))
+    ref = O.diag_cov_linear(a, g, bias, None, D)
+    assert O.rel_fro(w, ref[0]) < TOL
+    if bias:
+        assert O.rel_fro(b, ref[1]) < TOL
+    else:
+        assert b is None
+
+
+@pytest.mark.parametrize('shape,cout,k,s,p,d', [
+    ((2, 3, 8, 8), 4, (3, 3), (1, 1), (1, 1), (1, 1)),
+    ((5, 3, 9, 8), 4, (3, 2), (2, 1), (1, 0), (1, 2)),
+    ((128, 3, 32, 32), 64, (5, 5), (1, 1), (0, 0), (1, 1)),       # config 2, conv1
+    ((16, 64, 14, 14), 130, (5, 5), (1, 1), (0, 0), (1, 1)),      # several tiles, split over samples
+    ((3, 200, 7, 7), 140, (3, 3), (2, 2), (1, 1), (1, 1)),
+    ((1, 1, 1, 1), 1, (1, 1), (1, 1), (0, 0), (1, 1)),
+])
+def test_diag_cov_conv2d(ops, dev, shape, cout, k, s, p, d):
+    torch.manual_seed(sum(shape) + cout)
+    x = torch.randn(*shape)
+    oh = O.conv_out_size(shape[2], k[0], s[0], p[0], d[0])
+    ow = O.conv_out_size(shape[3], k[1], s[1], p[1], d[1])
+    g = torch.randn(shape[0], cout, oh, ow) * 1e-2
+    out = ops.diag_cov_conv2d(g.to(dev), x.to(dev), k, s, p, d, float(shape[0]))
+    ref = O.diag_cov_conv2d(x, g, k, s, p, d, False, None, D)[0]
+    assert O.rel_fro(out.reshape(ref.shape), ref) < TOL
+
+
+def test_diag_element_wise_tails(ops, dev):
+    torch.manual_seed(11)
+    xs = [torch.rand(n) + 0.1 for n in (1, 7, 1000, 4097)]
+    ys = [torch.empty(n, device=dev) for n in (1, 7, 1000, 4097)]
+    ops.sqrt_batched([x.to(dev) for x in xs], ys)
+    for x, y in zip(xs, ys):
+        assert O.rel_fro(y, x.double().sqrt()) < 1e-6
+    old = [torch.rand(n) for n in (1, 7, 1000, 4097)]
+    ys = [o.to(dev) for o in old]
+    ops.max_batched([x.to(dev) for x in xs], ys)
+    for x, o, y in zip(xs, old, ys):
+        assert torch.equal(y.cpu(), torch.max(x, o))
+    means = [torch.randn(n) for n in (3, 1025)]
+    stds = [torch.rand(n) for n in (3, 1025)]
+    noise = [torch.randn(n) for n in (3, 1025)]
+    ps = [e.to(dev) for e in noise]
+    ops.diag_sample_batched([m.to(dev) for m in means], [s.to(dev) for s in stds], ps, [0.5, 2.0])
+    for m, s, e, p, sc in zip(means, stds, noise, ps, (0.5, 2.0)):
+        assert O.rel_fro(p, m.double() + sc * e.double() * s.double()) < 1e-6
+
+
 # ---- Fisher weighting ---------------------------------------------------------------
 
 def test_fisher_weighted_factors(ops, dev):
@@ -339,6 +395,19 @@ def test_fisher_weighted_factors(ops, dev):
     wc, bc = ops.bn_diag_combine(sx, sg, 8.0, True)
     ref = O.fisher_bn_diag(O.bn_restore_input(out.double(), w.double(), b.double()), g4, prob, True, D)
     assert O.rel_fro(wc, ref[0]) < TOL and O.rel_fro(bc, ref[1]) < TOL
+    # diagonal Fisher of Linear / Conv2d: sqrt(prob) on the output gradient, then the Cov kernels
+    a = torch.randn(n, 50)
+    prob = torch.rand(n)
+    pg = ops.scale_rows(g.to(dev), prob.to(dev), True)
+    dw, db = ops.diag_cov_linear(pg, a.to(dev), True, float(n))
+    ref = O.diag_cov_linear(a, g, True, prob, D)
+    assert O.rel_fro(dw, ref[0]) < TOL and O.rel_fro(db, ref[1]) < TOL
+    x4 = torch.randn(8, 6, 7, 8)
+    prob = torch.rand(8)
+    pg = ops.scale_rows(g4.to(dev), prob.to(dev), True)
+    dw = ops.diag_cov_conv2d(pg, x4.to(dev), (3, 3), (1, 1), (0, 0), (1, 1), 8.0)
+    ref = O.diag_cov_conv2d(x4, g4, (3, 3), (1, 1), (0, 0), (1, 1), False, prob, D)[0]
+    assert O.rel_fro(dw.reshape(ref.shape), ref) < TOL
 
 
 def test_factor_input_above_one_gib_is_consumed_in_slices(ops, dev):

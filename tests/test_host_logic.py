@@ -85,6 +85,27 @@ def test_vi_optimizer_accumulation_matches_reference(oracle_ops):
     T.compare_with_golden(snaps, gold, 2e-4)
 
 
+def test_vogn_matches_reference_with_sampling(oracle_ops):
+    """VOGN (diagonal curvature everywhere) against the vectors the reference wrote
+    on CPU, posterior sampling included: pins the diagonal Conv2d/Linear/BatchNorm
+    curvature, the element-wise std and the order and shape in which the
+    generator is consumed (one draw per parameter, in param_group order)."""
+    gold = T.load_golden('ref_convnet_vogn')
+    model = T.load_init(T.build_convnet(), gold)
+    x, y = torch.from_numpy(gold['x']), torch.from_numpy(gold['y'])
+    opt = torchsso.optim.VOGN(model, 60, lr=0.01, num_mc_samples=2,
+                              warmup_kl_weighting_steps=None,
+                              curv_kwargs={'ema_decay': 0.1, 'damping': 1e-3})
+    names = [type(g['curv']).__name__ for g in opt.param_groups]
+    assert names == ['DiagCovConv2d', 'DiagCovBatchNorm2d', 'DiagCovConv2d', 'DiagCovLinear']
+    snaps = []
+    for s in range(3):
+        loss, _ = opt.step(closure=_closure(model, x, y))
+        assert abs(loss.item() - float(gold['step%d.loss' % s])) < 1e-3 * max(1, abs(loss.item()))
+        snaps.append(T.snapshot_optimizer(opt))
+    T.compare_with_golden(snaps, gold, 2e-4)
+
+
 def test_vi_sampling_consumes_generator_in_group_order(oracle_ops):
     """With a std present, params = mean + std_scale * U_G E U_A with E drawn by
     torch.randn in param_group order after manual_seed(step + seed)."""

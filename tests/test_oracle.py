@@ -159,6 +159,60 @@ def test_bn_diag_is_mean_of_squared_per_sample_grads():
     assert torch.allclose(w2, ref_w * n * n, atol=1e-8)
 
 
+def test_diag_cov_is_mean_of_squared_per_sample_grads():
+    """DiagCovLinear / DiagCovConv2d: with the layer's real output gradient of a
+    mean-reduced loss, n^2-rescaled data == mean over samples of the squared gradient
+    of that sample's own loss, taken sample by sample through autograd.  The conv
+    bias entry is the reference's sum of squares (not the squared sum that the
+    per-sample bias gradient would give), checked by loops."""
+    torch.manual_seed(12)
+    n = 5
+    lin = nn.Linear(7, 4).double()
+    x = torch.randn(n, 7, dtype=D)
+    y = torch.randint(0, 4, (n,))
+    out = lin(x)
+    out.retain_grad()
+    F.cross_entropy(out, y).backward()
+    w, b = O.diag_cov_linear(x, out.grad, True, None, D)
+    ref_w, ref_b = torch.zeros_like(lin.weight), torch.zeros_like(lin.bias)
+    for i in range(n):
+        gw, gb = torch.autograd.grad(F.cross_entropy(lin(x[i:i + 1]), y[i:i + 1]), [lin.weight, lin.bias])
+        ref_w += gw ** 2 / n
+        ref_b += gb ** 2 / n
+    assert torch.allclose(w, ref_w, atol=1e-12) and torch.allclose(b, ref_b, atol=1e-12)
+    # prob weighting scales each sample's squared gradient
+    prob = torch.rand(n, dtype=D)
+    wp, bp = O.diag_cov_linear(x, out.grad, True, prob, D)
+    ref_w.zero_()
+    for i in range(n):
+        gw, = torch.autograd.grad(F.cross_entropy(lin(x[i:i + 1]), y[i:i + 1]), [lin.weight])
+        ref_w += prob[i] * gw ** 2 / n
+    assert torch.allclose(wp, ref_w, atol=1e-12)
+
+    conv = nn.Conv2d(3, 4, (3, 2), stride=(2, 1), padding=(1, 0), dilation=(1, 2)).double()
+    xc = torch.randn(n, 3, 9, 8, dtype=D)
+    oc = conv(xc)
+    oc.retain_grad()
+    head = torch.randn(oc[0].numel(), 4, dtype=D)
+    F.cross_entropy(oc.reshape(n, -1) @ head, y).backward()
+    w, b = O.diag_cov_conv2d(xc, oc.grad, (3, 2), (2, 1), (1, 0), (1, 2), True, None, D)
+    assert w.shape == conv.weight.shape
+    ref_w = torch.zeros_like(conv.weight)
+    for i in range(n):
+        li = F.cross_entropy(conv(xc[i:i + 1]).reshape(1, -1) @ head, y[i:i + 1])
+        gw, = torch.autograd.grad(li, [conv.weight])
+        ref_w += gw ** 2 / n
+    assert torch.allclose(w, ref_w, atol=1e-12)
+    g = oc.grad
+    ref_b = torch.zeros(4, dtype=D)
+    for i in range(n):
+        for c in range(4):
+            for r in range(g.shape[2]):
+                for q in range(g.shape[3]):
+                    ref_b[c] += g[i, c, r, q] ** 2
+    assert torch.allclose(b, ref_b * n, atol=1e-12)          # mean over n, times n^2
+
+
 # ---- EMA / accumulate -------------------------------------------------------
 
 def test_ema_weights_new_data_and_first_call_copies():
