@@ -147,6 +147,30 @@ class Curvature(object):
     def update_in_backward(self, grad_output):
         raise NotImplementedError
 
+    # ---- checkpointing --------------------------------------------------------
+
+    _STATE_LISTS = ('ema', 'ema_max', 'inv', 'std')
+
+    def state_dict(self):
+        """The running state as tensors and numbers only: ema, ema_max, inv, std
+        (lists of tensors or None) and the two l2 scalars.  (The reference has no
+        such method: its optimizer checkpoint pickles the Curvature objects, hooks
+        and module included.)"""
+        out = {'l2_reg': float(self._l2_reg), 'l2_reg_ema': float(self._l2_reg_ema)}
+        for name in self._STATE_LISTS:
+            val = getattr(self, name)
+            out[name] = None if val is None else [t.detach().clone() for t in val]
+        return out
+
+    def load_state_dict(self, state):
+        device = self.device
+        self._l2_reg = state['l2_reg']
+        self._l2_reg_ema = state['l2_reg_ema']
+        for name in self._STATE_LISTS:
+            val = state.get(name)
+            setattr(self, name, None if val is None
+                    else [t.detach().to(device=device, dtype=torch.float32).clone() for t in val])
+
     # ---- per-layer step (wrappers over the list-based engine calls) --------
 
     def step(self, update_std=False, update_inv=True):

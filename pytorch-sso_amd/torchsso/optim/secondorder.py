@@ -12,9 +12,9 @@ into the HIP engine:
     precondition phase   G^-1 [dW|db] A^-1 for all layers      (two MFMA launches)
     update phase         weight decay, momentum, p -= lr * g   (one fused kernel)
 
-Options that need norms or extra buffers (raw-gradient momentum, gradient EMA,
-bias correction, LARS, weight normalisation) run as in-place torch tensor ops
-on the device, in the reference's order.
+Raw-gradient momentum, gradient EMA and bias correction run on the same
+element-wise kernels in the reference's order; LARS and weight normalisation
+need tensor norms on the host and use torch's norm() for them.
 """
 import math
 
@@ -140,6 +140,58 @@ class SecondOrderOptimizer(Optimizer):
         assert curv_class is not None, f"Failed to lookup Curvature class {curv_name} for {module}."
 
         return curv_class
+
+    # ----------------------------------------------------------- checkpointing
+
+    _GROUP_OBJECTS = ('params', 'curv', 'acc_curv', 'acc_grads', 'mean')
+
+    def state_dict(self):
+        """Checkpoint of tensors, numbers and strings only (loadable with
+        torch.load(..., weights_only=True)): the step counters and, per param
+        group, its options (lr, momentum, ...), the curvature's ema / inv / std, the
+        momentum and gradient-EMA buffers and, for VI, the posterior means.
+        torch's default would pickle the Curvature objects held in param_groups, as
+        the reference's checkpoints do."""
+        groups = []
+        for group in self.param_groups:
+            entry = {'options': {k: v for k, v in group.items() if k not in self._GROUP_OBJECTS}}
+            curv = group['curv']
+            entry['curvature'] = None if curv is None else curv.state_dict()
+            for target in ('params', 'mean'):
+                if target not in group:
+                    continue
+                entry[target + '_buffers'] = [
+                    {k: v.detach().clone() for k, v in self.state[t].items() if torch.is_tensor(v)}
+                    for t in group[target]]
+            if 'mean' in group:
+                entry['mean'] = [m.detach().clone() for m in group['mean']]
+            groups.append(entry)
+        return {'optim_state': dict(self.optim_state), 'groups': groups}
+
+    def load_state_dict(self, state_dict):
+        groups = state_dict['groups']
+        if len(groups) != len(self.param_groups):
+            raise ValueError('checkpoint has %d param groups, the optimizer has %d'
+                             % (len(groups), len(self.param_groups)))
+        for group, entry in zip(self.param_groups, groups):
+            group.update(entry['options'])
+            curv = group['curv']
+            if curv is not None and entry['curvature'] is not None:
+                curv.load_state_dict(entry['curvature'])
+            for target in ('params', 'mean'):
+                bufs = entry.get(target + '_buffers')
+                if bufs is None or target not in group:
+                    continue
+                if len(bufs) != len(group[target]):
+                    raise ValueError('checkpoint group has %d %s, the optimizer has %d'
+                                     % (len(bufs), target, len(group[target])))
+                for t, saved in zip(group[target], bufs):
+                    for k, v in saved.items():
+                        self.state[t][k] = v.detach().to(device=t.device, dtype=t.dtype).clone()
+            if 'mean' in entry and 'mean' in group:
+                for m, saved in zip(group['mean'], entry['mean']):
+                    m.data.copy_(saved)
+        self.optim_state = dict(state_dict['optim_state'])
 
     # ------------------------------------------------------------------ step
 
@@ -304,8 +356,8 @@ class SecondOrderOptimizer(Optimizer):
             bias_correction2 = 1 - beta2 ** self.optim_state['step']
             if getattr(curv, 'use_sqrt_ema', False):
                 bias_correction2 = math.sqrt(bias_correction2)
-            for p in params:
-                p.grad.mul_(bias_correction2 / bias_correction1)
+            grads = [p.grad for p in params]
+            _ops.axpby_batched(grads, grads, bias_correction2 / bias_correction1, 0.)
 
         if group['lars_type'] == grad_type and group['lars']:
             thr, eps = 1e-2, 1e-9

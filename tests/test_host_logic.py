@@ -158,6 +158,102 @@ def test_accumulation_steps_average_gradients_and_factors(oracle_ops):
     assert torch.allclose(opt.param_groups[0]['curv'].ema[0], 0.5 * (A0 + A1), atol=1e-6)
 
 
+def test_checkpoint_is_tensor_only_and_resumes_exactly(oracle_ops, tmp_path):
+    import copy
+    gold = T.load_golden('ref_convnet_kfac')
+    x, y = torch.from_numpy(gold['x']), torch.from_numpy(gold['y'])
+
+    def make(model):
+        return torchsso.optim.SecondOrderOptimizer(
+            model, 'Cov', {'Linear': 'Kron', 'Conv2d': 'Kron', 'BatchNorm2d': 'Diag'},
+            {'damping': 1e-2, 'ema_decay': 0.9}, lr=0.02, momentum=0.5, l2_reg=1e-4)
+
+    model = T.load_init(T.build_convnet(), gold)
+    opt = make(model)
+    for _ in range(2):
+        opt.step(closure=_closure(model, x, y))
+    path = str(tmp_path / 'ckpt.pt')
+    torch.save({'model': model.state_dict(), 'optimizer': opt.state_dict()}, path)
+    # nothing but tensors, numbers, strings and containers: the safe loader accepts it
+    ckpt = torch.load(path, weights_only=True)
+
+    model2 = T.build_convnet()
+    model2.load_state_dict(ckpt['model'])
+    opt2 = make(model2)
+    opt2.param_groups[0]['lr'] = 123.          # overwritten by the checkpoint
+    opt2.load_state_dict(ckpt['optimizer'])
+    assert opt2.optim_state == opt.optim_state and opt2.param_groups[0]['lr'] == 0.02
+    for g, g2 in zip(opt.param_groups, opt2.param_groups):
+        assert g2['curv'].damping == g['curv'].damping
+        for a, b in zip(g['curv'].ema, g2['curv'].ema):
+            assert torch.equal(a, b) and a.data_ptr() != b.data_ptr()
+    opt.step(closure=_closure(model, x, y))
+    opt2.step(closure=_closure(model2, x, y))
+    for p, q in zip(model.parameters(), model2.parameters()):
+        assert torch.equal(p, q)
+
+    # VI: the posterior means and their momentum buffers travel too
+    vm = T.load_init(T.build_mlp(), T.load_golden('ref_mlp_vi_nosample'))
+    vx, vy = torch.randn(8, 12), torch.randint(0, 5, (8,))
+    vargs = dict(curv_kwargs={'damping': 1e-3, 'ema_decay': 0.95}, lr=0.05, momentum=0.9,
+                 num_mc_samples=2)
+    vopt = torchsso.optim.VIOptimizer(vm, 100, 'Cov', {'Linear': 'Kron'}, **vargs)
+    vopt.step(closure=_closure(vm, vx, vy))
+    sd = copy.deepcopy(vopt.state_dict())
+    vm2 = T.build_mlp()
+    vm2.load_state_dict(vm.state_dict())
+    vopt2 = torchsso.optim.VIOptimizer(vm2, 100, 'Cov', {'Linear': 'Kron'}, **vargs)
+    vopt2.load_state_dict(sd)
+    la, _ = vopt.step(closure=_closure(vm, vx, vy))
+    lb, _ = vopt2.step(closure=_closure(vm2, vx, vy))
+    assert la.item() == lb.item()
+    for g, g2 in zip(vopt.param_groups, vopt2.param_groups):
+        for a, b in zip(g['mean'], g2['mean']):
+            assert torch.equal(a, b)
+
+
+def test_iteration_lr_schedules():
+    from torchsso.optim import lr_scheduler as L
+    model = nn.Linear(3, 2)
+    opt = torch.optim.SGD(model.parameters(), lr=0.4, momentum=0.9)
+    with pytest.raises(TypeError):
+        L.PolynomialDecayIterLR(model, rate=2, max_count=10)
+    sched = L.PolynomialDecayIterLR(opt, rate=2, max_count=10, start_iter=2)
+    lrs = []
+    for _ in range(12):
+        sched.step()
+        lrs.append(opt.param_groups[0]['lr'])
+    # iterations 0, 1: untouched; from 2 on: 0.4 * (1 - (t - 2) / 8)^2, clamped at 0
+    want = [0.4, 0.4] + [0.4 * max(1 - (t - 2) / 8, 0) ** 2 for t in range(2, 12)]
+    assert lrs == pytest.approx(want, abs=1e-15)
+    assert sched.state_dict()['last_iter'] == 11 and 'optimizer' not in sched.state_dict()
+
+    opt = torch.optim.SGD(model.parameters(), lr=0.4, momentum=0.9)
+    sched = L.PolynomialDecayIterLR(opt, rate=1, max_count=10, target=0.1)
+    seen = []
+    for _ in range(9):
+        sched.step()
+        seen.append(opt.param_groups[0]['lr'])
+    assert seen == pytest.approx([max(0.4 * (1 - t / 10), 0.1) for t in range(9)], abs=1e-15)
+
+    opt = torch.optim.SGD(model.parameters(), lr=0.4, momentum=0.9)
+    warm = L.MomentumCorrectionLR(L.GradualWarmupIterLR(opt, initial_lr=0.1, max_count=4))
+    assert opt.param_groups[0]['init_momentum'] == 0.9 and warm.max_count == 4
+    lrs, moms = [], []
+    for _ in range(6):
+        warm.step()
+        lrs.append(opt.param_groups[0]['lr'])
+        moms.append(opt.param_groups[0]['momentum'])
+    assert lrs == pytest.approx([0.1, 0.175, 0.25, 0.325, 0.4, 0.4], abs=1e-15)
+    # momentum follows lr / previous lr (first step: no previous rate)
+    assert moms[0] == 0.9 and moms[2] == pytest.approx(0.9 * 0.25 / 0.175)
+    assert moms[5] == pytest.approx(0.9)
+    # resuming needs initial_lr in the groups
+    fresh = torch.optim.SGD(model.parameters(), lr=0.4)
+    with pytest.raises(KeyError):
+        L.GradualWarmupIterLR(fresh, 0.0, 4, last_iter=3)
+
+
 def test_constructor_validation_and_class_lookup():
     model = nn.Sequential(nn.Linear(4, 3))
     kw = dict(curv_type='Cov', curv_shapes={'Linear': 'Kron'}, curv_kwargs={'damping': 1e-3})
