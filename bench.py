@@ -27,10 +27,15 @@ sys.path.insert(0, ROOT)
 
 METRIC = 'K-FAC step ms (factor+invert+precondition) & fp32 MFMA TFLOP/s, 1 MI355X'
 PEAK_FP32_MFMA_TFLOPS = 157.3
-# HBM bytes per syrk_kernel launch, averaged over the 108 launches of a resnet50 step, from two
-# rocprofv3 --pmc runs (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration with a 1 GiB copy):
-# 39.5 MB read + 22.5 MB written.
-RESNET50_SYRK_TRAFFIC_BYTES = 62.0e6
+# HBM bytes per launch of the factor-build kernels (syrk_kernel, corr_kernel and their reduce /
+# assemble kernels), averaged over the 226 launches of a resnet50 step, from two rocprofv3 --pmc runs
+# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration with a 1 GiB copy): 52.7 MB read + 15.7 MB
+# written.
+RESNET50_FACTOR_TRAFFIC_BYTES = 68.4e6
+# flops the matrix cores execute for the factor products of one resnet50 step
+# (512 x SQ_INSTS_VALU_MFMA_MOPS_F32 from a rocprofv3 --pmc run): the symmetric products run one
+# triangle, and the stride-1 3x3 layers take 13 spatial correlations instead of 45 block products
+RESNET50_FACTOR_EXECUTED_FLOP = 560.6e9
 
 
 # ---------------------------------------------------------------------------
@@ -407,12 +412,21 @@ def main():
                           'invert': round(work['inverse'] / inv_ms / 1e9, 2),
                           'precondition': round(work['precondition'] / pre_ms / 1e9, 2)},
         'not_spd_factors': not_spd,
-        'roofline': {'bound': 'mfma', 'kernel': 'syrk_kernel (Kronecker factor build, all layers)',
+        'roofline': {'bound': 'mfma',
+                     'kernel': 'Kronecker factor build, all layers (syrk_kernel, corr_kernel)',
                      'achieved': round(work['factor'] / f_ms / 1e9, 2),
                      'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
                      'frac': round(work['factor'] / f_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4),
-                     'traffic': RESNET50_SYRK_TRAFFIC_BYTES if args.workload == 'resnet50' else None},
+                     'traffic': RESNET50_FACTOR_TRAFFIC_BYTES if args.workload == 'resnet50' else None,
+                     'note': 'achieved counts the algorithmic flops 2*d^2*L of every factor (dense '
+                             'convention); the kernels execute fewer (one triangle of each symmetric '
+                             'product, shared spatial correlations for stride-1 kxk convolutions), so '
+                             'frac can exceed 1; executed_* is what the matrix cores really do'},
     }
+    if args.workload == 'resnet50':
+        ex = RESNET50_FACTOR_EXECUTED_FLOP / f_ms / 1e9
+        out['roofline']['executed_tflops'] = round(ex, 2)
+        out['roofline']['executed_frac'] = round(ex / PEAK_FP32_MFMA_TFLOPS, 4)
     if not args.no_cpu_baseline:
         cpu_ms, cores, sample = run_cpu_baseline(specs, batch)
         out['cpu_baseline'] = {'value': round(cpu_ms, 1), 'unit': 'ms', 'cores': cores,
