@@ -199,6 +199,14 @@ struct indexed_epilogue : std::false_type {};
 template <class T>
 struct indexed_epilogue<T, std::void_t<decltype(T::indexed)>> : std::bool_constant<T::indexed> {};
 
+// An epilogue with `static constexpr bool reads_output = true` offers
+// reads() / fetch(row, col) / store_with(row, col, v, old) next to store().
+template <class T, class = void>
+struct reading_epilogue : std::false_type {};
+template <class T>
+struct reading_epilogue<T, std::void_t<decltype(T::reads_output)>>
+    : std::bool_constant<T::reads_output> {};
+
 // Position in C of accumulator element i of block (a, b) of the calling thread;
 // the epilogue visits (a, b, i) in lexicographic order, 64 elements per thread.
 template <int WM, int WN>
@@ -304,6 +312,34 @@ __device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0
     __syncthreads();
   }
 
+  if constexpr (reading_epilogue<EPI>::value) {
+    // C = alpha*acc + beta*C_old: the old values are loaded 32 at a time ahead of the
+    // stores.  Interleaved load/store pairs would each wait for their own load (a store
+    // to C may alias the next load of C, so the compiler keeps them in order).
+    if (epi.reads()) {
+#pragma unroll
+      for (int a = 0; a < 2; ++a) {
+        float old[32];
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            int row, col;
+            acc_coords<WM, WN>(m0, n0, a, b, i, row, col);
+            old[b * 16 + i] = epi.fetch(row, col);
+          }
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            int row, col;
+            acc_coords<WM, WN>(m0, n0, a, b, i, row, col);
+            epi.store_with(row, col, acc[a][b][i], old[b * 16 + i]);
+          }
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int a = 0; a < 2; ++a)
 #pragma unroll

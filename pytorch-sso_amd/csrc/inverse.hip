@@ -358,7 +358,7 @@ __global__ __launch_bounds__(NTHREADS) void potrf_panel_kernel(const MatDesc* ta
 // which cuts the read-modify-write passes over the trailing matrix by that factor.
 constexpr int OUTER_BLOCKS = 4;
 
-__global__ __launch_bounds__(NTHREADS) void potrf_trail_kernel(const MatDesc* table, int kb0,
+__global__ __launch_bounds__(NTHREADS, 3) void potrf_trail_kernel(const MatDesc* table, int kb0,
                                                                int nk, int row_lo, int row_hi) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   const MatDesc m = table[blockIdx.y];

@@ -166,10 +166,22 @@ struct ConvA {
 
 // C[row][col] = alpha*acc + beta*C_old ; optionally also the mirrored element.
 struct EpiStore {
+  static constexpr bool reads_output = true;
   float* C;
   int ld, M, N;
   float alpha, beta;
   bool mirror;
+  __device__ __forceinline__ bool reads() const { return beta != 0.f; }
+  __device__ __forceinline__ float fetch(int row, int col) const {
+    return (row < M && col < N) ? C[(size_t)row * ld + col] : 0.f;
+  }
+  __device__ __forceinline__ void store_with(int row, int col, float v, float old) const {
+    if (row < M && col < N) {
+      const float o = alpha * v + beta * old;
+      C[(size_t)row * ld + col] = o;
+      if (mirror && row != col) C[(size_t)col * ld + row] = o;
+    }
+  }
   __device__ __forceinline__ void store(int row, int col, float v) const {
     if (row < M && col < N) {
       const size_t idx = (size_t)row * ld + col;
