@@ -32,80 +32,99 @@ constexpr int EW_THREADS = 256;
 constexpr int EW_PER_THREAD = 4;
 constexpr int EW_BLOCK = EW_THREADS * EW_PER_THREAD;
 
-template <int OP>
-__device__ __forceinline__ void apply(const VecDesc& m, long i) {
-  if (OP == OP_AXPBY) {
-    // b = s0 * a + s1 * b     (s1 == 0: b is not read)
-    float v = m.s0 * m.a[i];
-    if (m.s1 != 0.f) v += m.s1 * m.b[i];
-    m.b[i] = v;
-  } else if (OP == OP_DIAG_INV) {
-    // b = 1 / ((s1 ? sqrt(a) : a) + s0)
-    float v = m.a[i];
-    if (m.s1 != 0.f) v = sqrtf(v);
-    m.b[i] = 1.f / (v + m.s0);
-  } else if (OP == OP_MUL) {
-    // b *= a
-    m.b[i] = m.b[i] * m.a[i];
-  } else if (OP == OP_SQRT) {
-    m.b[i] = sqrtf(m.a[i]);
-  } else if (OP == OP_MAX) {
-    m.b[i] = fmaxf(m.a[i], m.b[i]);
-  } else if (OP == OP_ADDCMUL) {
-    // b = a + s0 * b * c     (a = mean, b = noise in / parameter out, c = std)
-    m.b[i] = fmaf(m.s0 * m.b[i], m.c[i], m.a[i]);
-  } else {
-    // a = param, b = grad, c = momentum buffer; s0 = lr, s1 = momentum, s2 = weight decay
-    float g = m.b[i];
-    const float p = m.a[i];
-    if (m.s2 != 0.f) g += m.s2 * p;
-    if (m.s1 != 0.f) {
-      g = m.s1 * m.c[i] + g;
-      m.c[i] = g;
-    }
-    m.b[i] = g;
-    m.a[i] = p - m.s0 * g;
-  }
-}
-
+// Each thread handles EW_PER_THREAD elements: all loads first, then the
+// arithmetic, then all stores.  (Load/store pairs issued one element at a time
+// would each wait for their own load: a store may alias the next load, so the
+// compiler keeps them in order.)
 template <int OP>
 __global__ __launch_bounds__(EW_THREADS) void vec_kernel(const VecDesc* table) {
   const VecDesc m = table[blockIdx.y];
   const long nblocks = (m.numel + EW_BLOCK - 1) / EW_BLOCK;
+  constexpr bool USES_B = OP == OP_AXPBY || OP == OP_MUL || OP == OP_SGD || OP == OP_MAX ||
+                          OP == OP_ADDCMUL;
+  constexpr bool USES_C = OP == OP_SGD || OP == OP_ADDCMUL;
   for (long blk = blockIdx.x; blk < nblocks; blk += gridDim.x) {
     const long base = blk * EW_BLOCK + threadIdx.x;
+    float a[EW_PER_THREAD], b[EW_PER_THREAD], c[EW_PER_THREAD];
 #pragma unroll
     for (int k = 0; k < EW_PER_THREAD; ++k) {
       const long i = base + (long)k * EW_THREADS;
-      if (i < m.numel) apply<OP>(m, i);
+      const bool in = i < m.numel;
+      a[k] = in ? m.a[i] : 0.f;
+      b[k] = 0.f;
+      c[k] = 0.f;
+      if (USES_B && in && !(OP == OP_AXPBY && m.s1 == 0.f)) b[k] = m.b[i];
+      if (USES_C && in && !(OP == OP_SGD && m.s1 == 0.f)) c[k] = m.c[i];
+    }
+#pragma unroll
+    for (int k = 0; k < EW_PER_THREAD; ++k) {
+      const long i = base + (long)k * EW_THREADS;
+      if (i >= m.numel) continue;
+      if (OP == OP_AXPBY) {
+        // b = s0 * a + s1 * b     (s1 == 0: b is not read)
+        float v = m.s0 * a[k];
+        if (m.s1 != 0.f) v += m.s1 * b[k];
+        m.b[i] = v;
+      } else if (OP == OP_DIAG_INV) {
+        // b = 1 / ((s1 ? sqrt(a) : a) + s0)
+        float v = a[k];
+        if (m.s1 != 0.f) v = sqrtf(v);
+        m.b[i] = 1.f / (v + m.s0);
+      } else if (OP == OP_MUL) {
+        m.b[i] = b[k] * a[k];                       // b *= a
+      } else if (OP == OP_SQRT) {
+        m.b[i] = sqrtf(a[k]);
+      } else if (OP == OP_MAX) {
+        m.b[i] = fmaxf(a[k], b[k]);
+      } else if (OP == OP_ADDCMUL) {
+        // b = a + s0 * b * c     (a = mean, b = noise in / parameter out, c = std)
+        m.b[i] = fmaf(m.s0 * b[k], c[k], a[k]);
+      } else {
+        // a = param, b = grad, c = momentum buffer; s0 = lr, s1 = momentum, s2 = weight decay
+        float g = b[k];
+        const float p = a[k];
+        if (m.s2 != 0.f) g += m.s2 * p;
+        if (m.s1 != 0.f) {
+          g = m.s1 * c[k] + g;
+          m.c[i] = g;
+        }
+        m.b[i] = g;
+        m.a[i] = p - m.s0 * g;
+      }
     }
   }
 }
 
 // y = s0*x + s1*y on float4 (all pointers 16-byte aligned, numel % 4 == 0): the
-// running average of the factors moves the most bytes of all tails
+// running average of the factors moves the most bytes of all tails.  Four float4
+// per thread and iteration, loads ahead of stores.
 __global__ __launch_bounds__(EW_THREADS) void axpby4_kernel(const VecDesc* table) {
   const VecDesc m = table[blockIdx.y];
   const long n4 = m.numel >> 2;
   const float4* x = reinterpret_cast<const float4*>(m.a);
   float4* y = reinterpret_cast<float4*>(m.b);
   const long stride = (long)gridDim.x * EW_THREADS;
-  for (long i = (long)blockIdx.x * EW_THREADS + threadIdx.x; i < n4; i += stride) {
-    const float4 a = x[i];
-    float4 o;
-    if (m.s1 != 0.f) {
-      const float4 b = y[i];
-      o.x = m.s0 * a.x + m.s1 * b.x;
-      o.y = m.s0 * a.y + m.s1 * b.y;
-      o.z = m.s0 * a.z + m.s1 * b.z;
-      o.w = m.s0 * a.w + m.s1 * b.w;
-    } else {
-      o.x = m.s0 * a.x;
-      o.y = m.s0 * a.y;
-      o.z = m.s0 * a.z;
-      o.w = m.s0 * a.w;
+  const bool rd = m.s1 != 0.f;
+  for (long i0 = (long)blockIdx.x * EW_THREADS + threadIdx.x; i0 < n4; i0 += 4 * stride) {
+    float4 a[4], b[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const long i = i0 + k * stride;
+      a[k] = i < n4 ? x[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+      b[k] = (rd && i < n4) ? y[i] : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    y[i] = o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const long i = i0 + k * stride;
+      if (i < n4) {
+        float4 o;
+        o.x = m.s0 * a[k].x + m.s1 * b[k].x;
+        o.y = m.s0 * a[k].y + m.s1 * b[k].y;
+        o.z = m.s0 * a[k].z + m.s1 * b[k].z;
+        o.w = m.s0 * a[k].w + m.s1 * b[k].w;
+        y[i] = o;
+      }
+    }
   }
 }
 

@@ -48,6 +48,23 @@ struct EpiSplit {
   const float* mb;
   int dG, dA, dAw;
   float scale;
+  static constexpr bool reads_output = true;     // the means, when sampling
+  __device__ __forceinline__ bool reads() const { return mW != nullptr; }
+  __device__ __forceinline__ float fetch(int row, int col) const {
+    if (row < dG && col < dA) {
+      if (col < dAw) return mW[(size_t)row * dAw + col];
+      return mb ? mb[row] : 0.f;
+    }
+    return 0.f;
+  }
+  __device__ __forceinline__ void store_with(int row, int col, float v, float old) const {
+    if (row < dG && col < dA) {
+      if (col < dAw)
+        W[(size_t)row * dAw + col] = old + scale * v;
+      else
+        b[row] = old + scale * v;
+    }
+  }
   __device__ __forceinline__ void store(int row, int col, float v) const {
     if (row < dG && col < dA) {
       if (col < dAw) {
