@@ -259,18 +259,30 @@ __global__ __launch_bounds__(256) void scale_rows_kernel(const float* x, const f
 }
 
 // w_curv[c] = alpha * sum_n sx[n][c] * sg[n][c] ; b_curv[c] = alpha * sum_n sg[n][c]
-__global__ void bn_combine_kernel(const float* sx, const float* sg, int N, int C, float alpha,
-                                  float* w_curv, float* b_curv) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= C) return;
+// 64 channels x 4 slices of n per workgroup: the loads of a thread are independent,
+// and the four slice sums are added in slice order.
+__global__ __launch_bounds__(256) void bn_combine_kernel(const float* sx, const float* sg, int N,
+                                                         int C, float alpha, float* w_curv,
+                                                         float* b_curv) {
+  __shared__ float rw[4][64], rb[4][64];
+  const int lane = threadIdx.x & 63, slice = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + lane;
   float sw = 0.f, sb = 0.f;
-  for (int n = 0; n < N; ++n) {
-    const float g = sg[(long)n * C + c];
-    sw += sx[(long)n * C + c] * g;
-    sb += g;
+  if (c < C) {
+#pragma unroll 4
+    for (int n = slice; n < N; n += 4) {
+      const float g = sg[(long)n * C + c];
+      sw += sx[(long)n * C + c] * g;
+      sb += g;
+    }
   }
-  w_curv[c] = alpha * sw;
-  if (b_curv) b_curv[c] = alpha * sb;
+  rw[slice][lane] = sw;
+  rb[slice][lane] = sb;
+  __syncthreads();
+  if (slice == 0 && c < C) {
+    w_curv[c] = alpha * (((rw[0][lane] + rw[1][lane]) + rw[2][lane]) + rw[3][lane]);
+    if (b_curv) b_curv[c] = alpha * (((rb[0][lane] + rb[1][lane]) + rb[2][lane]) + rb[3][lane]);
+  }
 }
 
 }  // namespace kfac
@@ -397,7 +409,7 @@ int kfac_scale_rows(const float* x, const float* w, int64_t rows, int64_t len, i
 int kfac_bn_diag_combine(const float* sx, const float* sg, int n, int channels, float alpha,
                          float* w_curv, float* b_curv, void* stream) {
   if (!sx || !sg || !w_curv || n <= 0 || channels <= 0) return KFAC_ERR_ARG;
-  hipLaunchKernelGGL(bn_combine_kernel, dim3(cdiv(channels, 128)), dim3(128), 0,
+  hipLaunchKernelGGL(bn_combine_kernel, dim3(cdiv(channels, 64)), dim3(256), 0,
                      (hipStream_t)stream, sx, sg, n, channels, alpha, w_curv, b_curv);
   return launch_status();
 }

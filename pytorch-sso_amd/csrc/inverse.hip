@@ -83,13 +83,23 @@ __global__ __launch_bounds__(256) void inv_copy_damp_kernel(const MatDesc* table
   upper_tile(blockIdx.x, m.T, bi, bj);
   const float damp = effective_damp(table, m);
   const int n = m.n;
-  for (int e = threadIdx.x; e < BM * BN; e += 256) {
-    const int row = bi * BM + (e >> 7);
-    const int col = bj * BN + (e & 127);
-    if (row < n && col < n) {
-      float v = m.src[(size_t)row * n + col];
-      if (row == col) v += damp;
-      m.U[(size_t)row * n + col] = v;
+  // 8 loads in flight per thread, then 8 stores
+  for (int e0 = threadIdx.x; e0 < BM * BN; e0 += 256 * 8) {
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int e = e0 + 256 * k;
+      const int row = bi * BM + (e >> 7);
+      const int col = bj * BN + (e & 127);
+      v[k] = (row < n && col < n) ? m.src[(size_t)row * n + col] : 0.f;
+      if (row == col) v[k] += damp;
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int e = e0 + 256 * k;
+      const int row = bi * BM + (e >> 7);
+      const int col = bj * BN + (e & 127);
+      if (row < n && col < n) m.U[(size_t)row * n + col] = v[k];
     }
   }
 }
