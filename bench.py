@@ -220,16 +220,16 @@ class LayerSet(object):
 
     def timed_phases(self, iters):
         """Average ms of: Kronecker factor build (the syrk kernels only) / BatchNorm
-        diagonal curvature / EMA / inversion / precondition+update, bracketed by HIP
+        diagonal curvature / EMA / inversion / preconditioning / parameter update, bracketed by HIP
         events on the stream the kernels are launched on (torch's current stream)."""
         torch = self.torch
         from torchsso.curv import curvature as _curv
         ev = lambda: torch.cuda.Event(enable_timing=True)
-        acc = [0.] * 5
+        acc = [0.] * 6
         groups = self.opt.param_groups
         for _ in range(iters):
             self.restore_grads()
-            e = [ev() for _ in range(6)]
+            e = [ev() for _ in range(7)]
             e[0].record()
             self.build_factors(('conv', 'linear'))
             e[1].record()
@@ -240,10 +240,11 @@ class LayerSet(object):
             _curv.update_inv_all(self.curvs)
             e[4].record()
             _curv.precondition_all([(g['curv'], g['params']) for g in groups])
-            self.opt._fused_update(groups, 'params')
             e[5].record()
+            self.opt._fused_update(groups, 'params')
+            e[6].record()
             torch.cuda.synchronize()
-            for i in range(5):
+            for i in range(6):
                 acc[i] += e[i].elapsed_time(e[i + 1])
         return [a / iters for a in acc]
 
@@ -390,7 +391,7 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    f_ms, bn_ms, ema_ms, inv_ms, pre_ms = phases
+    f_ms, bn_ms, ema_ms, inv_ms, pre_ms, upd_ms = phases
     total_flops = work['factor'] + work['inverse'] + work['precondition']
 
     out = {
@@ -407,7 +408,8 @@ def main():
         'algorithmic_gflop': {k: round(v / 1e9, 1) for k, v in work.items() if not k.endswith('bytes')},
         'phases_ms': {'factor': round(f_ms, 4), 'batchnorm_diag': round(bn_ms, 4),
                       'ema': round(ema_ms, 4),
-                      'invert': round(inv_ms, 4), 'precondition_update': round(pre_ms, 4)},
+                      'invert': round(inv_ms, 4), 'precondition': round(pre_ms, 4),
+                      'update': round(upd_ms, 4)},
         'phases_tflops': {'factor': round(work['factor'] / f_ms / 1e9, 2),
                           'invert': round(work['inverse'] / inv_ms / 1e9, 2),
                           'precondition': round(work['precondition'] / pre_ms / 1e9, 2)},
