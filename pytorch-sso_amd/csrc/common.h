@@ -10,8 +10,8 @@ namespace kfac {
 
 inline int cdiv(int a, int b) { return (a + b - 1) / b; }
 
-// Kernels built on the 2x2 tile engine stage 72 KiB in LDS, above the 64 KiB
-// that a kernel may use without opting in; the opt-in is done once per kernel.
+// Dynamic LDS sizes are registered once per kernel (required above 64 KiB, as
+// for the 148 KiB of the diagonal-block kernel; harmless below).
 bool enable_large_lds(const void* kernel, int bytes);
 
 #define KFAC_LAUNCH_TILE2(kernel, grid, stream, ...)                                         \

@@ -63,7 +63,7 @@ struct JobDesc {
   short splits, pad;       // k-splits
   int K;                   // n * hh * ww
   int cps;                 // chunks per split
-  int tiles0;              // (unused by the kernels) first work item, kept for the host
+  int pad2;
   int part0;               // index (in C*C units) of its first partial in the workspace
 };
 
@@ -295,7 +295,7 @@ static TapPlanHost plan_taps(int n, int c, int H, int Wd, int kh, int kw, int ph
     splits = (nchunks + cps - 1) / cps;
     jd.splits = (short)splits;
     jd.cps = (int)cps;
-    jd.tiles0 = item;
+    jd.pad2 = 0;
     pd.item0[j] = item;
     jd.part0 = part;
     item += (int)splits * ntiles;

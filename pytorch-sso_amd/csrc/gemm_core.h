@@ -10,11 +10,12 @@
 //   * the two chained preconditioning GEMMs,
 // without ever materialising a transposed, concatenated or unfolded copy.
 //
-// Operand functor contract (see operands.h):
+// Operand functor contract (details in operands.h):
 //   static constexpr int layout;      KM: consecutive m are contiguous in memory
 //                                     MK: consecutive k are contiguous in memory
-//   MS mstate(int m) / KS kstate(int k): per-index precomputation
-//   float load(MS, KS): the element, 0 outside the operand's own bounds
+//   MS mstate(int m) / KS kstate(int k, bool valid): per-index precomputation
+//   unsigned off(MS, KS): byte offset for a raw buffer load; an element outside
+//                         the operand gets an offset beyond the buffer and reads 0
 // The layout only chooses how the 256 threads sweep the 16x128 chunk so that
 // global loads coalesce, and how the chunk sits in LDS:
 //   KM chunk -> lds[k][m]   (row length = tile width), MFMA lanes read ds_read_b32
@@ -37,9 +38,9 @@ constexpr int NTHREADS = 256;    // threads of the default configuration
 //   tile = (64*WM) x (64*WN), threads = 64*WM*WN.
 // 2x2 is the default; 1x1 (one wave, 64x64) serves small factors, where a
 // 128-wide tile would be mostly padding.
-// KC is the reduction depth per LDS stage: 32 for the 2x2 configuration (the
-// 64 MFMAs per wave and stage then cover the latency of the next stage's
-// global loads), 16 for 1x1 (one wave stages the whole chunk by itself).
+// KC = 16 is the reduction depth per LDS stage (32 MFMAs per wave and stage);
+// two stages of the 2x2 configuration take 40 KiB, so that three workgroups
+// fit the 160 KiB of a CU.
 template <int WM, int WN>
 struct Cfg {
   static constexpr int TM = 64 * WM;
@@ -51,7 +52,7 @@ struct Cfg {
   static constexpr int Q_FLOATS = LDS_MK * TN;
   static constexpr int SMEM_FLOATS = 2 * (P_FLOATS + Q_FLOATS);
 };
-constexpr int SMEM_FLOATS = Cfg<2, 2>::SMEM_FLOATS;   // 72 KiB
+constexpr int SMEM_FLOATS = Cfg<2, 2>::SMEM_FLOATS;   // 40 KiB
 
 enum { KM = 0, MK = 1 };
 

@@ -5,11 +5,6 @@
 namespace kfac {
 
 // ---------------------------------------------------------------------------
-// Dense row-major matrix read as P(k, m) = p[k*ld + m]  (m contiguous).
-// Optional last column (index M-1) that is not in memory:
-//   extra == 1 : the constant 1 (bias augmentation of a Linear input)
-//   extra == 2 : taken from vec[k] (bias gradient appended to a weight gradient)
-// ---------------------------------------------------------------------------
 // Operand functor contract used by the staging code of the tile engine.
 // Elements are read with raw buffer loads (buffer_load_dword ... offen): the
 // functor supplies a buffer resource over its tensor and a 32-bit BYTE offset
@@ -24,6 +19,8 @@ namespace kfac {
 // Offsets of valid elements are below 2^30 (tensors are limited to 1 GiB per
 // call; the entry points split larger ones); an invalid row adds 2^31 and an
 // invalid k adds 2^30, so every sum with an invalid part lands in [2^30, 2^32).
+// ---------------------------------------------------------------------------
+
 // Dense row-major matrix read as P(k, m) = p[k*ld + m]  (m contiguous), K rows.
 // Optional last column (index M-1) that is not in memory:
 //   extra == 1 : the constant 1 (bias augmentation of a Linear input)
