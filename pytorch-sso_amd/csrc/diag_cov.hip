@@ -67,9 +67,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void diag_conv_kernel(
   EpiSquares epi;
 #pragma unroll
   for (int i = 0; i < 64; ++i) epi.sq[i] = 0.f;
+  const ConvA Q0{x, c, H, Wd, kh, kw, sh, sw, ph, pw, dh, dw, OH, OW, ckk, 0};
   for (int b = b0; b < b1; ++b) {
     DenseMK P{g + (size_t)b * cout * L, L, cout};
-    ConvA Q{x + (size_t)b * c * H * Wd, c, H, Wd, kh, kw, sh, sw, ph, pw, dh, dw, OH, OW, ckk, 0};
+    const ConvA Q(Q0, x + (size_t)b * c * H * Wd);
     gemm_tile(P, Q, m0, n0, 0, L, false, epi, smem);
   }
   float* dst = splits == 1 ? out : ws + (size_t)split * cout * ckk;

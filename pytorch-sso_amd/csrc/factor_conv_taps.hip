@@ -39,6 +39,7 @@ struct ShiftX {
   static constexpr bool has_second = false;
   const float* p;
   int C, H, W, u0, v0, hh, ww;     // u0, v0 already include the displacement
+  FastDiv by_area, by_ww;
   struct MS { unsigned off; };
   struct KS { unsigned off; };
   __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc() const { return make_rsrc(p); }
@@ -46,10 +47,9 @@ struct ShiftX {
     return MS{m < C ? (unsigned)(m * H * W) * 4u : INV_M};
   }
   __device__ __forceinline__ KS kstate(int k, bool valid) const {
-    const int area = hh * ww;
-    const int n = k / area;
-    const int rem = k - n * area;
-    const int ry = rem / ww;
+    const int n = by_area.div(k);
+    const int rem = k - n * hh * ww;
+    const int ry = by_ww.div(rem);
     const int rx = rem - ry * ww;
     return KS{valid ? (unsigned)(n * C * H * W + (u0 + ry) * W + v0 + rx) * 4u : INV_K};
   }
@@ -58,12 +58,12 @@ struct ShiftX {
 };
 
 struct JobDesc {
-  short u0, v0, hh, ww;    // rectangle of the first factor
+  short u0, v0, hh, ww;    // rectangle of the first factor; the reduction runs over n * hh * ww
   short dy, dx;            // displacement of the second factor
-  short splits, pad;       // k-splits
-  int K;                   // n * hh * ww
+  short splits;            // k-splits
+  unsigned char sh_area, sh_ww;   // shifts of the two FastDiv (by hh * ww and by ww)
+  unsigned m_area, m_ww;          // their multipliers
   int cps;                 // chunks per split
-  int pad2;
   int part0;               // index (in C*C units) of its first partial in the workspace
 };
 
@@ -87,7 +87,8 @@ struct TapPlanDev {
 static_assert(sizeof(TapPlanDev) <= 3800, "plan must fit the kernel argument buffer");
 template <int W>
 __global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void corr_kernel(
-    const float* x, int C, int H, int Wd, const TapPlanDev plan, int tiles_side, float* ws) {
+    const float* x, int nimg, int C, int H, int Wd, const TapPlanDev plan, int tiles_side,
+    float* ws) {
   constexpr int TS = 64 * W;
   constexpr int KC = Cfg<W, W>::KC;
   extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -102,11 +103,17 @@ __global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void corr_kernel(
   const int split = local / ntiles;
   const int tile = local - split * ntiles;
   const int bi = tile / tiles_side, bj = tile - bi * tiles_side;
+  const int K = nimg * jd.hh * jd.ww;
   const int kbeg = split * jd.cps * KC;
   int kend = kbeg + jd.cps * KC;
-  if (kend > jd.K) kend = jd.K;
-  ShiftX P{x, C, H, Wd, jd.u0, jd.v0, jd.hh, jd.ww};
-  ShiftX Q{x, C, H, Wd, jd.u0 + jd.dy, jd.v0 + jd.dx, jd.hh, jd.ww};
+  if (kend > K) kend = K;
+  FastDiv by_area, by_ww;
+  by_area.m = jd.m_area;
+  by_area.sh = jd.sh_area;
+  by_ww.m = jd.m_ww;
+  by_ww.sh = jd.sh_ww;
+  ShiftX P{x, C, H, Wd, jd.u0, jd.v0, jd.hh, jd.ww, by_area, by_ww};
+  ShiftX Q{x, C, H, Wd, jd.u0 + jd.dy, jd.v0 + jd.dx, jd.hh, jd.ww, by_area, by_ww};
   EpiStore epi{ws + (size_t)(jd.part0 + split) * C * C, C, C, C, 1.f, 0.f, false};
   gemm_tile_cfg<W, W>(P, Q, bi * TS, bj * TS, kbeg, kend, false, epi, smem);
 }
@@ -267,7 +274,11 @@ static TapPlanHost plan_taps(int n, int c, int H, int Wd, int kh, int kw, int ph
             jd.v0 = (short)ax.pieces[px].lo;
             jd.ww = (short)(ax.pieces[px].hi - ax.pieces[px].lo);
             jd.dx = (short)ax.pieces[px].delta;
-            jd.K = n * (int)jd.hh * (int)jd.ww;
+            const FastDiv fa((unsigned)(jd.hh * jd.ww)), fw((unsigned)jd.ww);
+            jd.m_area = fa.m;
+            jd.sh_area = (unsigned char)fa.sh;
+            jd.m_ww = fw.m;
+            jd.sh_ww = (unsigned char)fw.sh;
           }
           if (npj >= MAX_PAIR_JOBS) return hp;
           pd.pair_jobs[npj++] = (short)j;
@@ -282,20 +293,20 @@ static TapPlanHost plan_taps(int n, int c, int H, int Wd, int kh, int kw, int ph
   const int ntiles = hp.tiles_side * hp.tiles_side;
   const int kc = hp.w == 1 ? Cfg<1, 1>::KC : Cfg<2, 2>::KC;
   double total = 0;
-  for (int j = 0; j < pd.njobs; ++j) total += (double)pd.jobs[j].K;
+  auto job_k = [&](const JobDesc& jd) { return (long)n * jd.hh * jd.ww; };
+  for (int j = 0; j < pd.njobs; ++j) total += (double)job_k(pd.jobs[j]);
   const double target_items = hp.w == 1 ? 3072.0 : 1024.0;
   int item = 0, part = 0;
   for (int j = 0; j < pd.njobs; ++j) {
     JobDesc& jd = pd.jobs[j];
-    const long nchunks = ((long)jd.K + kc - 1) / kc;
-    long splits = (long)(target_items * ((double)jd.K / total) / ntiles + 0.5);
+    const long nchunks = (job_k(jd) + kc - 1) / kc;
+    long splits = (long)(target_items * ((double)job_k(jd) / total) / ntiles + 0.5);
     const long max_splits = std::max<long>(1, nchunks / (128 / kc));
     splits = std::max<long>(1, std::min(std::min(splits, max_splits), 4096L));
     long cps = (nchunks + splits - 1) / splits;
     splits = (nchunks + cps - 1) / cps;
     jd.splits = (short)splits;
     jd.cps = (int)cps;
-    jd.pad2 = 0;
     pd.item0[j] = item;
     jd.part0 = part;
     item += (int)splits * ntiles;
@@ -334,13 +345,13 @@ int conv_a_taps(const float* x, int n, int c, int H, int W, int kh, int kw, int 
   if (hp.w == 1) {
     constexpr int lds = Cfg<1, 1>::SMEM_FLOATS * (int)sizeof(float);
     if (!enable_large_lds((const void*)corr_kernel<1>, lds)) return KFAC_ERR_LAUNCH;
-    hipLaunchKernelGGL(corr_kernel<1>, dim3(hp.items), dim3(64), lds, stream, x, c, H, W, hp.dev,
-                       hp.tiles_side, ws);
+    hipLaunchKernelGGL(corr_kernel<1>, dim3(hp.items), dim3(64), lds, stream, x, n, c, H, W,
+                       hp.dev, hp.tiles_side, ws);
   } else {
     constexpr int lds = Cfg<2, 2>::SMEM_FLOATS * (int)sizeof(float);
     if (!enable_large_lds((const void*)corr_kernel<2>, lds)) return KFAC_ERR_LAUNCH;
-    hipLaunchKernelGGL(corr_kernel<2>, dim3(hp.items), dim3(256), lds, stream, x, c, H, W, hp.dev,
-                       hp.tiles_side, ws);
+    hipLaunchKernelGGL(corr_kernel<2>, dim3(hp.items), dim3(256), lds, stream, x, n, c, H, W,
+                       hp.dev, hp.tiles_side, ws);
   }
   hipLaunchKernelGGL(block_sum_kernel, dim3(cdiv(c * c / 4, 256), hp.dev.npairs), dim3(256), 0,
                      stream, hp.dev, ws, c * c, B);

@@ -68,6 +68,25 @@ typedef __attribute__((address_space(3))) float lds_f;
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4f lds_f4;
 
+// Division of an index below 2^31 by a divisor fixed per launch, as a multiply
+// and a shift: with l = ceil(log2 d) and m = ceil(2^(31+l) / d) (which fits 32
+// bits), floor(n / d) == (n * m) >> (31 + l) for every n < 2^31.  The operand
+// functors turn a reduction index into (image, row, column) once per thread and
+// chunk; a hardware-less integer division there costs about 40 instructions.
+struct FastDiv {
+  unsigned m, sh;
+  FastDiv() = default;
+  __host__ __device__ explicit FastDiv(unsigned d) {
+    unsigned l = 0;
+    while ((1ull << l) < d) ++l;
+    sh = 31 + l;
+    m = (unsigned)(((1ull << sh) + d - 1) / d);
+  }
+  __host__ __device__ __forceinline__ int div(int n) const {
+    return (int)(((unsigned long long)(unsigned)n * m) >> sh);
+  }
+};
+
 // ---- raw buffer addressing (see the operand contract in operands.h) ----------
 constexpr unsigned INV_M = 0x80000000u;
 constexpr unsigned INV_K = 0x40000000u;

@@ -87,6 +87,10 @@ struct ConvG {
   static constexpr bool has_second = false;
   const float* p;
   int C, HW;
+  FastDiv by_hw;
+  ConvG() = default;
+  __host__ __device__ ConvG(const float* p_, int C_, int HW_)
+      : p(p_), C(C_), HW(HW_), by_hw((unsigned)HW_) {}
   struct MS { unsigned off; };
   struct KS { unsigned off; };
   __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc() const {
@@ -96,7 +100,7 @@ struct ConvG {
     return MS{m < C ? (unsigned)(m * HW) * 4u : INV_M};
   }
   __device__ __forceinline__ KS kstate(int k, bool valid) const {
-    const int n = k / HW;
+    const int n = by_hw.div(k);
     return KS{valid ? (unsigned)(n * C * HW + (k - n * HW)) * 4u : INV_K};
   }
   __device__ __forceinline__ unsigned off(const MS& m, const KS& k) const { return m.off + k.off; }
@@ -111,6 +115,15 @@ struct ConvA {
   static constexpr bool has_second = false;
   const float* p;
   int C, H, W, KH, KW, SH, SW, PH, PW, DH, DW, OH, OW, M, ones;
+  FastDiv by_l, by_ow;        // divisions by OH*OW and by OW
+  ConvA() = default;
+  __host__ __device__ ConvA(const float* p_, int C_, int H_, int W_, int KH_, int KW_, int SH_,
+                            int SW_, int PH_, int PW_, int DH_, int DW_, int OH_, int OW_, int M_,
+                            int ones_)
+      : p(p_), C(C_), H(H_), W(W_), KH(KH_), KW(KW_), SH(SH_), SW(SW_), PH(PH_), PW(PW_), DH(DH_),
+        DW(DW_), OH(OH_), OW(OW_), M(M_), ones(ones_), by_l((unsigned)(OH_ * OW_)),
+        by_ow((unsigned)OW_) {}
+  __host__ __device__ ConvA(const ConvA& o, const float* p_) : ConvA(o) { p = p_; }
   // Per row m: the byte offset of (c, kh, kw) and the two patch displacements
   // packed as (dy << 16) | (dx & 0xffff), so that the 8 row states of a thread
   // take 16 registers.  dy = -32768 marks a row outside the operand (every bounds
@@ -136,9 +149,9 @@ struct ConvA {
     return s;
   }
   __device__ __forceinline__ KS kstate(int k, bool valid) const {
-    const int n = k / (OH * OW);
+    const int n = by_l.div(k);
     const int rem = k - n * OH * OW;
-    const int oh = rem / OW;
+    const int oh = by_ow.div(rem);
     const int ow = rem - oh * OW;
     KS s;
     s.y0 = valid ? oh * SH - PH : -(1 << 20);
