@@ -112,25 +112,35 @@ constexpr int DLD = DB + 1;      // LDS leading dimension
 constexpr int WLD = 65;
 constexpr int DIAG_SMEM_BYTES = (2 * DB * DLD + 64 * WLD) * (int)sizeof(float);
 
-// One wave factors the 32x32 block at (c0, c0) of S (lane j holds column j in
-// registers), inverts the factor, and writes U_qq to S and Y_qq to Yb.
-// Each step needs one row of the block in every lane: the lanes write their
-// element of the row to a 32-float LDS buffer and read the whole row back with
-// broadcast ds_read_b128 (no cross-lane register traffic).  `scr` is 16-byte
-// aligned scratch of at least 64 + 32*32 floats.
-__device__ __forceinline__ void chol_inv_32(lds_f* S, lds_f* Yb, lds_f* scr, int c0, int row_base,
-                                            int* info) {
+// One wave runs the 32 elimination steps of the 32-row strip at row c0 of S on two
+// column blocks at once: lanes 0-31 hold the columns of the diagonal leaf
+// (c0 .. c0+31), lanes 32-63 the columns pcol .. pcol+31 of the same rows (a
+// block of the row panel to the right; pcol < 0: none, the lanes shadow the leaf).
+// Lane j keeps its column in registers.  Each step needs row c of the leaf in every
+// lane: the leaf lanes write their element to a 64-float LDS buffer private to
+// the wave and all lanes read the row back with broadcast ds_read_b128 (no
+// cross-lane register traffic).  The panel columns see the same eliminations as
+// the leaf columns, so the strip ends up holding U[q][*] without a triangular
+// solve.  Several waves may run this on the same leaf with different panel
+// blocks (the leaf is then factored redundantly; only `owner` writes it out, as
+// a dense 32x32 copy `ubuf`, which the caller copies over the leaf in S once all
+// waves are past reading it, and which feeds the back substitution).
+__device__ __forceinline__ void chol_strip_32(lds_f* S, lds_f* rowbuf, lds_f* ubuf, int c0,
+                                              int pcol, bool owner, int row_base, int* info) {
   const int lane = threadIdx.x & 63;
   const int j = lane & 31;
-  lds_f* rowbuf = scr;           // 32 floats
-  lds_f* ubuf = scr + 64;        // 32 x 32, row-major, rows 16-byte aligned
+  const bool leaf = lane < 32;
+  const int col = (leaf || pcol < 0) ? c0 + j : pcol + j;
   float a[32];
 #pragma unroll
-  for (int i = 0; i < 32; ++i) a[i] = S[(c0 + i) * DLD + c0 + j];
+  for (int i = 0; i < 32; ++i) a[i] = S[(c0 + i) * DLD + col];
   int bad = 0;
 #pragma unroll
   for (int c = 0; c < 32; ++c) {
-    rowbuf[j] = a[c];            // A[c][j] after the updates of the earlier steps
+    // A[c][c0 + j] after the updates of the earlier steps; the panel lanes write
+    // into the unused second half of the buffer, so that the store is unconditional
+    rowbuf[lane] = a[c];
+    __builtin_amdgcn_wave_barrier();
     float row[32];
 #pragma unroll
     for (int g = c / 4; g < 8; ++g) {
@@ -147,15 +157,29 @@ __device__ __forceinline__ void chol_inv_32(lds_f* S, lds_f* Yb, lds_f* scr, int
     const float d = piv * rd;
     const float f = a[c] * (rd * rd);
 #pragma unroll
-    for (int i = c + 1; i < 32; ++i) a[i] = fmaf(-row[i], f, a[i]);   // A[i][j] -= U[c][i] U[c][j]
-    a[c] = (j > c) ? a[c] * rd : (j == c ? d : 0.f);
+    for (int i = c + 1; i < 32; ++i) a[i] = fmaf(-row[i], f, a[i]);   // A[i][col] -= U[c][i] U[c][col]
+    const float u = a[c] * rd;
+    a[c] = leaf ? (j > c ? u : (j == c ? d : 0.f)) : u;
   }
-  if (bad != 0 && lane == 0) {
+  if (owner && bad != 0 && lane == 0) {
     if (*info == 0) *info = bad;
   }
+  if (leaf) {
+    if (owner) {
 #pragma unroll
-  for (int i = 0; i < 32; ++i) ubuf[i * 32 + j] = (i <= j) ? a[i] : 0.f;
-  // Y = U^-1 by back substitution: column j of Y in lane j, row i of U broadcast
+      for (int i = 0; i < 32; ++i) ubuf[i * 32 + j] = (i <= j) ? a[i] : 0.f;
+    }
+  } else if (pcol >= 0) {
+#pragma unroll
+    for (int i = 0; i < 32; ++i) S[(c0 + i) * DLD + pcol + j] = a[i];
+  }
+}
+
+// One wave: Y = U^-1 of the 32x32 upper-triangular leaf in ubuf (dense, row-major),
+// written to Yb at (c0, c0).  Column j of Y in lane j, row i of U broadcast.
+__device__ __forceinline__ void backsub_32(const lds_f* ubuf, lds_f* Yb, int c0) {
+  const int lane = threadIdx.x & 63;
+  const int j = lane & 31;
   float y[32];
 #pragma unroll
   for (int i = 31; i >= 0; --i) {
@@ -182,10 +206,7 @@ __device__ __forceinline__ void chol_inv_32(lds_f* S, lds_f* Yb, lds_f* scr, int
   }
   if (lane < 32) {
 #pragma unroll
-    for (int i = 0; i < 32; ++i) {
-      S[(c0 + i) * DLD + c0 + j] = (i <= j) ? a[i] : 0.f;
-      Yb[(c0 + i) * DLD + c0 + j] = (i <= j) ? y[i] : 0.f;
-    }
+    for (int i = 0; i < 32; ++i) Yb[(c0 + i) * DLD + c0 + j] = (i <= j) ? y[i] : 0.f;
   }
 }
 
@@ -284,20 +305,31 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
   }
   __syncthreads();
 
+  // Scratch (in Wt, free until the doubling below): a 64-float row buffer per
+  // wave and two dense leaf copies, used alternately.
+  lds_f* const rowbuf = Wt + 64 * wave;
+  lds_f* const ubuf0 = Wt + 256;
   const int nq = (nb + 31) / 32;
   for (int q = 0; q < nq; ++q) {
     const int c0 = 32 * q;
-    if (t < 64) chol_inv_32(S, Yb, Wt, c0, r0, info + m.out);
-    __syncthreads();
     const int rest = nq - q - 1;     // 32-blocks to the right
+    if (wave < 3) {
+      // waves 0..2: the strip of leaf q, each with one block of the row panel
+      if (wave == 0 || wave < rest)
+        chol_strip_32(S, rowbuf, ubuf0 + 1024 * (q & 1), c0, wave < rest ? c0 + 32 * (wave + 1) : -1,
+                      wave == 0, r0, info + m.out);
+    } else if (q > 0) {
+      // wave 3, meanwhile: inverse of the previous leaf (off the critical path)
+      backsub_32(ubuf0 + 1024 * ((q - 1) & 1), Yb, c0 - 32);
+    }
+    __syncthreads();
+    if (wave == 0 && (t & 32) == 0) {
+      // the factored leaf replaces A[q][q] now that no wave reads the original any more
+      const lds_f* ub = ubuf0 + 1024 * (q & 1);
+#pragma unroll
+      for (int i = 0; i < 32; ++i) S[(c0 + i) * DLD + c0 + t] = ub[i * 32 + t];
+    }
     if (rest > 0) {
-      // row panel: U[q][j] = Yqq^T A[q][j], one 32x32 block per wave, in place
-      if (wave < rest) {
-        const int cj = c0 + 32 * (wave + 1);
-        const v16f acc = lds_mma32(Yb + c0 * DLD + c0, DLD, 1, S + c0 * DLD + cj, DLD, 1, 32);
-        lds_put32(S + c0 * DLD + cj, DLD, acc, 1.f);
-      }
-      __syncthreads();
       // trailing update: A[i][j] -= U[q][i]^T U[q][j], q < i <= j
       const int nblk = rest * (rest + 1) / 2;
       for (int blk = wave; blk < nblk; blk += 4) {
@@ -310,6 +342,8 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
       __syncthreads();
     }
   }
+  if (wave == 3) backsub_32(ubuf0 + 1024 * ((nq - 1) & 1), Yb, 32 * (nq - 1));
+  __syncthreads();
 
   // inverse of the whole block by doubling: 32 -> 64 -> 128
   if (nq > 1) {
