@@ -48,6 +48,29 @@ __global__ void inv_setup_kernel(DescChunk chunk, MatDesc* table, int offset, in
   if (i < count) table[offset + i] = chunk.d[i];
 }
 
+// Launches cover the matrices that still have work with a 1-D grid of exactly the
+// workgroups needed: cum[i] is the first work item of the i-th listed matrix
+// (table index first + i), cum[n] the grid size.  (A rectangular grid
+// "largest tile count x matrices" would start tens of thousands of workgroups
+// that only find out that their matrix is too small.)
+constexpr int WL_MAX = 128;
+struct WorkList {
+  int n, first;
+  int cum[WL_MAX + 1];
+};
+
+// matrix (table index) and local work item of the calling workgroup
+__device__ __forceinline__ void work_find(const WorkList& wl, int& mat, int& local) {
+  const int item = blockIdx.x;
+  int lo = 0, hi = wl.n;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (wl.cum[mid] <= item) lo = mid; else hi = mid;
+  }
+  mat = wl.first + lo;
+  local = item - wl.cum[lo];
+}
+
 // trace of src (one workgroup per matrix)
 __global__ __launch_bounds__(256) void inv_trace_kernel(MatDesc* table) {
   __shared__ float red[256];
@@ -74,13 +97,14 @@ __device__ __forceinline__ float effective_damp(const MatDesc* table, const MatD
 }
 
 // U = upper tiles of (src + damp I); also clears info
-__global__ __launch_bounds__(256) void inv_copy_damp_kernel(const MatDesc* table, int* info) {
-  const MatDesc m = table[blockIdx.y];
-  const int ntiles = m.T * (m.T + 1) / 2;
-  if ((int)blockIdx.x >= ntiles) return;
-  if (blockIdx.x == 0 && threadIdx.x == 0) info[m.out] = 0;
+__global__ __launch_bounds__(256) void inv_copy_damp_kernel(const MatDesc* table, int* info,
+                                                            const WorkList wl) {
+  int mat, local;
+  work_find(wl, mat, local);
+  const MatDesc m = table[mat];
+  if (local == 0 && threadIdx.x == 0) info[m.out] = 0;
   int bi, bj;
-  upper_tile(blockIdx.x, m.T, bi, bj);
+  upper_tile(local, m.T, bi, bj);
   const float damp = effective_damp(table, m);
   const int n = m.n;
   // 8 loads in flight per thread, then 8 stores
@@ -381,10 +405,13 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
 }
 
 // row panel of the blocked Cholesky: U[p, j] = Ypp^T * A[p, j], j > p
-__global__ __launch_bounds__(NTHREADS) void potrf_panel_kernel(const MatDesc* table, int p) {
+__global__ __launch_bounds__(NTHREADS) void potrf_panel_kernel(const MatDesc* table, int p,
+                                                               const WorkList wl) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  const MatDesc m = table[blockIdx.y];
-  const int bj = p + 1 + blockIdx.x;
+  int mat, local;
+  work_find(wl, mat, local);
+  const MatDesc m = table[mat];
+  const int bj = p + 1 + local;
   if (bj >= m.T) return;
   const int n = m.n;
   const int r0 = p * DB;
@@ -403,9 +430,12 @@ __global__ __launch_bounds__(NTHREADS) void potrf_panel_kernel(const MatDesc* ta
 constexpr int OUTER_BLOCKS = 4;
 
 __global__ __launch_bounds__(NTHREADS, 3) void potrf_trail_kernel(const MatDesc* table, int kb0,
-                                                               int nk, int row_lo, int row_hi) {
+                                                               int nk, int row_lo, int row_hi,
+                                                               const WorkList wl) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  const MatDesc m = table[blockIdx.y];
+  int mat, local;
+  work_find(wl, mat, local);
+  const MatDesc m = table[mat];
   const int T = m.T;
   const int hi = min(row_hi, T);
   if (row_lo >= hi) return;
@@ -413,16 +443,16 @@ __global__ __launch_bounds__(NTHREADS, 3) void potrf_trail_kernel(const MatDesc*
   if (row_hi >= T) {
     // all remaining rows: walk the upper triangle of the (T - row_lo)^2 block grid
     const int Tr = T - row_lo;
-    if ((int)blockIdx.x >= Tr * (Tr + 1) / 2) return;
-    upper_tile(xcd_remap(blockIdx.x, Tr * (Tr + 1) / 2), Tr, bi, bj);
+    if (local >= Tr * (Tr + 1) / 2) return;
+    upper_tile(xcd_remap(local, Tr * (Tr + 1) / 2), Tr, bi, bj);
     bi += row_lo;
     bj += row_lo;
   } else {
     // a few rows: rectangular walk, tiles left of the diagonal exit
     const int width = T - row_lo;
-    const int rr = blockIdx.x / width;
+    const int rr = local / width;
     bi = row_lo + rr;
-    bj = row_lo + (blockIdx.x - rr * width);
+    bj = row_lo + (local - rr * width);
     if (bi >= hi || bj < bi) return;
   }
   const int n = m.n;
@@ -447,13 +477,13 @@ __device__ __forceinline__ int seg_of(int b, int depth, int T) {
   return (int)((((long)(b + 1) << depth) - 1) / T);
 }
 
-__device__ __forceinline__ MergeTile merge_tile(const MatDesc& m, int depth) {
+__device__ __forceinline__ MergeTile merge_tile(const MatDesc& m, int depth, int local) {
   MergeTile t;
   t.valid = false;
   const int T = m.T;
-  if (T < 2 || (int)blockIdx.x >= (T - 1) * T / 2) return t;
+  if (T < 2 || local >= (T - 1) * T / 2) return t;
   int bi, bj;
-  upper_tile(xcd_remap(blockIdx.x, (T - 1) * T / 2), T - 1, bi, bj);
+  upper_tile(xcd_remap(local, (T - 1) * T / 2), T - 1, bi, bj);
   bj += 1;
   const int P = seg_of(bi, depth, T);
   if (seg_of(bj, depth, T) != P) return t;
@@ -473,10 +503,13 @@ __device__ __forceinline__ MergeTile merge_tile(const MatDesc& m, int depth) {
 
 // first product:  W^T[j][i] = sum_{k <= j} Y22[k][j] * U12[i][k], stored at
 // Y[X2 rows][X1 cols] (the unused lower triangle of Y)
-__global__ __launch_bounds__(NTHREADS) void trtri_w_kernel(const MatDesc* table, int depth) {
+__global__ __launch_bounds__(NTHREADS) void trtri_w_kernel(const MatDesc* table, int depth,
+                                                           const WorkList wl) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  const MatDesc m = table[blockIdx.y];
-  const MergeTile t = merge_tile(m, depth);
+  int mat, local;
+  work_find(wl, mat, local);
+  const MatDesc m = table[mat];
+  const MergeTile t = merge_tile(m, depth, local);
   if (!t.valid) return;
   const int n = m.n;
   DenseKM P{m.Y + (size_t)t.X2 * n + t.X2, nullptr, n, t.b2, 0};
@@ -486,10 +519,13 @@ __global__ __launch_bounds__(NTHREADS) void trtri_w_kernel(const MatDesc* table,
 }
 
 // second product:  Y12[i][j] = - sum_{k >= i} Y11[i][k] * W^T[j][k]
-__global__ __launch_bounds__(NTHREADS) void trtri_y_kernel(const MatDesc* table, int depth) {
+__global__ __launch_bounds__(NTHREADS) void trtri_y_kernel(const MatDesc* table, int depth,
+                                                           const WorkList wl) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  const MatDesc m = table[blockIdx.y];
-  const MergeTile t = merge_tile(m, depth);
+  int mat, local;
+  work_find(wl, mat, local);
+  const MatDesc m = table[mat];
+  const MergeTile t = merge_tile(m, depth, local);
   if (!t.valid) return;
   const int n = m.n;
   DenseMK P{m.Y + (size_t)t.X1 * n + t.X1, n, t.b1};
@@ -499,13 +535,14 @@ __global__ __launch_bounds__(NTHREADS) void trtri_y_kernel(const MatDesc* table,
 }
 
 // dst = Y Y^T over the upper tiles (k >= the later block), mirrored
-__global__ __launch_bounds__(NTHREADS) void lauum_kernel(const MatDesc* table) {
+__global__ __launch_bounds__(NTHREADS) void lauum_kernel(const MatDesc* table, const WorkList wl) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  const MatDesc m = table[blockIdx.y];
+  int mat, local;
+  work_find(wl, mat, local);
+  const MatDesc m = table[mat];
   const int ntiles = m.T * (m.T + 1) / 2;
-  if ((int)blockIdx.x >= ntiles) return;
   int bi, bj;
-  upper_tile(xcd_remap(blockIdx.x, ntiles), m.T, bi, bj);   // a tile row per L2
+  upper_tile(xcd_remap(local, ntiles), m.T, bi, bj);   // a tile row per L2
   const int n = m.n;
   DenseMK P{m.Y, n, n};
   EpiStore epi{m.U, n, n, n, 1.f, 0.f, bi != bj};
@@ -513,12 +550,13 @@ __global__ __launch_bounds__(NTHREADS) void lauum_kernel(const MatDesc* table) {
 }
 
 // zero the strictly lower triangle (Cholesky-factor output)
-__global__ __launch_bounds__(256) void zero_lower_kernel(const MatDesc* table) {
-  const MatDesc m = table[blockIdx.y];
+__global__ __launch_bounds__(256) void zero_lower_kernel(const MatDesc* table, const WorkList wl) {
+  int mat, local;
+  work_find(wl, mat, local);
+  const MatDesc m = table[mat];
   const int n = m.n;
   const int T = m.T;
-  if ((int)blockIdx.x >= T * T) return;
-  const int bi = blockIdx.x / T, bj = blockIdx.x - bi * T;
+  const int bi = local / T, bj = local - bi * T;
   if (bj > bi) return;
   for (int e = threadIdx.x; e < BM * BN; e += 256) {
     const int row = bi * BM + (e >> 7);
@@ -608,11 +646,27 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
     return c;
   };
 
+  // Runs `launch(worklist)` over the first `count` matrices of the sorted table,
+  // WL_MAX at a time, with items(T) work items for a matrix of T blocks; matrices
+  // without items are skipped at the ends and cost nothing in between.
+  auto for_worklists = [&](int count, auto&& items, auto&& launch) {
+    for (int s0 = 0; s0 < count; s0 += WL_MAX) {
+      WorkList wl;
+      wl.first = s0;
+      wl.n = std::min(WL_MAX, count - s0);
+      wl.cum[0] = 0;
+      for (int i = 0; i < wl.n; ++i) wl.cum[i + 1] = wl.cum[i] + std::max(0, (int)items(Ts[s0 + i]));
+      for (int i = wl.n + 1; i <= WL_MAX; ++i) wl.cum[i] = wl.cum[wl.n];
+      if (wl.cum[wl.n] > 0) launch(wl, wl.cum[wl.n]);
+    }
+  };
+
   bool any_pi = false;
   for (auto& h : mats) any_pi |= h.partner >= 0;
   if (any_pi) hipLaunchKernelGGL(inv_trace_kernel, dim3(nmat), dim3(256), 0, stream, table);
-  hipLaunchKernelGGL(inv_copy_damp_kernel, dim3(Tmax * (Tmax + 1) / 2, nmat), dim3(256), 0, stream,
-                     table, info);
+  for_worklists(nmat, [](int T) { return T * (T + 1) / 2; }, [&](const WorkList& wl, int grid) {
+    hipLaunchKernelGGL(inv_copy_damp_kernel, dim3(grid), dim3(256), 0, stream, table, info, wl);
+  });
 
   for (int P0 = 0; P0 < Tmax; P0 += OUTER_BLOCKS) {
     const int Pend = std::min(P0 + OUTER_BLOCKS, Tmax);
@@ -622,36 +676,52 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
                          p, info);
       const int nb = active(p + 2);
       if (nb == 0) continue;
-      KFAC_LAUNCH_TILE2(potrf_panel_kernel, dim3(Tmax - p - 1, nb), stream, table, p);
+      for_worklists(nb, [&](int T) { return T - p - 1; }, [&](const WorkList& wl, int grid) {
+        KFAC_LAUNCH_TILE2(potrf_panel_kernel, dim3(grid), stream, table, p, wl);
+      });
       if (p + 1 < Pend) {
         // rows (p, Pend) of the outer panel, all columns to the right
-        const int rows = Pend - p - 1, width = Tmax - p - 1;
-        KFAC_LAUNCH_TILE2(potrf_trail_kernel, dim3(rows * width, nb), stream, table, p, 1, p + 1,
-                          Pend);
+        for_worklists(nb,
+                      [&](int T) { return (std::min(Pend, T) - p - 1) * (T - p - 1); },
+                      [&](const WorkList& wl, int grid) {
+                        KFAC_LAUNCH_TILE2(potrf_trail_kernel, dim3(grid), stream, table, p, 1,
+                                          p + 1, Pend, wl);
+                      });
       }
     }
     const int nc = active(Pend + 1);
     if (Pend < Tmax && nc > 0) {
-      const int Tr = Tmax - Pend;
-      KFAC_LAUNCH_TILE2(potrf_trail_kernel, dim3(Tr * (Tr + 1) / 2, nc), stream, table, P0,
-                        Pend - P0, Pend, Tmax);
+      for_worklists(nc, [&](int T) { const int Tr = T - Pend; return Tr * (Tr + 1) / 2; },
+                    [&](const WorkList& wl, int grid) {
+                      KFAC_LAUNCH_TILE2(potrf_trail_kernel, dim3(grid), stream, table, P0,
+                                        Pend - P0, Pend, Tmax, wl);
+                    });
     }
   }
   if (mode == MODE_CHOLESKY) {
-    hipLaunchKernelGGL(zero_lower_kernel, dim3(Tmax * Tmax, nmat), dim3(256), 0, stream, table);
+    for_worklists(nmat, [](int T) { return T * T; }, [&](const WorkList& wl, int grid) {
+      hipLaunchKernelGGL(zero_lower_kernel, dim3(grid), dim3(256), 0, stream, table, wl);
+    });
     return launch_status();
   }
   if (Tmax > 1) {
     int D = 0;
     while ((1 << D) < Tmax) ++D;
     const int na = active(2);
-    const dim3 grid((Tmax - 1) * Tmax / 2, na);
     for (int depth = D - 1; depth >= 0 && na > 0; --depth) {
-      KFAC_LAUNCH_TILE2(trtri_w_kernel, grid, stream, table, depth);
-      KFAC_LAUNCH_TILE2(trtri_y_kernel, grid, stream, table, depth);
+      // matrices with fewer than 2^depth blocks have no merge this deep
+      auto pairs = [&](int T) { return (1 << depth) < T ? (T - 1) * T / 2 : 0; };
+      for_worklists(na, pairs, [&](const WorkList& wl, int grid) {
+        KFAC_LAUNCH_TILE2(trtri_w_kernel, dim3(grid), stream, table, depth, wl);
+      });
+      for_worklists(na, pairs, [&](const WorkList& wl, int grid) {
+        KFAC_LAUNCH_TILE2(trtri_y_kernel, dim3(grid), stream, table, depth, wl);
+      });
     }
   }
-  KFAC_LAUNCH_TILE2(lauum_kernel, dim3(Tmax * (Tmax + 1) / 2, nmat), stream, table);
+  for_worklists(nmat, [](int T) { return T * (T + 1) / 2; }, [&](const WorkList& wl, int grid) {
+    KFAC_LAUNCH_TILE2(lauum_kernel, dim3(grid), stream, table, wl);
+  });
   return launch_status();
 }
 
