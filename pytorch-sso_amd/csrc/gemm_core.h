@@ -392,6 +392,29 @@ __device__ __forceinline__ int xcd_remap(int id, int total) {
   return base + (id >> 3);
 }
 
+// Batched launches (one for many matrices or layers of different sizes) use a 1-D
+// grid of exactly the workgroups needed: cum[i] is the first work item of the i-th
+// listed matrix (table index first + i), cum[n] the grid size.  (A rectangular grid
+// "largest tile count x matrices" would start tens of thousands of workgroups
+// that only find out that their matrix is too small.)
+constexpr int WL_MAX = 128;
+struct WorkList {
+  int n, first;
+  int cum[WL_MAX + 1];
+};
+
+// matrix (table index) and local work item of the calling workgroup
+__device__ __forceinline__ void work_find(const WorkList& wl, int& mat, int& local) {
+  const int item = blockIdx.x;
+  int lo = 0, hi = wl.n;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (wl.cum[mid] <= item) lo = mid; else hi = mid;
+  }
+  mat = wl.first + lo;
+  local = item - wl.cum[lo];
+}
+
 // tile index t (0-based, row-major over the upper triangle incl. diagonal of a
 // T x T block grid) -> (bi, bj), bi <= bj
 __device__ __forceinline__ void upper_tile(int t, int T, int& bi, int& bj) {

@@ -48,29 +48,6 @@ __global__ void inv_setup_kernel(DescChunk chunk, MatDesc* table, int offset, in
   if (i < count) table[offset + i] = chunk.d[i];
 }
 
-// Launches cover the matrices that still have work with a 1-D grid of exactly the
-// workgroups needed: cum[i] is the first work item of the i-th listed matrix
-// (table index first + i), cum[n] the grid size.  (A rectangular grid
-// "largest tile count x matrices" would start tens of thousands of workgroups
-// that only find out that their matrix is too small.)
-constexpr int WL_MAX = 128;
-struct WorkList {
-  int n, first;
-  int cum[WL_MAX + 1];
-};
-
-// matrix (table index) and local work item of the calling workgroup
-__device__ __forceinline__ void work_find(const WorkList& wl, int& mat, int& local) {
-  const int item = blockIdx.x;
-  int lo = 0, hi = wl.n;
-  while (hi - lo > 1) {
-    const int mid = (lo + hi) >> 1;
-    if (wl.cum[mid] <= item) lo = mid; else hi = mid;
-  }
-  mat = wl.first + lo;
-  local = item - wl.cum[lo];
-}
-
 // trace of src (one workgroup per matrix)
 __global__ __launch_bounds__(256) void inv_trace_kernel(MatDesc* table) {
   __shared__ float red[256];

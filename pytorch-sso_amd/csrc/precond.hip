@@ -78,12 +78,14 @@ struct EpiSplit {
 };
 
 template <bool SAMPLE>
-__global__ __launch_bounds__(NTHREADS) void precond_first_kernel(const LayerDesc* table) {
+__global__ __launch_bounds__(NTHREADS) void precond_first_kernel(const LayerDesc* table,
+                                                                 const WorkList wl) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  const LayerDesc m = table[blockIdx.y];
+  int layer, local;
+  work_find(wl, layer, local);
+  const LayerDesc m = table[layer];
   const int ta = tiles128(m.dA), tg = tiles128(m.dG);
-  if ((int)blockIdx.x >= ta * tg) return;
-  const int item = xcd_remap(blockIdx.x, ta * tg);
+  const int item = xcd_remap(local, ta * tg);
   const int bi = item / tg, bj = item - bi * tg;   // bi over dA, bj over dG
   EpiStore epi{m.Tt, m.dG, m.dA, m.dG, 1.f, 0.f, false};
   if (SAMPLE) {
@@ -99,12 +101,14 @@ __global__ __launch_bounds__(NTHREADS) void precond_first_kernel(const LayerDesc
 }
 
 template <bool SAMPLE>
-__global__ __launch_bounds__(NTHREADS) void precond_second_kernel(const LayerDesc* table) {
+__global__ __launch_bounds__(NTHREADS) void precond_second_kernel(const LayerDesc* table,
+                                                                 const WorkList wl) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  const LayerDesc m = table[blockIdx.y];
+  int layer, local;
+  work_find(wl, layer, local);
+  const LayerDesc m = table[layer];
   const int ta = tiles128(m.dA), tg = tiles128(m.dG);
-  if ((int)blockIdx.x >= ta * tg) return;
-  const int item = xcd_remap(blockIdx.x, ta * tg);
+  const int item = xcd_remap(local, ta * tg);
   const int bi = item / ta, bj = item - bi * ta;   // bi over dG, bj over dA
   DenseKM P{m.Tt, nullptr, m.dG, m.dG, 0};
   DenseKM Q{m.R, nullptr, m.dA, m.dA, 0};
@@ -132,7 +136,6 @@ static int run_layers(int layers, const int* dG, const int* dA, const float* con
   LayerDesc* table = (LayerDesc*)workspace;
   char* tbase = (char*)workspace + align256((size_t)layers * sizeof(LayerDesc));
   size_t off = 0;
-  int maxtiles = 0;
   // longest tiles first: the table (= grid.y) is ordered by the reduction length of
   // the second, larger product so that the tail of the launch is made of short tiles
   std::vector<int> order(layers);
@@ -159,18 +162,32 @@ static int run_layers(int layers, const int* dG, const int* dA, const float* con
       d.dAw = dA[l] - (has_bias[l] ? 1 : 0);
       d.scale = scale;
       d.pad = 0;
-      maxtiles = std::max(maxtiles, cdiv(dG[l], BM) * cdiv(dA[l], BN));
     }
     hipLaunchKernelGGL(layer_setup_kernel, dim3(1), dim3(LAYER_CHUNK), 0, stream, chunk, table, s0,
                        cnt);
   }
-  const dim3 grid(maxtiles, layers);
-  if (sample) {
-    KFAC_LAUNCH_TILE2(precond_first_kernel<true>, grid, stream, table);
-    KFAC_LAUNCH_TILE2(precond_second_kernel<true>, grid, stream, table);
-  } else {
-    KFAC_LAUNCH_TILE2(precond_first_kernel<false>, grid, stream, table);
-    KFAC_LAUNCH_TILE2(precond_second_kernel<false>, grid, stream, table);
+  // both products have one tile per 128 x 128 block of the [dG, dA] result; every
+  // first product is enqueued before any second one (stream order is the dependency)
+  for (int pass = 0; pass < 2; ++pass) {
+    for (int s0 = 0; s0 < layers; s0 += WL_MAX) {
+      WorkList wl;
+      wl.first = s0;
+      wl.n = std::min(WL_MAX, layers - s0);
+      wl.cum[0] = 0;
+      for (int i = 0; i < wl.n; ++i) {
+        const int l = order[s0 + i];
+        wl.cum[i + 1] = wl.cum[i] + cdiv(dG[l], BM) * cdiv(dA[l], BN);
+      }
+      for (int i = wl.n + 1; i <= WL_MAX; ++i) wl.cum[i] = wl.cum[wl.n];
+      const dim3 grid(wl.cum[wl.n]);
+      if (pass == 0) {
+        if (sample) KFAC_LAUNCH_TILE2(precond_first_kernel<true>, grid, stream, table, wl);
+        else KFAC_LAUNCH_TILE2(precond_first_kernel<false>, grid, stream, table, wl);
+      } else {
+        if (sample) KFAC_LAUNCH_TILE2(precond_second_kernel<true>, grid, stream, table, wl);
+        else KFAC_LAUNCH_TILE2(precond_second_kernel<false>, grid, stream, table, wl);
+      }
+    }
   }
   return launch_status();
 }
