@@ -186,6 +186,31 @@ def test_precondition_batched(ops, dev):
             assert O.rel_fro(dgb[i], rb) < TOL
 
 
+def test_more_than_128_matrices_and_layers_in_one_call(ops, dev):
+    """The batched launches list their work 128 matrices / layers at a time: 150 of
+    mixed sizes must come out the same as one by one."""
+    dims = [1 + (37 * i) % 300 for i in range(150)]
+    mats = [spd(n, seed=i) for i, n in enumerate(dims)]
+    outs, info = ops.damped_inverse_batched([m.to(dev) for m in mats], [0.05] * len(mats))
+    assert info.cpu().tolist() == [0] * len(mats)
+    for m, o in zip(mats, outs):
+        assert O.rel_fro(o, O.damped_inverse(m, 0.05, D)) < TOL
+    torch.manual_seed(9)
+    shapes = [(1 + (13 * i) % 140, 2 + (29 * i) % 260, i % 2 == 0) for i in range(140)]
+    Gis = [spd(g, seed=1) for g, a, b in shapes]
+    Ais = [spd(a, seed=2) for g, a, b in shapes]
+    gws = [torch.randn(g, a - (1 if b else 0)) for g, a, b in shapes]
+    gbs = [torch.randn(g) if b else None for g, a, b in shapes]
+    dgw = [x.to(dev).clone() for x in gws]
+    dgb = [None if x is None else x.to(dev).clone() for x in gbs]
+    ops.precondition_batched([x.to(dev) for x in Gis], [x.to(dev) for x in Ais], dgw, dgb)
+    for i in range(len(shapes)):
+        rw, rb = O.precondition(Gis[i], Ais[i], gws[i], gbs[i], D)
+        assert O.rel_fro(dgw[i], rw) < TOL
+        if rb is not None:
+            assert O.rel_fro(dgb[i], rb) < TOL
+
+
 def test_precondition_conv_shaped_gradient(ops, dev):
     torch.manual_seed(2)
     Gi, Ai = spd(6), spd(4 * 3 * 3 + 1)
