@@ -45,16 +45,18 @@ int kfac_abi_version(void);
  * K terms (K = rows for Linear, n*h_out*w_out for Conv2d). */
 size_t kfac_factor_workspace_bytes(int d, int64_t K);
 
-/* C = alpha * [x,1]^T [x,1] + beta * C     (C is d x d, d = f + add_bias)
+/* C = alpha * [x,1]^T [x,1] + beta * C_prev     (C is d x d, d = f + add_bias;
+ * C_prev == NULL: the old contents of C; a C_prev different from C lets the
+ * running average be written into a second buffer while C_prev stays intact)
  * x is [rows, f] with row stride ldx.  The ones column is the LAST column.
  * Replaces torch.cat + torch.einsum('ki,kj->ij') + div in
  * torchsso/curv/cov/linear.py:50-59 (A, alpha = 1/n, add_bias = module has
  * bias) and :61-67 with the n^2 rescale of curvature.py:154-155,299-300
  * (G, alpha = n, add_bias = 0).  beta != 0 fuses the accumulation of
  * utils/accumulator.py:23-38 or the running average of curvature.py:185-186
- * into the GEMM epilogue; with beta == 0, C is not read. */
+ * into the GEMM epilogue; with beta == 0, neither C nor C_prev is read. */
 int kfac_factor_linear(const float* x, int64_t rows, int f, int64_t ldx, int add_bias,
-                       float alpha, float beta, float* C,
+                       float alpha, float beta, const float* C_prev, float* C,
                        void* workspace, size_t workspace_bytes, void* stream);
 
 /* Scratch needed by kfac_factor_conv_a for this geometry (it may exceed
@@ -63,7 +65,7 @@ size_t kfac_factor_conv_a_workspace_bytes(int n, int c, int H, int W, int kh, in
                                           int sh, int sw, int ph, int pw, int dh, int dw,
                                           int add_bias);
 
-/* C = alpha * M M^T + beta * C with M = im2col(x) as [c*kh*kw (+1), n*oh*ow],
+/* C = alpha * M M^T + beta * C_prev with M = im2col(x) as [c*kh*kw (+1), n*oh*ow],
  * row order (c, kh, kw), ones ROW last; M is never written to memory.
  * x is [n, c, H, W].  Two kernels, same result: in general the patches are
  * gathered tile by tile into LDS; for a stride-1, bias-free layer with 2..9
@@ -73,15 +75,15 @@ size_t kfac_factor_conv_a_workspace_bytes(int n, int c, int H, int W, int kh, in
  * torchsso/curv/cov/conv.py:47-67 (alpha = 1/n).  groups are ignored, as there. */
 int kfac_factor_conv_a(const float* x, int n, int c, int H, int W,
                        int kh, int kw, int sh, int sw, int ph, int pw, int dh, int dw,
-                       int add_bias, float alpha, float beta, float* C,
+                       int add_bias, float alpha, float beta, const float* C_prev, float* C,
                        void* workspace, size_t workspace_bytes, void* stream);
 
-/* C = alpha * m m^T + beta * C with m = g viewed as [c, n*h*w]; g is
+/* C = alpha * m m^T + beta * C_prev with m = g viewed as [c, n*h*w]; g is
  * [n, c, h, w] and is read in place (no transpose copy).
  * Replaces torchsso/curv/cov/conv.py:69-74 plus the n^2 rescale of
  * curvature.py:154-155,299-300 (alpha = n / (h*w)). */
 int kfac_factor_conv_g(const float* g, int n, int c, int h, int w,
-                       float alpha, float beta, float* C,
+                       float alpha, float beta, const float* C_prev, float* C,
                        void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- Damped factor inversion ------------------------------------------- */

@@ -29,8 +29,8 @@ bool conv_a_taps_applicable(int c, int kh, int kw, int sh, int sw, int add_bias)
 size_t conv_a_taps_workspace(int n, int c, int H, int W, int kh, int kw, int ph, int pw, int dh,
                              int dw);
 int conv_a_taps(const float* x, int n, int c, int H, int W, int kh, int kw, int ph, int pw, int dh,
-                int dw, float alpha, float beta, float* A, void* workspace, size_t workspace_bytes,
-                hipStream_t stream);
+                int dw, float alpha, float beta, const float* A_prev, float* A, void* workspace,
+                size_t workspace_bytes, hipStream_t stream);
 
 inline int launch_status() {
   hipError_t e = hipGetLastError();

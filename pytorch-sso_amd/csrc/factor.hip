@@ -58,8 +58,8 @@ static SyrkPlan plan_syrk(int d, long K) {
 template <class OP, int W>
 __global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void syrk_kernel(OP op, int d, int K, int T, int ntiles,
                                                           int splits, int chunks_per_split,
-                                                          float* C, float alpha, float beta,
-                                                          float* ws) {
+                                                          float* C, const float* Cin,
+                                                          float alpha, float beta, float* ws) {
   constexpr int TS = 64 * W;
   constexpr int KC = Cfg<W, W>::KC;
   extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -74,7 +74,7 @@ __global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void syrk_kernel(OP op,
   int kend = kbeg + chunks_per_split * KC;
   if (kend > K) kend = K;
   if (splits == 1) {
-    EpiStore epi{C, d, d, d, alpha, beta, bi != bj};
+    EpiStore epi{C, d, d, d, alpha, beta, bi != bj, Cin};
     gemm_tile_cfg<W, W>(op, op, bi * TS, bj * TS, kbeg, kend, bi == bj, epi, smem);
   } else {
     EpiPartial epi{ws + ((size_t)split * ntiles + tile) * (TS * TS), bi * TS, bj * TS, d, d, TS};
@@ -90,7 +90,8 @@ __global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void syrk_kernel(OP op,
 template <int TS>
 __global__ __launch_bounds__(256) void syrk_reduce_kernel(const float* ws, int d, int T,
                                                            int ntiles, int splits, float* C,
-                                                           float alpha, float beta) {
+                                                           const float* Cin, float alpha,
+                                                           float beta) {
   __shared__ float4 red[16][16];
   const int tile = blockIdx.x;
   int bi, bj;
@@ -134,7 +135,7 @@ __global__ __launch_bounds__(256) void syrk_reduce_kernel(const float* ws, int d
       if (col < d) {
         const size_t idx = (size_t)row * d + col;
         float o = alpha * vals[k];
-        if (beta != 0.f) o += beta * C[idx];
+        if (beta != 0.f) o += beta * (Cin ? Cin : C)[idx];
         C[idx] = o;
         if (bi != bj) C[(size_t)col * d + row] = o;
       }
@@ -144,31 +145,33 @@ __global__ __launch_bounds__(256) void syrk_reduce_kernel(const float* ws, int d
 
 template <class OP, int W>
 static void launch_syrk_cfg(const OP& op, const SyrkPlan& p, int d, int64_t K, float alpha,
-                            float beta, float* C, void* workspace, hipStream_t stream) {
+                            float beta, const float* Cin, float* C, void* workspace,
+                            hipStream_t stream) {
   constexpr int TS = 64 * W;
   constexpr int lds_bytes = Cfg<W, W>::SMEM_FLOATS * (int)sizeof(float);
   if (!enable_large_lds((const void*)syrk_kernel<OP, W>, lds_bytes)) return;
   hipLaunchKernelGGL((syrk_kernel<OP, W>), dim3(p.ntiles, p.splits), dim3(64 * W * W), lds_bytes,
-                     stream, op, d, (int)K, p.T, p.ntiles, p.splits, p.cps, C, alpha, beta,
+                     stream, op, d, (int)K, p.T, p.ntiles, p.splits, p.cps, C, Cin, alpha, beta,
                      (float*)workspace);
   if (p.splits > 1) {
     hipLaunchKernelGGL((syrk_reduce_kernel<TS>), dim3(p.ntiles, TS * (TS / 64)), dim3(256), 0,
-                       stream, (const float*)workspace, d, p.T, p.ntiles, p.splits, C, alpha, beta);
+                       stream, (const float*)workspace, d, p.T, p.ntiles, p.splits, C, Cin, alpha,
+                       beta);
   }
 }
 
 template <class OP>
-static int launch_syrk(const OP& op, int d, int64_t K, float alpha, float beta, float* C,
-                       void* workspace, size_t workspace_bytes, hipStream_t stream) {
+static int launch_syrk(const OP& op, int d, int64_t K, float alpha, float beta, const float* Cin,
+                       float* C, void* workspace, size_t workspace_bytes, hipStream_t stream) {
   const SyrkPlan p = plan_syrk(d, (long)K);
   if (p.splits > 1) {
     const size_t need = (size_t)p.splits * p.ntiles * p.ts * p.ts * sizeof(float);
     if (workspace == nullptr || workspace_bytes < need) return KFAC_ERR_WORKSPACE;
   }
   if (p.w == 1)
-    launch_syrk_cfg<OP, 1>(op, p, d, K, alpha, beta, C, workspace, stream);
+    launch_syrk_cfg<OP, 1>(op, p, d, K, alpha, beta, Cin, C, workspace, stream);
   else
-    launch_syrk_cfg<OP, 2>(op, p, d, K, alpha, beta, C, workspace, stream);
+    launch_syrk_cfg<OP, 2>(op, p, d, K, alpha, beta, Cin, C, workspace, stream);
   return launch_status();
 }
 
@@ -178,7 +181,7 @@ using namespace kfac;
 
 extern "C" {
 
-int kfac_abi_version(void) { return 1; }
+int kfac_abi_version(void) { return 2; }
 
 size_t kfac_factor_workspace_bytes(int d, int64_t K) {
   if (d <= 0 || K <= 0) return 0;
@@ -218,7 +221,7 @@ size_t kfac_factor_conv_a_workspace_bytes(int n, int c, int H, int W, int kh, in
 }
 
 int kfac_factor_linear(const float* x, int64_t rows, int f, int64_t ldx, int add_bias,
-                       float alpha, float beta, float* C, void* workspace,
+                       float alpha, float beta, const float* C_prev, float* C, void* workspace,
                        size_t workspace_bytes, void* stream) {
   if (!x || !C || rows <= 0 || f <= 0 || ldx < f) return KFAC_ERR_ARG;
   const int d = f + (add_bias ? 1 : 0);
@@ -228,8 +231,9 @@ int kfac_factor_linear(const float* x, int64_t rows, int f, int64_t ldx, int add
   for (int64_t r0 = 0; r0 < rows; r0 += step) {
     const int64_t cnt = rows - r0 < step ? rows - r0 : step;
     DenseKM op{x + r0 * ldx, nullptr, (int)ldx, d, add_bias ? 1 : 0};
-    const int st = launch_syrk(op, d, cnt, alpha, r0 == 0 ? beta : 1.f, C, workspace,
-                               workspace_bytes, (hipStream_t)stream);
+    const int st = launch_syrk(op, d, cnt, alpha, r0 == 0 ? beta : 1.f,
+                               r0 == 0 ? C_prev : nullptr, C, workspace, workspace_bytes,
+                               (hipStream_t)stream);
     if (st != KFAC_OK) return st;
   }
   return KFAC_OK;
@@ -237,7 +241,8 @@ int kfac_factor_linear(const float* x, int64_t rows, int f, int64_t ldx, int add
 
 int kfac_factor_conv_a(const float* x, int n, int c, int H, int W, int kh, int kw, int sh, int sw,
                        int ph, int pw, int dh, int dw, int add_bias, float alpha, float beta,
-                       float* C, void* workspace, size_t workspace_bytes, void* stream) {
+                       const float* C_prev, float* C, void* workspace, size_t workspace_bytes,
+                       void* stream) {
   if (!x || !C || n <= 0 || c <= 0 || H <= 0 || W <= 0 || kh <= 0 || kw <= 0 || sh <= 0 ||
       sw <= 0 || ph < 0 || pw < 0 || dh <= 0 || dw <= 0)
     return KFAC_ERR_ARG;
@@ -254,22 +259,23 @@ int kfac_factor_conv_a(const float* x, int n, int c, int H, int W, int kh, int k
   for (int64_t n0 = 0; n0 < n; n0 += step) {
     const int cnt = (int)(n - n0 < step ? n - n0 : step);
     const float bslice = n0 == 0 ? beta : 1.f;
+    const float* prev = n0 == 0 ? C_prev : nullptr;
     if (kh == 1 && kw == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && !add_bias) {
       // a pointwise convolution: M is the input itself, viewed as [c, n*H*W]
       ConvG op{x + n0 * image, c, H * W};
-      const int st = launch_syrk(op, d, (int64_t)cnt * H * W, alpha, bslice, C, workspace,
+      const int st = launch_syrk(op, d, (int64_t)cnt * H * W, alpha, bslice, prev, C, workspace,
                                  workspace_bytes, (hipStream_t)stream);
       if (st != KFAC_OK) return st;
       continue;
     }
     if (conv_a_taps_applicable(c, kh, kw, sh, sw, add_bias)) {
       const int st = conv_a_taps(x + n0 * image, cnt, c, H, W, kh, kw, ph, pw, dh, dw, alpha,
-                                 bslice, C, workspace, workspace_bytes, (hipStream_t)stream);
+                                 bslice, prev, C, workspace, workspace_bytes, (hipStream_t)stream);
       if (st == KFAC_OK) continue;
       if (st != -1) return st;
     }
     ConvA op{x + n0 * image, c, H, W, kh, kw, sh, sw, ph, pw, dh, dw, OH, OW, d, add_bias ? 1 : 0};
-    const int st = launch_syrk(op, d, (int64_t)cnt * OH * OW, alpha, bslice, C, workspace,
+    const int st = launch_syrk(op, d, (int64_t)cnt * OH * OW, alpha, bslice, prev, C, workspace,
                                workspace_bytes, (hipStream_t)stream);
     if (st != KFAC_OK) return st;
   }
@@ -277,7 +283,8 @@ int kfac_factor_conv_a(const float* x, int n, int c, int H, int W, int kh, int k
 }
 
 int kfac_factor_conv_g(const float* g, int n, int c, int h, int w, float alpha, float beta,
-                       float* C, void* workspace, size_t workspace_bytes, void* stream) {
+                       const float* C_prev, float* C, void* workspace, size_t workspace_bytes,
+                       void* stream) {
   if (!g || !C || n <= 0 || c <= 0 || h <= 0 || w <= 0) return KFAC_ERR_ARG;
   if ((int64_t)c * c * 4 > MAX_OPERAND_BYTES) return KFAC_ERR_ARG;
   const int64_t image = (int64_t)c * h * w;
@@ -286,8 +293,9 @@ int kfac_factor_conv_g(const float* g, int n, int c, int h, int w, float alpha, 
   for (int64_t n0 = 0; n0 < n; n0 += step) {
     const int cnt = (int)(n - n0 < step ? n - n0 : step);
     ConvG op{g + n0 * image, c, h * w};
-    const int st = launch_syrk(op, c, (int64_t)cnt * h * w, alpha, n0 == 0 ? beta : 1.f, C,
-                               workspace, workspace_bytes, (hipStream_t)stream);
+    const int st = launch_syrk(op, c, (int64_t)cnt * h * w, alpha, n0 == 0 ? beta : 1.f,
+                               n0 == 0 ? C_prev : nullptr, C, workspace, workspace_bytes,
+                               (hipStream_t)stream);
     if (st != KFAC_OK) return st;
   }
   return KFAC_OK;

@@ -144,7 +144,7 @@ __global__ __launch_bounds__(256) void block_sum_kernel(const TapPlanDev plan, c
 // channels [8J, 8J+8), all taps: (8T)^2 elements, staged in LDS.
 __global__ __launch_bounds__(256) void interleave_kernel(const TapPlanDev plan, const float* B,
                                                          int C, int T, float alpha, float beta,
-                                                         float* A) {
+                                                         const float* Ain, float* A) {
   __shared__ float region[CT * MAX_TAPS][CT * MAX_TAPS + 1];
   const int I = blockIdx.y, J = blockIdx.x;
   const int d = C * T;
@@ -177,7 +177,7 @@ __global__ __launch_bounds__(256) void interleave_kernel(const TapPlanDev plan, 
     if (r < rows && q < cols) {
       const size_t idx = (size_t)(I * side + r) * d + J * side + q;
       float o = alpha * region[r][q];
-      if (beta != 0.f) o += beta * A[idx];
+      if (beta != 0.f) o += beta * (Ain ? Ain : A)[idx];
       A[idx] = o;
     }
   }
@@ -334,8 +334,8 @@ size_t conv_a_taps_workspace(int n, int c, int H, int W, int kh, int kw, int ph,
 // returns KFAC_OK, an error, or -1 when the geometry is not covered (the caller
 // then uses the im2col kernel)
 int conv_a_taps(const float* x, int n, int c, int H, int W, int kh, int kw, int ph, int pw, int dh,
-                int dw, float alpha, float beta, float* A, void* workspace, size_t workspace_bytes,
-                hipStream_t stream) {
+                int dw, float alpha, float beta, const float* A_prev, float* A, void* workspace,
+                size_t workspace_bytes, hipStream_t stream) {
   const TapPlanHost hp = plan_taps(n, c, H, W, kh, kw, ph, pw, dh, dw);
   if (!hp.ok) return -1;
   if (!workspace || workspace_bytes < hp.partial_floats * sizeof(float)) return KFAC_ERR_WORKSPACE;
@@ -357,7 +357,7 @@ int conv_a_taps(const float* x, int n, int c, int H, int W, int kh, int kw, int 
                      stream, hp.dev, ws, c * c, B);
   const int regions = cdiv(c, CT);
   hipLaunchKernelGGL(interleave_kernel, dim3(regions, regions), dim3(256), 0, stream, hp.dev, B, c,
-                     T, alpha, beta, A);
+                     T, alpha, beta, A_prev, A);
   return launch_status();
 }
 

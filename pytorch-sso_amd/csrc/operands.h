@@ -174,16 +174,18 @@ struct ConvA {
 // Epilogues
 // ---------------------------------------------------------------------------
 
-// C[row][col] = alpha*acc + beta*C_old ; optionally also the mirrored element.
+// C[row][col] = alpha*acc + beta*Cin[row][col] ; optionally also the mirrored
+// element.  Cin == nullptr: the old values of C itself.
 struct EpiStore {
   static constexpr bool reads_output = true;
   float* C;
   int ld, M, N;
   float alpha, beta;
   bool mirror;
+  const float* Cin = nullptr;
   __device__ __forceinline__ bool reads() const { return beta != 0.f; }
   __device__ __forceinline__ float fetch(int row, int col) const {
-    return (row < M && col < N) ? C[(size_t)row * ld + col] : 0.f;
+    return (row < M && col < N) ? (Cin ? Cin : C)[(size_t)row * ld + col] : 0.f;
   }
   __device__ __forceinline__ void store_with(int row, int col, float v, float old) const {
     if (row < M && col < N) {
@@ -196,7 +198,7 @@ struct EpiStore {
     if (row < M && col < N) {
       const size_t idx = (size_t)row * ld + col;
       float o = alpha * v;
-      if (beta != 0.f) o += beta * C[idx];
+      if (beta != 0.f) o += beta * (Cin ? Cin : C)[idx];
       C[idx] = o;
       if (mirror && row != col) C[(size_t)col * ld + row] = o;
     }

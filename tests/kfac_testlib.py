@@ -164,26 +164,30 @@ class OracleOps(object):
 
     dtype = torch.float32
 
-    def factor_linear(self, x, add_bias, alpha, out=None, beta=0.):
+    def factor_linear(self, x, add_bias, alpha, out=None, beta=0., prev=None):
         n = x.shape[0]
         r = O.factor_linear_a(x, add_bias, self.dtype) * (n * alpha)
-        return self._emit(r, out, beta)
+        return self._emit(r, out, beta, prev)
 
-    def factor_conv_a(self, x, kernel_size, stride, padding, dilation, add_bias, alpha, out=None, beta=0.):
+    def factor_conv_a(self, x, kernel_size, stride, padding, dilation, add_bias, alpha, out=None, beta=0.,
+                      prev=None):
         n = x.shape[0]
         r = O.factor_conv_a(x, kernel_size, stride, padding, dilation, add_bias, self.dtype) * (n * alpha)
-        return self._emit(r, out, beta)
+        return self._emit(r, out, beta, prev)
 
-    def factor_conv_g(self, g, alpha, out=None, beta=0.):
+    def factor_conv_g(self, g, alpha, out=None, beta=0., prev=None):
         n, c, h, w = g.shape
         r = O.factor_conv_g(g, self.dtype, scale_by_batch=False) * (n * h * w * alpha)
-        return self._emit(r, out, beta)
+        return self._emit(r, out, beta, prev)
 
     @staticmethod
-    def _emit(r, out, beta):
+    def _emit(r, out, beta, prev=None):
+        old = out if prev is None else prev
+        if beta != 0:
+            r = r + beta * old
         if out is None:
             return r
-        out.copy_(r + beta * out)
+        out.copy_(r)
         return out
 
     def pi_damped_inverse_batched(self, As, Gs, dampings, A_invs=None, G_invs=None, info=None):

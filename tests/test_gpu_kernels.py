@@ -52,6 +52,11 @@ def test_factor_linear_fused_running_average(ops, dev):
         out = ops.factor_linear(x.to(dev), True, 0.95 / n, out=old.to(dev).clone(), beta=0.05)
         ref = 0.95 * O.factor_linear_a(x, True, D) + 0.05 * old.double()
         assert O.rel_fro(out, ref) < TOL
+        # the same into a second buffer: the previous average stays untouched
+        prev = old.to(dev).clone()
+        nxt = torch.full_like(prev, float('nan'))
+        ops.factor_linear(x.to(dev), True, 0.95 / n, out=nxt, beta=0.05, prev=prev)
+        assert O.rel_fro(nxt, ref) < TOL and torch.equal(prev.cpu(), old)
 
 
 @pytest.mark.parametrize('shape,k,s,p,d,bias', [
@@ -111,6 +116,9 @@ def test_factor_conv_a_by_correlations(ops, dev, shape, k, p, d):
     out = ops.factor_conv_a(x.to(dev), k, (1, 1), p, d, False, 0.9 / shape[0],
                             out=old.to(dev).clone(), beta=0.1)
     assert O.rel_fro(out, 0.9 * ref + 0.1 * old.double()) < TOL
+    prev = old.to(dev).clone()
+    nxt = ops.factor_conv_a(x.to(dev), k, (1, 1), p, d, False, 0.9 / shape[0], beta=0.1, prev=prev)
+    assert O.rel_fro(nxt, 0.9 * ref + 0.1 * old.double()) < TOL and torch.equal(prev.cpu(), old)
 
 
 @pytest.mark.parametrize('shape', [(1, 1, 1, 1), (2, 3, 4, 4), (8, 64, 7, 7), (4, 130, 14, 14),
@@ -121,6 +129,11 @@ def test_factor_conv_g(ops, dev, shape):
     n, c, h, w = shape
     out = ops.factor_conv_g(g.to(dev), float(n) / (h * w))
     assert O.rel_fro(out, O.factor_conv_g(g, D)) < TOL
+    old = spd(c)
+    prev = old.to(dev).clone()
+    nxt = ops.factor_conv_g(g.to(dev), 0.5 * float(n) / (h * w), beta=0.5, prev=prev)
+    assert O.rel_fro(nxt, 0.5 * O.factor_conv_g(g, D) + 0.5 * old.double()) < TOL
+    assert torch.equal(prev.cpu(), old)
 
 
 DIMS = [1, 2, 31, 32, 33, 64, 96, 97, 127, 128, 129, 255, 256, 257, 300, 513, 785]
