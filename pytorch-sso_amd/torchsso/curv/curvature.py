@@ -222,7 +222,14 @@ class DiagCurvature(Curvature):
 
 
 class KronCurvature(Curvature):
-    """Kronecker-factored curvature A (x) G (reference: curvature.py:255-331)."""
+    """Kronecker-factored curvature A (x) G (reference: curvature.py:255-331).
+
+    With `fuse_ema` set (SecondOrderOptimizer does it when no accumulation over
+    micro-steps needs the raw factors) the factor kernels write the running
+    average themselves: a hook builds  ema_decay * factor + (1 - ema_decay) * ema
+    into a second buffer (`_next`) in the epilogue of the factor product, and
+    `update_ema` just swaps the two buffers.  The raw factor is then never
+    stored; `data`, `A` and `G` rebuild it on demand from the two averages."""
 
     kind = 'kron'
 
@@ -230,20 +237,89 @@ class KronCurvature(Curvature):
         super(KronCurvature, self).__init__(*args, **kwargs)
         self._A = None
         self._G = None
+        self.fuse_ema = False
+        self._next = [None, None]        # receives the next running average
+        self._fresh = [False, False]     # _next[i] holds the next average (hook ran since the last step)
+        self._prev_ok = [False, False]   # _next[i] holds the average before the current one
+
+    # ---- raw factors ------------------------------------------------------------
+
+    def _build_factor(self, idx, build):
+        """Runs `build(scale, out, beta, prev)` (a factor kernel computing
+        out = scale * factor + beta * prev) either for the raw factor or, in
+        fused mode, for the next running average."""
+        beta = self.ema_decay
+        if self.fuse_ema and self.ema is not None and beta != 1:
+            ema = self.ema[idx]
+            nxt = self._next[idx]
+            if nxt is None or nxt.shape != ema.shape:
+                nxt = torch.empty_like(ema)
+            self._next[idx] = build(beta, nxt, 1. - beta, ema)
+            self._fresh[idx] = True
+            self._prev_ok[idx] = False
+            raw = None
+        else:
+            raw = build(1., None, 0., None)
+            self._fresh[idx] = False
+        if idx == 0:
+            self._A = raw
+        else:
+            self._G = raw
+
+    def _raw(self, idx):
+        t = self._A if idx == 0 else self._G
+        if t is None and self.ema is not None and (self._fresh[idx] or self._prev_ok[idx]):
+            # factor = (newer average - (1 - beta) * older average) / beta
+            beta = self.ema_decay
+            newer, older = ((self._next[idx], self.ema[idx]) if self._fresh[idx]
+                            else (self.ema[idx], self._next[idx]))
+            t = newer.clone()
+            _ops.axpby_batched([older], [t], -(1. - beta) / beta, 1. / beta)
+        return t
 
     @property
     def data(self):
-        return [self._A, self._G]
+        return [self._raw(0), self._raw(1)]
 
     @data.setter
     def data(self, value):
         self._A, self._G = value
+        self._fresh = [False, False]
 
     @property
     def shape(self):
         if self._A is None or self._G is None:
             return self._get_shape()
         return self._A.shape, self._G.shape
+
+    def _advance_average(self, xs, ys, stale):
+        """update_ema in fused mode.  Factors whose next average is ready: swap the
+        buffers.  Factors built the ordinary way go to the (xs, ys) lists of the
+        axpby launch.  A factor that no hook has rebuilt since the last step
+        enters again, as in the reference, where `data` simply persists:
+        beta * factor + (1 - beta) * ema  with  factor = (ema - (1 - beta) * prev) / beta
+        is (2 - beta) * ema - (1 - beta) * prev, written over prev (`stale` list)."""
+        for idx in (0, 1):
+            raw = self._A if idx == 0 else self._G
+            if self._fresh[idx]:
+                self.ema[idx], self._next[idx] = self._next[idx], self.ema[idx]
+                self._fresh[idx] = False
+                self._prev_ok[idx] = True
+            elif raw is not None:
+                xs.append(raw.contiguous())
+                ys.append(self.ema[idx])
+                self._prev_ok[idx] = False
+            elif self._prev_ok[idx]:
+                stale.append((self, idx))
+            else:
+                raise RuntimeError('update_ema: no factor has been built for %s'
+                                   % type(self._module).__name__)
+
+    def load_state_dict(self, state):
+        super(KronCurvature, self).load_state_dict(state)
+        self._next = [None, None]
+        self._fresh = [False, False]
+        self._prev_ok = [False, False]
 
     def _get_shape(self):
         raise NotImplementedError
@@ -255,11 +331,11 @@ class KronCurvature(Curvature):
 
     @property
     def A(self):
-        return self._A
+        return self._raw(0)
 
     @property
     def G(self):
-        return self._G
+        return self._raw(1)
 
     def adjust_data_scale(self, scale):
         self._G.mul_(scale)
@@ -291,9 +367,15 @@ def update_ema_all(curvs):
     """Curvature.update_ema for every curvature in the list
     (reference: curvature.py:174-191).  ema_decay weighs the NEW data."""
     by_beta = {}
+    stale = []
     for c in curvs:
-        data = c.data
         beta = c.ema_decay
+        if c.kind == 'kron' and c.fuse_ema and c.ema is not None and beta != 1:
+            xs, ys = by_beta.setdefault(beta, ([], []))
+            c._advance_average(xs, ys, stale)
+            c._l2_reg_ema = c._l2_reg * beta + c._l2_reg_ema * (1 - beta)
+            continue
+        data = c.data
         if c.ema is None or beta == 1:
             if c.ema is None:
                 c.ema = [d.clone() for d in data]
@@ -310,6 +392,10 @@ def update_ema_all(curvs):
             c._l2_reg_ema = c._l2_reg * beta + c._l2_reg_ema * (1 - beta)
     for beta, (xs, ys) in by_beta.items():
         _ops.axpby_batched(xs, ys, beta, 1 - beta)
+    for c, idx in stale:
+        beta = c.ema_decay
+        _ops.axpby_batched([c.ema[idx]], [c._next[idx]], 2. - beta, -(1. - beta))
+        c.ema[idx], c._next[idx] = c._next[idx], c.ema[idx]
     xs, ys = [], []
     for c in curvs:
         if c.use_max_ema:

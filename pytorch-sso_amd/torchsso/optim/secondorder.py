@@ -112,12 +112,22 @@ class SecondOrderOptimizer(Optimizer):
         # (secondorder.py:94-106), which current torch no longer tolerates.
         super(SecondOrderOptimizer, self).__init__(groups, defaults)
 
+        # Without accumulation over micro-steps nothing reads the raw Kronecker
+        # factors between the hooks and step(): the factor kernels then write the
+        # running average themselves (curvature.py, KronCurvature.fuse_ema).
+        if acc_steps == 1 and self._fuse_running_average:
+            for group in self.param_groups:
+                if type(group['curv']) in (torchsso.KronCovLinear, torchsso.KronCovConv2d):
+                    group['curv'].fuse_ema = True
+
         for group in self.param_groups:
             self.init_buffer(group['params'])
         for group in bn_groups:
             group['l2_reg'] = 0
             group['weight_decay'] = 0
             group['normalizing_weights'] = False
+
+    _fuse_running_average = True     # VIOptimizer accumulates over MC samples: off there
 
     def init_buffer(self, params):
         for p in params:

@@ -13,6 +13,7 @@ import torch.nn.functional as F
 import torchsso
 from torchsso import _hip, _ops
 import kfac_testlib as T
+from oracle import kfac_oracle as O
 
 
 @pytest.fixture
@@ -252,6 +253,66 @@ def test_iteration_lr_schedules():
     fresh = torch.optim.SGD(model.parameters(), lr=0.4)
     with pytest.raises(KeyError):
         L.GradualWarmupIterLR(fresh, 0.0, 4, last_iter=3)
+
+
+def test_running_average_written_by_the_factor_kernels(oracle_ops):
+    """With acc_steps == 1 the hooks build beta*factor + (1-beta)*ema straight into
+    a second buffer and update_ema swaps buffers.  Same numbers as the unfused
+    sequence; `data` is rebuilt on demand; a step without new factors re-applies
+    the previous ones, as the reference's persistent `data` does."""
+    gold = T.load_golden('ref_convnet_kfac')
+    x, y = torch.from_numpy(gold['x']), torch.from_numpy(gold['y'])
+
+    def make(fuse):
+        model = T.load_init(T.build_convnet(), gold)
+        opt = torchsso.optim.SecondOrderOptimizer(
+            model, 'Cov', {'Linear': 'Kron', 'Conv2d': 'Kron', 'BatchNorm2d': 'Diag'},
+            {'damping': 1e-2, 'ema_decay': 0.9}, lr=0.02, momentum=0.5, l2_reg=1e-4)
+        kron = [g['curv'] for g in opt.param_groups if g['curv'].kind == 'kron']
+        assert all(c.fuse_ema for c in kron)
+        if not fuse:
+            for c in kron:
+                c.fuse_ema = False
+        return model, opt, kron
+
+    (ma, oa, ka), (mb, ob, kb) = make(True), make(False)
+    for step in range(3):
+        seen = {}
+
+        def closure_a():
+            ret = _closure(ma, x, y)()
+            seen['raw'] = [[d.clone() for d in c.data] for c in ka]
+            seen['stored'] = [c._A is None and c._G is None for c in ka]
+            return ret
+        oa.step(closure=closure_a)
+        ob.step(closure=_closure(mb, x, y))
+        # first step: no average yet, the raw factors are stored; afterwards they are not
+        assert seen['stored'] == [step > 0] * len(ka)
+        for ca, cb, raw in zip(ka, kb, seen['raw']):
+            for ea, eb, ra, rb in zip(ca.ema, cb.ema, raw, cb.data):
+                assert O.rel_fro(ea, eb) < 1e-6
+                assert O.rel_fro(ra, rb) < 1e-5          # rebuilt from the two averages
+            assert abs(ca.damping - cb.damping) < 1e-12
+    for p, q in zip(ma.parameters(), mb.parameters()):
+        assert O.rel_fro(p.detach(), q.detach()) < 1e-6
+    # a step with no forward/backward in between: the last factors enter again
+    for m in (ma, mb):
+        for p in m.parameters():
+            p.grad = torch.ones_like(p) * 1e-3
+    oa.step()
+    ob.step()
+    for ca, cb in zip(ka, kb):
+        for ea, eb in zip(ca.ema, cb.ema):
+            assert O.rel_fro(ea, eb) < 1e-5
+    # accumulation over micro-steps and VI keep the raw factors
+    m2 = T.load_init(T.build_convnet(), gold)
+    o2 = torchsso.optim.SecondOrderOptimizer(m2, 'Cov', {'Linear': 'Kron', 'Conv2d': 'Kron'},
+                                             {'damping': 1e-2, 'ema_decay': 0.9}, acc_steps=2)
+    assert not any(getattr(g['curv'], 'fuse_ema', False) for g in o2.param_groups)
+    m3 = T.build_mlp()
+    o3 = torchsso.optim.VIOptimizer(m3, 100, 'Cov', {'Linear': 'Kron'},
+                                    {'damping': 1e-3, 'ema_decay': 0.95}, num_mc_samples=2)
+    assert not any(g['curv'].fuse_ema for g in o3.param_groups)
 
 
 def test_constructor_validation_and_class_lookup():
