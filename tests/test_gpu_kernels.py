@@ -350,6 +350,26 @@ def test_factor_linearity_at_full_size(ops, dev):
     assert O.rel_fro(one, u @ u.t()) < TOL
 
 
+@pytest.mark.parametrize('c,hw,stride', [(128, 28, 1), (256, 14, 1), (512, 7, 1), (256, 28, 2)])
+def test_conv_a_at_resnet50_shapes_against_unfold_on_device(ops, dev, c, hw, stride):
+    """The 3x3 layers of BASELINE config 3 at batch 32 (d = 1152 / 2304 / 4608, both the
+    correlation path and the strided im2col path) against F.unfold + matmul in float64
+    on the device (library routines)."""
+    torch.manual_seed(c + hw)
+    x = torch.randn(32, c, hw, hw, device=dev)
+    out = ops.factor_conv_a(x, (3, 3), (stride, stride), (1, 1), (1, 1), False, 1.0 / 32)
+    ref = torch.zeros(9 * c, 9 * c, dtype=D, device=dev)
+    for i in range(0, 32, 4):
+        u = torch.nn.functional.unfold(x[i:i + 4].double(), 3, padding=1, stride=stride)
+        u = u.transpose(0, 1).reshape(9 * c, -1)
+        ref += u @ u.t()
+    ref /= 32
+    assert O.rel_fro(out, ref) < TOL
+    assert torch.equal(out, out.t())
+    ev = torch.linalg.eigvalsh(out.double())
+    assert ev.min().item() > -1e-4 * ev.max().item()       # a Gram matrix: positive semi-definite
+
+
 # ---- diagonal covariance of Linear / Conv2d (VOGN) ------------------------------------
 
 @pytest.mark.parametrize('n,fin,fout,bias', [(1, 1, 1, True), (7, 5, 3, False), (128, 784, 1000, True),
