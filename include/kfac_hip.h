@@ -261,6 +261,27 @@ int kfac_rowsq_sum(const float* x, int64_t rows, int channels, int len,
 int kfac_bn_diag_combine(const float* sx, const float* sg, int n, int channels, float alpha,
                          float* w_curv, float* b_curv, void* stream);
 
+/* ---- Wire format: triangular packing ------------------------------------ */
+
+/* The reference ships factors between ranks as one flat fp32 buffer: arrays back
+ * to back, a symmetric matrix as its upper triangle row by row (element (y, x),
+ * x >= y, at n*y - y*(y+1)/2 + x -- what cuBLAS strttp(FILL_MODE_LOWER) makes of
+ * the row-major array), anything else whole.  Replaces Packer.pack / unpack and
+ * the 'unpack' element-wise kernel of
+ * torchsso/utils/chainer_communicators/_utility.py:16-104.  Per array i (HOST
+ * arrays): numel[i] elements; triangular[i] != 0: a dims[i] x dims[i] matrix
+ * (numel[i] == dims[i]^2).  The list starts at buffer + offset (in elements);
+ * kfac_packed_numel gives its length.  unpack fills both triangles. */
+size_t kfac_pack_workspace_bytes(int count);
+int64_t kfac_packed_numel(int count, const int64_t* numel, const int* dims,
+                          const int* triangular);
+int kfac_pack_batched(int count, const float* const* arrays, const int64_t* numel,
+                      const int* dims, const int* triangular, float* buffer, int64_t offset,
+                      void* workspace, size_t workspace_bytes, void* stream);
+int kfac_unpack_batched(int count, float* const* arrays, const int64_t* numel,
+                        const int* dims, const int* triangular, const float* buffer,
+                        int64_t offset, void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

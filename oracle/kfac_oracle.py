@@ -30,6 +30,8 @@ which retypes the formula):
                        logits layer equals mean_n(diag(p_n) - p_n p_n^T) (closed form)
   cholesky_upper       U^T U == X, U upper, diag > 0
   sample               injected-noise Kronecker identity
+  tri_pack / unpack    the reference's own index formula evaluated by loops
+                       (utils/chainer_communicators/_utility.py:19-31), round trip
   kfac_step / vi_step  golden vectors written by the reference itself
                        (tests/golden/*.npz) and torch.optim.SGD equivalence
 The reference ships no golden vectors or known-answer tests for this path.
@@ -394,6 +396,31 @@ def sgd_tail(p, grad, buf, lr, momentum=0., weight_decay=0.):
 # --------------------------------------------------------------------------
 # helpers
 # --------------------------------------------------------------------------
+
+def tri_pack(mat):
+    """Upper triangle of a square matrix, row by row: the packed form in which the
+    reference sends symmetric factors (cuBLAS strttp with FILL_MODE_LOWER on the
+    row-major array, torchsso/utils/chainer_communicators/_utility.py:59-86)."""
+    n = mat.shape[0]
+    iu = torch.triu_indices(n, n)
+    return mat[iu[0], iu[1]]
+
+
+def tri_unpack(vec, n):
+    """Symmetric n x n matrix from its packed upper triangle: element (y, x) and
+    (x, y) are vec[n*y - y*(y+1)/2 + x] for x >= y (_utility.py:19-31)."""
+    out = torch.empty(n, n, dtype=vec.dtype)
+    iu = torch.triu_indices(n, n)
+    out[iu[0], iu[1]] = vec
+    out[iu[1], iu[0]] = vec
+    return out
+
+
+def pack_arrays(arrays):
+    """Flat buffer of a list of (tensor, triangular): arrays back to back, symmetric
+    ones as triangles (Packer.pack, _utility.py:33-44)."""
+    return torch.cat([tri_pack(t) if tri else t.reshape(-1) for t, tri in arrays])
+
 
 def rel_fro(x, ref):
     """||x - ref||_F / ||ref||_F in float64."""

@@ -59,6 +59,12 @@ _SIGNATURES = {
                                    c_ptr, c_size, c_ptr]),
     'kfac_diag_inverse_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_int,
                                           c_ptr, c_size, c_ptr]),
+    'kfac_pack_workspace_bytes': (c_size, [c_int]),
+    'kfac_packed_numel': (c_i64, [c_int, c_ptr, c_ptr, c_ptr]),
+    'kfac_pack_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64,
+                                  c_ptr, c_size, c_ptr]),
+    'kfac_unpack_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64,
+                                    c_ptr, c_size, c_ptr]),
     'kfac_sqrt_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_size, c_ptr]),
     'kfac_max_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_size, c_ptr]),
     'kfac_diag_sample_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,

@@ -436,3 +436,53 @@ def scale_rows(x, w, use_sqrt):
                              _hip.stream_ptr(x.device))
     _hip.check(st, 'kfac_scale_rows')
     return out
+
+
+def _pack_lists(arrays):
+    """arrays: list of (tensor, triangular).  Returns tensors, numel, dims, flags."""
+    tensors, numel, dims, flags = [], [], [], []
+    for i, (t, tri) in enumerate(arrays):
+        if tri and (t.dim() != 2 or t.shape[0] != t.shape[1]):
+            raise RuntimeError('non square matrix')
+        if not t.is_contiguous():
+            raise _hip.KfacHipError('pack/unpack: array %d is not contiguous' % i)
+        tensors.append(t)
+        numel.append(t.numel())
+        dims.append(t.shape[0] if tri else 0)
+        flags.append(1 if tri else 0)
+    return tensors, numel, dims, flags
+
+
+def packed_numel(arrays):
+    """Length in elements of the packed form of a list of (tensor, triangular)."""
+    return sum(t.shape[0] * (t.shape[0] + 1) // 2 if tri else t.numel() for t, tri in arrays)
+
+
+def pack_batched(arrays, buf, offset=0):
+    """Packs a list of (tensor, triangular) into the flat buffer `buf` from element
+    `offset` on; returns the offset behind the last array."""
+    return _pack_call(arrays, buf, offset, False)
+
+
+def unpack_batched(arrays, buf, offset=0):
+    """Inverse of pack_batched: fills the tensors (both triangles of a symmetric one)."""
+    return _pack_call(arrays, buf, offset, True)
+
+
+def _pack_call(arrays, buf, offset, unpack):
+    lib = _hip.load()
+    if len(arrays) == 0:
+        return offset
+    tensors, numel, dims, flags = _pack_lists(arrays)
+    total = packed_numel(arrays)
+    if buf.dim() != 1 or not buf.is_contiguous() or offset < 0 or offset + total > buf.numel():
+        raise _hip.KfacHipError('pack/unpack: buffer of %d elements cannot hold %d from offset %d'
+                                % (buf.numel(), total, offset))
+    dev = buf.device
+    ws, ws_bytes = _hip.workspace(dev, lib.kfac_pack_workspace_bytes(len(tensors)))
+    fn = lib.kfac_unpack_batched if unpack else lib.kfac_pack_batched
+    st = fn(len(tensors), _hip.ptr_array(tensors, 'array'), _hip.i64_array(numel),
+            _hip.int_array(dims), _hip.int_array(flags), _hip.dev_ptr(buf, 'buffer'), int(offset),
+            _ws_ptr(ws), ws_bytes, _hip.stream_ptr(dev))
+    _hip.check(st, 'kfac_unpack_batched' if unpack else 'kfac_pack_batched')
+    return offset + total

@@ -291,6 +291,28 @@ def _oracle_diag_cov_conv2d(self, g, x, kernel_size, stride, padding, dilation, 
     return out[0].reshape(c_out, -1) * (n * alpha)
 
 
+def _oracle_pack_batched(self, arrays, buf, offset=0):
+    flat = O.pack_arrays(arrays)
+    buf[offset:offset + flat.numel()] = flat
+    return offset + flat.numel()
+
+
+def _oracle_unpack_batched(self, arrays, buf, offset=0):
+    for t, tri in arrays:
+        n = t.shape[0] * (t.shape[0] + 1) // 2 if tri else t.numel()
+        seg = buf[offset:offset + n]
+        t.copy_(O.tri_unpack(seg, t.shape[0]) if tri else seg.reshape(t.shape))
+        offset += n
+    return offset
+
+
+def _oracle_packed_numel(self, arrays):
+    return sum(t.shape[0] * (t.shape[0] + 1) // 2 if tri else t.numel() for t, tri in arrays)
+
+
+OracleOps.pack_batched = _oracle_pack_batched
+OracleOps.unpack_batched = _oracle_unpack_batched
+OracleOps.packed_numel = _oracle_packed_numel
 OracleOps.sqrt_batched = _oracle_sqrt_batched
 OracleOps.max_batched = _oracle_max_batched
 OracleOps.diag_sample_batched = _oracle_diag_sample_batched

@@ -370,6 +370,44 @@ def test_conv_a_at_resnet50_shapes_against_unfold_on_device(ops, dev, c, hw, str
     assert ev.min().item() > -1e-4 * ev.max().item()       # a Gram matrix: positive semi-definite
 
 
+# ---- wire format ----------------------------------------------------------------------
+
+def test_pack_and_unpack_against_the_oracle(ops, dev):
+    torch.manual_seed(31)
+    arrays = []
+    for n in (1, 2, 63, 64, 65, 130, 1000):
+        a = torch.randn(n, n)
+        arrays.append((a + a.t(), True))
+        arrays.append((torch.randn(n, 3), False))
+    arrays.append((torch.randn(5000), False))
+    total = ops.packed_numel(arrays)
+    want = O.pack_arrays(arrays)
+    assert total == want.numel()
+    buf = torch.full((total + 11,), float('nan'), device=dev)
+    end = ops.pack_batched([(t.to(dev), tri) for t, tri in arrays], buf, 11)
+    assert end == total + 11
+    assert torch.equal(buf[11:].cpu(), want) and torch.isnan(buf[:11]).all()
+    outs = [(torch.full_like(t, float('nan')).to(dev), tri) for t, tri in arrays]
+    ops.unpack_batched(outs, buf, 11)
+    for (o, _), (t, _) in zip(outs, arrays):
+        assert torch.equal(o.cpu(), t)
+    # more arrays than one launch lists, and a factor of the largest benchmark size
+    many = [(torch.randn(3 + i % 40, 3 + i % 40), i % 3 != 0) for i in range(150)]
+    many = [((t + t.t()) if tri else t, tri) for t, tri in many]
+    buf = torch.empty(ops.packed_numel(many), device=dev)
+    ops.pack_batched([(t.to(dev), tri) for t, tri in many], buf)
+    assert torch.equal(buf.cpu(), O.pack_arrays(many))
+    big = torch.randn(4608, 4608, device=dev)
+    big = big + big.t()
+    buf = torch.empty(4608 * 4609 // 2, device=dev)
+    ops.pack_batched([(big, True)], buf)
+    back = torch.empty_like(big)
+    ops.unpack_batched([(back, True)], buf)
+    assert torch.equal(back, big)
+    iu = torch.triu_indices(4608, 4608, device=dev)
+    assert torch.equal(buf, big[iu[0], iu[1]])
+
+
 # ---- diagonal covariance of Linear / Conv2d (VOGN) ------------------------------------
 
 @pytest.mark.parametrize('n,fin,fout,bias', [(1, 1, 1, True), (7, 5, 3, False), (128, 784, 1000, True),

@@ -315,6 +315,43 @@ def test_running_average_written_by_the_factor_kernels(oracle_ops):
     assert not any(g['curv'].fuse_ema for g in o3.param_groups)
 
 
+def test_packer_and_extractors_lay_out_the_wire_buffer(oracle_ops):
+    from torchsso.utils import packer as P
+    gold = T.load_golden('ref_mlp_kfac')
+    model = T.load_init(T.build_mlp(), gold)
+    x, y = torch.from_numpy(gold['x']), torch.from_numpy(gold['y'])
+    opt = torchsso.optim.SecondOrderOptimizer(model, 'Cov', {'Linear': 'Kron'},
+                                              {'damping': 1e-3, 'ema_decay': 0.95}, lr=0.05)
+    opt.step(closure=_closure(model, x, y))
+    # two rank blocks (layers 0-1 | layer 2): gradients whole, running averages as triangles
+    extractors = [P.extract_attr_from_params('grad'), P.extract_attr_from_curv('ema', True)]
+    arrays = P.extract(opt.param_groups, [[0, 1], [2]], extractors)
+    assert [len(a) for a in arrays] == [8, 4]
+    assert [tri for _, tri in arrays[0]] == [False, False, True, True] * 2
+    n = P.get_nelems(arrays)
+    want = 0
+    for g in opt.param_groups:
+        want += sum(p.numel() for p in g['params'])
+        want += sum(e.shape[0] * (e.shape[0] + 1) // 2 for e in g['curv'].ema)
+    assert n == want
+    buf = torch.zeros(n + 7)
+    packer = P.Packer()
+    assert packer.pack(arrays, buf, offset=7) == n + 7
+    first = opt.param_groups[0]
+    assert torch.equal(buf[7:7 + first['params'][0].numel()], first['params'][0].grad.reshape(-1))
+    # a reduced buffer coming back: unpack restores full symmetric matrices
+    saved = [[t.clone() for t, _ in a] for a in arrays]
+    for a in arrays:
+        for t, _ in a:
+            t.zero_()
+    packer.unpack(arrays, buf, offset=7)
+    for a, sv in zip(arrays, saved):
+        for (t, tri), ref in zip(a, sv):
+            assert torch.equal(t, ref)
+    with pytest.raises(RuntimeError):          # 'non square matrix', as the reference raises
+        _ops._pack_lists([(torch.zeros(2, 3), True)])
+
+
 def test_constructor_validation_and_class_lookup():
     model = nn.Sequential(nn.Linear(4, 3))
     kw = dict(curv_type='Cov', curv_shapes={'Linear': 'Kron'}, curv_kwargs={'damping': 1e-3})

@@ -371,3 +371,31 @@ def test_fisher_factors_reduce_to_cov_and_match_the_presoftmax_closed_form():
         G += O.fisher_linear_g(grad_k, p[:, k], D)
     closed = sum(torch.diag(p[i]) - torch.outer(p[i], p[i]) for i in range(n)) / n
     assert torch.allclose(G, closed, atol=1e-12)
+
+
+def test_triangular_wire_format_matches_the_reference_index_formula():
+    """mat[i] = vec[n*y - y*(y+1)/2 + x] with (y, x) = sorted(i // n, i % n): the
+    reference's unpack kernel, evaluated literally."""
+    torch.manual_seed(21)
+    for n in (1, 2, 5, 9):
+        a = torch.randn(n, n, dtype=D)
+        sym = a + a.t()
+        vec = O.tri_pack(sym)
+        assert vec.numel() == n * (n + 1) // 2
+        back = torch.empty(n * n, dtype=D)
+        for i in range(n * n):
+            x, y = i % n, i // n
+            if x < y:
+                x, y = y, x
+            back[i] = vec[n * y - y * (y + 1) // 2 + x]
+        assert torch.equal(back.reshape(n, n), sym)
+        assert torch.equal(O.tri_unpack(vec, n), sym)
+        # packing walks the rows from the diagonal to the right (what strttp writes)
+        k = 0
+        for y in range(n):
+            for x in range(y, n):
+                assert vec[k] == sym[y, x]
+                k += 1
+    g = torch.randn(3, 4, dtype=D)
+    buf = O.pack_arrays([(sym, True), (g, False)])
+    assert buf.numel() == 45 + 12 and torch.equal(buf[45:], g.reshape(-1))
