@@ -50,6 +50,29 @@ static SyrkPlan plan_syrk(int d, long K) {
   if (cps < 1) cps = 1;
   splits = (nchunks + cps - 1) / cps;
   if (splits < 1) splits = 1;
+  if (p.w == 2) {
+    // All workgroups of up to 3 per CU are resident at once and share the CU's matrix
+    // cores, so the launch takes (workgroups on the fullest CU) x (chunks per split):
+    // a few more splits can take a whole round off.  Every extra split costs one more
+    // partial tile written and read (the last term, in chunk times).
+    const int ncu = 256;
+    auto cost = [&](long s, long c) {
+      return (double)cdiv((int)(s * p.ntiles), ncu) * (c + 3) + (s > 1 ? 0.035 * s * p.ntiles : 0.);
+    };
+    double best = cost(splits, cps);
+    long best_s = splits, best_cps = cps;
+    for (long s = splits + 1; s <= max_splits && s * p.ntiles <= 3 * ncu; ++s) {
+      const long c = (nchunks + s - 1) / s;
+      if ((nchunks + c - 1) / c != s) continue;
+      if (cost(s, c) < best) {
+        best = cost(s, c);
+        best_s = s;
+        best_cps = c;
+      }
+    }
+    splits = best_s;
+    cps = best_cps;
+  }
   p.splits = (int)splits;
   p.cps = (int)cps;
   return p;

@@ -118,26 +118,49 @@ __global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void corr_kernel(
   gemm_tile_cfg<W, W>(P, Q, bi * TS, bj * TS, kbeg, kend, false, epi, smem);
 }
 
-// B[pair][c][c'] = sum over the pair's jobs and their k-splits, in a fixed order
+// B[pair][c][c'] = sum over the pair's jobs and their k-splits, in a fixed order.
+// One workgroup owns 64 float4 groups of the block; its 4 waves take the partials
+// (all splits of all jobs, as one list) round-robin, two loads in flight each, and
+// the 4 wave sums are added in wave order.
 __global__ __launch_bounds__(256) void block_sum_kernel(const TapPlanDev plan, const float* ws,
                                                         int CC, float* B) {
+  __shared__ float4 red[4][64];
   const int pair = blockIdx.y;
   const int jb = plan.pair_first[pair], je = plan.pair_first[pair + 1];
-  const int e = (blockIdx.x * 256 + threadIdx.x) * 4;
-  if (e >= CC) return;        // CC is a multiple of 4 (channel counts are >= 16 and even)
+  const int lane = threadIdx.x & 63, sl = threadIdx.x >> 6;
+  const int e = (blockIdx.x * 64 + lane) * 4;   // CC is a multiple of 4 (channel counts are even, >= 16)
+  const bool live = e < CC;
   float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int q = jb; q < je; ++q) {
-    const JobDesc jd = plan.jobs[plan.pair_jobs[q]];
-    const float* part = ws + (size_t)jd.part0 * CC + e;
-    for (int sp = 0; sp < jd.splits; ++sp) {
-      const float4 v = *reinterpret_cast<const float4*>(part + (size_t)sp * CC);
-      s.x += v.x;
-      s.y += v.y;
-      s.z += v.z;
-      s.w += v.w;
+  int turn = 0;                                 // position in the pair's list of partials, mod 4
+  if (live) {
+    for (int q = jb; q < je; ++q) {
+      const JobDesc jd = plan.jobs[plan.pair_jobs[q]];
+      const float* part = ws + (size_t)jd.part0 * CC + e;
+      int sp = (sl - turn) & 3;                 // first split of this job that is this wave's turn
+      for (; sp + 4 < jd.splits; sp += 8) {
+        const float4 v0 = *reinterpret_cast<const float4*>(part + (size_t)sp * CC);
+        const float4 v1 = *reinterpret_cast<const float4*>(part + (size_t)(sp + 4) * CC);
+        s.x += v0.x; s.y += v0.y; s.z += v0.z; s.w += v0.w;
+        s.x += v1.x; s.y += v1.y; s.z += v1.z; s.w += v1.w;
+      }
+      if (sp < jd.splits) {
+        const float4 v = *reinterpret_cast<const float4*>(part + (size_t)sp * CC);
+        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+      }
+      turn = (turn + jd.splits) & 3;
     }
   }
-  *reinterpret_cast<float4*>(B + (size_t)pair * CC + e) = s;
+  red[sl][lane] = s;
+  __syncthreads();
+  if (sl == 0 && live) {
+    float4 t = red[0][lane];
+#pragma unroll
+    for (int k = 1; k < 4; ++k) {
+      const float4 v = red[k][lane];
+      t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
+    }
+    *reinterpret_cast<float4*>(B + (size_t)pair * CC + e) = t;
+  }
 }
 
 // One workgroup writes the region of A that couples channels [8I, 8I+8) with
@@ -353,7 +376,7 @@ int conv_a_taps(const float* x, int n, int c, int H, int W, int kh, int kw, int 
     hipLaunchKernelGGL(corr_kernel<2>, dim3(hp.items), dim3(256), lds, stream, x, n, c, H, W,
                        hp.dev, hp.tiles_side, ws);
   }
-  hipLaunchKernelGGL(block_sum_kernel, dim3(cdiv(c * c / 4, 256), hp.dev.npairs), dim3(256), 0,
+  hipLaunchKernelGGL(block_sum_kernel, dim3(cdiv(c * c / 4, 64), hp.dev.npairs), dim3(256), 0,
                      stream, hp.dev, ws, c * c, B);
   const int regions = cdiv(c, CT);
   hipLaunchKernelGGL(interleave_kernel, dim3(regions, regions), dim3(256), 0, stream, hp.dev, B, c,
