@@ -20,8 +20,8 @@
 //  3. block_sum_kernel: B[(t,t')][c][c'] = sum over the block's jobs and their
 //     k-splits, in a fixed order (t <= t');
 //  4. interleave_kernel: A[(c,t),(c',t')] = alpha * B + beta * A_old, with the
-//     blocks below the diagonal taken transposed; an 8x8-channel region of A goes
-//     through LDS so that both the reads of B and the writes of A are row-contiguous.
+//     blocks below the diagonal taken transposed; the elements pass through LDS so
+//     that both the reads of B and the writes of A are row-contiguous.
 #include <limits.h>
 #include <string.h>
 
@@ -71,7 +71,8 @@ constexpr int MAX_JOBS = 64;
 constexpr int MAX_TAPS = 9;
 constexpr int MAX_PAIRS = MAX_TAPS * (MAX_TAPS + 1) / 2;
 constexpr int MAX_PAIR_JOBS = 512;     // pool shared by all pairs
-constexpr int CT = 8;                  // channels per side of an interleave region
+constexpr int IL_ROWS = 16;            // interleave_kernel: channels per workgroup along the rows
+constexpr int IL_COLS = 32;            //                    and along the columns of A
 
 // The whole plan travels as a kernel argument (below the 4 KiB limit).
 struct TapPlanDev {
@@ -163,46 +164,65 @@ __global__ __launch_bounds__(256) void block_sum_kernel(const TapPlanDev plan, c
   }
 }
 
-// One workgroup writes the region of A that couples channels [8I, 8I+8) with
-// channels [8J, 8J+8), all taps: (8T)^2 elements, staged in LDS.
+// One workgroup writes, for one tap t, the rows (c, t) of 16 channels c against the
+// columns (c', t') of 32 channels c' and all taps t': 16 runs of 32*T consecutive
+// elements of A.  The T blocks B[(t,t')] that feed them are read along their rows
+// (blocks below the diagonal: the transposed block, along its rows as well) and
+// go through LDS into the interleaved order.
 __global__ __launch_bounds__(256) void interleave_kernel(const TapPlanDev plan, const float* B,
                                                          int C, int T, float alpha, float beta,
                                                          const float* Ain, float* A) {
-  __shared__ float region[CT * MAX_TAPS][CT * MAX_TAPS + 1];
-  const int I = blockIdx.y, J = blockIdx.x;
+  __shared__ float out[IL_ROWS][IL_COLS * MAX_TAPS + 1];
+  const int t = blockIdx.z;
+  const int c0 = blockIdx.y * IL_ROWS, q0 = blockIdx.x * IL_COLS;
   const int d = C * T;
   const size_t CC = (size_t)C * C;
-  const int total = T * T * CT * CT;
-  for (int e = threadIdx.x; e < total; e += 256) {
-    const int tt = e / (CT * CT);
-    const int ij = e - tt * (CT * CT);
-    const int t = tt / T, t2 = tt - t * T;
-    float v = 0.f;
+  const int tid = threadIdx.x;
+  for (int t2 = 0; t2 < T; ++t2) {
     if (t <= t2) {
-      // B[(t,t2)][c][c2], read along c2
-      const int i = ij / CT, j = ij - i * CT;
-      const int c = I * CT + i, c2 = J * CT + j;
-      if (c < C && c2 < C) v = B[plan.pair_of[t * T + t2] * CC + (size_t)c * C + c2];
-      region[i * T + t][j * T + t2] = v;
+      // B[(t,t2)][c][c2]: lanes along c2
+      const float* blk = B + plan.pair_of[t * T + t2] * CC;
+      const int j = tid % IL_COLS;
+#pragma unroll
+      for (int k = 0; k < IL_ROWS * IL_COLS / 256; ++k) {
+        const int i = tid / IL_COLS + (256 / IL_COLS) * k;
+        const int c = c0 + i, c2 = q0 + j;
+        out[i][j * T + t2] = (c < C && c2 < C) ? blk[(size_t)c * C + c2] : 0.f;
+      }
     } else {
-      // transposed block: B[(t2,t)][c2][c], read along c
-      const int j = ij / CT, i = ij - j * CT;
-      const int c = I * CT + i, c2 = J * CT + j;
-      if (c < C && c2 < C) v = B[plan.pair_of[t2 * T + t] * CC + (size_t)c2 * C + c];
-      region[i * T + t][j * T + t2] = v;
+      // transposed block B[(t2,t)][c2][c]: lanes along c
+      const float* blk = B + plan.pair_of[t2 * T + t] * CC;
+      const int i = tid % IL_ROWS;
+#pragma unroll
+      for (int k = 0; k < IL_ROWS * IL_COLS / 256; ++k) {
+        const int j = tid / IL_ROWS + (256 / IL_ROWS) * k;
+        const int c = c0 + i, c2 = q0 + j;
+        out[i][j * T + t2] = (c < C && c2 < C) ? blk[(size_t)c2 * C + c] : 0.f;
+      }
     }
   }
   __syncthreads();
-  const int side = CT * T;
-  const int rows = min(side, d - I * side), cols = min(side, d - J * side);
-  for (int e = threadIdx.x; e < side * side; e += 256) {
-    const int r = e / side, q = e - r * side;
-    if (r < rows && q < cols) {
-      const size_t idx = (size_t)(I * side + r) * d + J * side + q;
-      float o = alpha * region[r][q];
-      if (beta != 0.f) o += beta * (Ain ? Ain : A)[idx];
-      A[idx] = o;
+  const int ncols = min(IL_COLS, C - q0) * T;       // run length in A
+  const int nrows = min(IL_ROWS, C - c0);
+  const int total = nrows * ncols;
+  const float* prev = Ain ? Ain : A;
+  constexpr int BATCH = 6;
+  for (int e0 = tid; e0 < total; e0 += 256 * BATCH) {
+    float old[BATCH];
+    size_t idx[BATCH];
+    float val[BATCH];
+#pragma unroll
+    for (int k = 0; k < BATCH; ++k) {
+      const int e = e0 + 256 * k;
+      const int i = e / ncols, q = e - i * ncols;
+      const bool in = e < total;
+      idx[k] = in ? (size_t)((c0 + i) * T + t) * d + (size_t)q0 * T + q : 0;
+      val[k] = in ? out[i][q] : 0.f;
+      old[k] = (in && beta != 0.f) ? prev[idx[k]] : 0.f;
     }
+#pragma unroll
+    for (int k = 0; k < BATCH; ++k)
+      if (e0 + 256 * k < total) A[idx[k]] = alpha * val[k] + beta * old[k];
   }
 }
 
@@ -378,8 +398,8 @@ int conv_a_taps(const float* x, int n, int c, int H, int W, int kh, int kw, int 
   }
   hipLaunchKernelGGL(block_sum_kernel, dim3(cdiv(c * c / 4, 64), hp.dev.npairs), dim3(256), 0,
                      stream, hp.dev, ws, c * c, B);
-  const int regions = cdiv(c, CT);
-  hipLaunchKernelGGL(interleave_kernel, dim3(regions, regions), dim3(256), 0, stream, hp.dev, B, c,
+  hipLaunchKernelGGL(interleave_kernel, dim3(cdiv(c, IL_COLS), cdiv(c, IL_ROWS), T), dim3(256), 0,
+                     stream, hp.dev, B, c,
                      T, alpha, beta, A_prev, A);
   return launch_status();
 }
