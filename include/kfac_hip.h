@@ -261,6 +261,19 @@ int kfac_rowsq_sum(const float* x, int64_t rows, int channels, int len,
 int kfac_bn_diag_combine(const float* sx, const float* sg, int n, int channels, float alpha,
                          float* w_curv, float* b_curv, void* stream);
 
+/* The backward half of the BatchNorm diagonal curvature in one call:
+ *   w_curv[c] = alpha * sum_n sx[n][c] * (sum_hw g[n][c][hw]^2),
+ *   b_curv[c] = alpha * sum_n (sum_hw g[n][c][hw]^2)            (b_curv may be NULL),
+ * i.e. kfac_rowsq_sum on grad_output followed by kfac_bn_diag_combine
+ * (cov/batchnorm.py:38-49, alpha as above).  For rows of up to 1024 elements one launch
+ * does both and the row sums never reach memory; longer rows take the two kernels and
+ * need kfac_bn_diag_cov_workspace_bytes(n, channels) bytes of workspace (the short-row
+ * path ignores it). */
+size_t kfac_bn_diag_cov_workspace_bytes(int n, int channels);
+int kfac_bn_diag_cov(const float* g, int n, int channels, int len, const float* sx, float alpha,
+                     float* w_curv, float* b_curv, void* workspace, size_t workspace_bytes,
+                     void* stream);
+
 /* ---- Wire format: triangular packing ------------------------------------ */
 
 /* The reference ships factors between ranks as one flat fp32 buffer: arrays back

@@ -1,6 +1,8 @@
 // HBM-bound tails of the K-FAC step, each one launch over a whole list of
 // tensors: running average / accumulation, diagonal (BatchNorm) curvature,
 // diagonal inverse and preconditioning, and the fused parameter update.
+#include <limits.h>
+
 #include <algorithm>
 #include <vector>
 
@@ -303,6 +305,135 @@ __global__ __launch_bounds__(256) void bn_combine_kernel(const float* sx, const 
   }
 }
 
+// Short rows (len up to 1024): one workgroup takes one channel c and all N samples,
+// i.e. the rows x + (n*C + c)*len.  A wave has 8 or 16 loads (float4 where the rows
+// allow it) in flight: UNROLL rows of CHUNKS loads each.  The 8 partial sums of a lane are
+// folded with 10 shuffles (halving the number of values a lane carries at each of the
+// first three steps).  COMBINE = false writes the row sums out[n*C + c]; COMBINE = true
+// keeps them in LDS and finishes the BatchNorm curvature of the channel,
+//   w_curv[c] = alpha * sum_n sx[n][c] * rowsum[n],  b_curv[c] = alpha * sum_n rowsum[n],
+// summed over n in order, so that neither the row sums nor a second launch touch memory.
+// These launches are short and run from a cold instruction cache: the code is kept small
+// (no per-row index arithmetic, few shuffles).
+constexpr int BN_MAX_ROWS = 2048;      // samples per workgroup
+
+template <int CHUNKS, bool VEC, bool COMBINE>
+__global__ __launch_bounds__(256) void bn_rows_kernel(const float* x, const float* scale,
+                                                      const float* shift, int N, int C, int len,
+                                                      const float* sx, float alpha, float* out,
+                                                      float* w_curv, float* b_curv) {
+  constexpr int UNROLL = CHUNKS == 4 ? 4 : 8;      // rows in flight per wave
+  __shared__ float rowsum[COMBINE ? BN_MAX_ROWS : 1];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int c = blockIdx.x;
+  const int units = VEC ? len >> 2 : len;          // loads per row
+  const float sh = shift ? shift[c] : 0.f;
+  const float rs = scale ? 1.f / scale[c] : 1.f;
+  const long stride = (long)C * len;               // from sample to sample
+  const float* base = x + (long)c * len;
+  for (int q0 = wave * UNROLL; q0 < N; q0 += 4 * UNROLL) {
+    // every load is issued unconditionally, at an index clamped into the row (and the row
+    // into the samples), so that nothing separates the loads; what a clamped load brought
+    // is dropped when the squares are summed
+    float4 v[UNROLL][CHUNKS];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const float* p = base + (long)min(q0 + u, N - 1) * stride;
+#pragma unroll
+      for (int k = 0; k < CHUNKS; ++k) {
+        const int i = min(lane + 64 * k, units - 1);
+        if (VEC)
+          v[u][k] = reinterpret_cast<const float4*>(p)[i];
+        else
+          v[u][k].x = p[i];
+      }
+    }
+    float s[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s[u] = 0.f;
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+#pragma unroll
+      for (int k = 0; k < CHUNKS; ++k) {
+        const float a = (v[u][k].x - sh) * rs;
+        float t = a * a;
+        if (VEC) {
+          const float b = (v[u][k].y - sh) * rs, c2 = (v[u][k].z - sh) * rs;
+          const float d = (v[u][k].w - sh) * rs;
+          t += b * b + c2 * c2 + d * d;
+        }
+        s[u] += (lane + 64 * k < units && q0 + u < N) ? t : 0.f;
+      }
+    }
+    // fold: after the steps with masks 32, 16, 8 a lane carries one value, that of row
+    // 4*bit5 + 2*bit4 + bit3 of its lane number; masks 4, 2, 1 finish the sum
+#pragma unroll
+    for (int half = 4, m = 32; half >= 1; half >>= 1, m >>= 1) {
+      const bool up = lane & m;
+#pragma unroll
+      for (int j = 0; j < half; ++j) {
+        const float send = up ? s[j] : s[j + half];
+        const float keep = up ? s[j + half] : s[j];
+        s[j] = keep + __shfl_xor(send, m);
+      }
+    }
+    float r = s[0];
+#pragma unroll
+    for (int m = 4; m > 0; m >>= 1) r += __shfl_xor(r, m);
+    const int q = q0 + ((lane >> 5) & 1) * 4 + ((lane >> 4) & 1) * 2 + ((lane >> 3) & 1);
+    if ((lane & 7) == 0 && q < q0 + UNROLL && q < N) {
+      if (COMBINE)
+        rowsum[q] = r;
+      else
+        out[(long)q * C + c] = r;
+    }
+  }
+  if (COMBINE) {
+    __shared__ float prod[BN_MAX_ROWS];
+    __syncthreads();
+    // sx[n][c] * rowsum[n] by all threads, then one thread adds over n in order
+    for (int q = threadIdx.x; q < N; q += 256) prod[q] = sx[(long)q * C + c] * rowsum[q];
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float sw = 0.f, sb = 0.f;
+#pragma unroll 8
+      for (int n = 0; n < N; ++n) {
+        sw += prod[n];
+        sb += rowsum[n];
+      }
+      w_curv[c] = alpha * sw;
+      if (b_curv) b_curv[c] = alpha * sb;
+    }
+  }
+}
+
+// Launch of bn_rows_kernel when the shape suits it (false: the caller takes the
+// general kernels).
+template <bool COMBINE>
+static bool launch_bn_rows(const float* x, const float* scale, const float* shift, int N, int C,
+                           int len, const float* sx, float alpha, float* out, float* w_curv,
+                           float* b_curv, hipStream_t stream) {
+  const bool vec = (len & 3) == 0 && ((uintptr_t)x & 15) == 0;
+  const int units = vec ? len >> 2 : len;
+  if (units > 256 || N > BN_MAX_ROWS) return false;
+  const int chunks = units <= 64 ? 1 : (units <= 128 ? 2 : 4);
+  const dim3 grid(C), block(256);
+#define KFAC_BN_ROWS(CH, V)                                                                  \
+  hipLaunchKernelGGL((bn_rows_kernel<CH, V, COMBINE>), grid, block, 0, stream, x, scale, shift, \
+                     N, C, len, sx, alpha, out, w_curv, b_curv)
+  if (vec) {
+    if (chunks == 1) KFAC_BN_ROWS(1, true);
+    else if (chunks == 2) KFAC_BN_ROWS(2, true);
+    else KFAC_BN_ROWS(4, true);
+  } else {
+    if (chunks == 1) KFAC_BN_ROWS(1, false);
+    else if (chunks == 2) KFAC_BN_ROWS(2, false);
+    else KFAC_BN_ROWS(4, false);
+  }
+#undef KFAC_BN_ROWS
+  return true;
+}
+
 }  // namespace kfac
 
 using namespace kfac;
@@ -400,16 +531,48 @@ int kfac_sgd_update_batched(int count, const int64_t* numel, float* const* param
   return run_vec<OP_SGD>(d, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
+static void launch_rowsq(const float* x, int64_t rows, int channels, int len, const float* scale,
+                         const float* shift, float* out, hipStream_t stream) {
+  if (rows % channels == 0 && rows / channels <= INT_MAX &&
+      launch_bn_rows<false>(x, scale, shift, (int)(rows / channels), channels, len, nullptr, 0.f,
+                            out, nullptr, nullptr, stream))
+    return;
+  if (len <= 256)
+    hipLaunchKernelGGL(rowsq_kernel<4>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, x,
+                       scale, shift, (long)rows, channels, len, out);
+  else
+    hipLaunchKernelGGL(rowsq_kernel<1>, dim3((unsigned)rows), dim3(256), 0, stream, x, scale,
+                       shift, (long)rows, channels, len, out);
+}
+
 int kfac_rowsq_sum(const float* x, int64_t rows, int channels, int len, const float* scale,
                    const float* shift, float* out, void* stream) {
   if (!x || !out || rows <= 0 || channels <= 0 || len <= 0 || rows >= (int64_t)1 << 31)
     return KFAC_ERR_ARG;
-  if (len <= 256)
-    hipLaunchKernelGGL(rowsq_kernel<4>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
-                       (hipStream_t)stream, x, scale, shift, (long)rows, channels, len, out);
-  else
-    hipLaunchKernelGGL(rowsq_kernel<1>, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, x,
-                       scale, shift, (long)rows, channels, len, out);
+  launch_rowsq(x, rows, channels, len, scale, shift, out, (hipStream_t)stream);
+  return launch_status();
+}
+
+size_t kfac_bn_diag_cov_workspace_bytes(int n, int channels) {
+  return n > 0 && channels > 0 ? (size_t)n * channels * sizeof(float) : 0;
+}
+
+int kfac_bn_diag_cov(const float* g, int n, int channels, int len, const float* sx, float alpha,
+                     float* w_curv, float* b_curv, void* workspace, size_t workspace_bytes,
+                     void* stream) {
+  if (!g || !sx || !w_curv || n <= 0 || channels <= 0 || len <= 0 ||
+      (int64_t)n * channels >= (int64_t)1 << 31)
+    return KFAC_ERR_ARG;
+  hipStream_t st = (hipStream_t)stream;
+  if (launch_bn_rows<true>(g, nullptr, nullptr, n, channels, len, sx, alpha, nullptr, w_curv,
+                           b_curv, st))
+    return launch_status();
+  if (!workspace || workspace_bytes < kfac_bn_diag_cov_workspace_bytes(n, channels))
+    return KFAC_ERR_WORKSPACE;
+  float* sg = (float*)workspace;
+  launch_rowsq(g, (int64_t)n * channels, channels, len, nullptr, nullptr, sg, st);
+  hipLaunchKernelGGL(bn_combine_kernel, dim3(cdiv(channels, 64)), dim3(256), 0, st, sx, sg, n,
+                     channels, alpha, w_curv, b_curv);
   return launch_status();
 }
 

@@ -119,13 +119,32 @@ constexpr int DIAG_SMEM_BYTES = (2 * DB * DLD + 64 * WLD) * (int)sizeof(float);
 // block of the row panel to the right; pcol < 0: none, the lanes shadow the leaf).
 // Lane j keeps its column in registers.  Each step needs row c of the leaf in every
 // lane: the leaf lanes write their element to a 64-float LDS buffer private to
-// the wave and all lanes read the row back with broadcast ds_read_b128 (no
-// cross-lane register traffic).  The panel columns see the same eliminations as
-// the leaf columns, so the strip ends up holding U[q][*] without a triangular
-// solve.  Several waves may run this on the same leaf with different panel
-// blocks (the leaf is then factored redundantly; only `owner` writes it out, as
-// a dense 32x32 copy `ubuf`, which the caller copies over the leaf in S once all
-// waves are past reading it, and which feeds the back substitution).
+// the wave and all lanes read the row back with broadcast ds_read_b128.  The steps
+// are software-pipelined: step c first finishes element c+1 of the column, publishes
+// it (two buffers alternate) and issues the reads of row c+1, and only then applies
+// row c to the rest of the column, so the LDS round trip of the next row runs under
+// those FMAs; the pivot itself comes through v_readlane and does not wait for LDS.
+// The panel columns see the same eliminations as the leaf columns, so the strip ends
+// up holding U[q][*] without a triangular solve.  Several waves may run this on the
+// same leaf with different panel blocks (the leaf is then factored redundantly; only
+// `owner` writes it out, as a dense 32x32 copy `ubuf`, which the caller copies over
+// the leaf in S once all waves are past reading it, and which feeds the back
+// substitution).
+__device__ __forceinline__ float lane_value(float v, int src_lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src_lane));
+}
+
+__device__ __forceinline__ void read_row(const lds_f* rowbuf, int first, float (&row)[32]) {
+#pragma unroll
+  for (int g = first / 4; g < 8; ++g) {
+    const v4f v = *(const lds_f4*)(rowbuf + 4 * g);
+    row[4 * g + 0] = v.x;
+    row[4 * g + 1] = v.y;
+    row[4 * g + 2] = v.z;
+    row[4 * g + 3] = v.w;
+  }
+}
+
 __device__ __forceinline__ void chol_strip_32(lds_f* S, lds_f* rowbuf, lds_f* ubuf, int c0,
                                               int pcol, bool owner, int row_base, int* info) {
   const int lane = threadIdx.x & 63;
@@ -136,31 +155,33 @@ __device__ __forceinline__ void chol_strip_32(lds_f* S, lds_f* rowbuf, lds_f* ub
 #pragma unroll
   for (int i = 0; i < 32; ++i) a[i] = S[(c0 + i) * DLD + col];
   int bad = 0;
+  // A[c][c0 + j] after the updates of the earlier steps; the panel lanes write into
+  // the unused second half of the buffer, so that the store is unconditional
+  float row[32];
+  rowbuf[lane] = a[0];
+  __builtin_amdgcn_wave_barrier();
+  read_row(rowbuf, 0, row);
 #pragma unroll
   for (int c = 0; c < 32; ++c) {
-    // A[c][c0 + j] after the updates of the earlier steps; the panel lanes write
-    // into the unused second half of the buffer, so that the store is unconditional
-    rowbuf[lane] = a[c];
-    __builtin_amdgcn_wave_barrier();
-    float row[32];
-#pragma unroll
-    for (int g = c / 4; g < 8; ++g) {
-      const v4f v = *(const lds_f4*)(rowbuf + 4 * g);
-      row[4 * g + 0] = v.x;
-      row[4 * g + 1] = v.y;
-      row[4 * g + 2] = v.z;
-      row[4 * g + 3] = v.w;
-    }
-    const float piv = row[c];
+    const float piv = lane_value(a[c], c);
     if (!(piv > 0.f) && bad == 0) bad = row_base + c0 + c + 1;
-    // 1/sqrt in one instruction: the next step's pivot row waits on this chain
+    // 1/sqrt in one instruction: the next step's pivot waits on this chain
     const float rd = __builtin_amdgcn_rsqf(piv);
-    const float d = piv * rd;
     const float f = a[c] * (rd * rd);
+    float next[32];
+    if (c + 1 < 32) {
+      a[c + 1] = fmaf(-row[c + 1], f, a[c + 1]);
+      lds_f* const nb = rowbuf + 64 * ((c + 1) & 1);
+      nb[lane] = a[c + 1];
+      __builtin_amdgcn_wave_barrier();
+      read_row(nb, c + 1, next);
+    }
 #pragma unroll
-    for (int i = c + 1; i < 32; ++i) a[i] = fmaf(-row[i], f, a[i]);   // A[i][col] -= U[c][i] U[c][col]
+    for (int i = c + 2; i < 32; ++i) a[i] = fmaf(-row[i], f, a[i]);   // A[i][col] -= U[c][i] U[c][col]
     const float u = a[c] * rd;
-    a[c] = leaf ? (j > c ? u : (j == c ? d : 0.f)) : u;
+    a[c] = leaf ? (j > c ? u : (j == c ? piv * rd : 0.f)) : u;
+#pragma unroll
+    for (int i = c + 1; i < 32; ++i) row[i] = next[i];
   }
   if (owner && bad != 0 && lane == 0) {
     if (*info == 0) *info = bad;
@@ -282,20 +303,20 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
   const int t = threadIdx.x;
   const int wave = t >> 6;
 
-  // load the upper triangle; pad with the identity up to 128.  16 loads are
-  // issued before the first is used, so the block costs 4 memory round trips
+  // load the upper triangle; pad with the identity up to 128.  32 loads are
+  // issued before the first is used, so the block costs 2 memory round trips
   // instead of 64.
-  for (int e0 = 0; e0 < DB * DB; e0 += 256 * 16) {
-    float v[16];
+  for (int e0 = 0; e0 < DB * DB; e0 += 256 * 32) {
+    float v[32];
 #pragma unroll
-    for (int u = 0; u < 16; ++u) {
+    for (int u = 0; u < 32; ++u) {
       const int e = e0 + u * 256 + t;
       const int i = e >> 7, j = e & 127;
       const bool in = i < nb && j < nb && j >= i;
       v[u] = m.U[in ? (size_t)(r0 + i) * n + r0 + j : (size_t)r0 * n + r0];
     }
 #pragma unroll
-    for (int u = 0; u < 16; ++u) {
+    for (int u = 0; u < 32; ++u) {
       const int e = e0 + u * 256 + t;
       const int i = e >> 7, j = e & 127;
       const bool in = i < nb && j < nb && j >= i;
@@ -306,17 +327,19 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
   }
   __syncthreads();
 
-  // Scratch (in Wt, free until the doubling below): a 64-float row buffer per
+  // Scratch (in Wt, free until the doubling below): two 64-float row buffers per
   // wave and two dense leaf copies, used alternately.
-  lds_f* const rowbuf = Wt + 64 * wave;
-  lds_f* const ubuf0 = Wt + 256;
+  lds_f* const rowbuf = Wt + 128 * wave;
+  lds_f* const ubuf0 = Wt + 512;
   const int nq = (nb + 31) / 32;
-  for (int q = 0; q < nq; ++q) {
+  // One more turn than there are leaves: the last one only inverts the last leaf
+  // (a second call site would be a second copy of that code, fetched cold).
+  for (int q = 0; q <= nq; ++q) {
     const int c0 = 32 * q;
     const int rest = nq - q - 1;     // 32-blocks to the right
     if (wave < 3) {
       // waves 0..2: the strip of leaf q, each with one block of the row panel
-      if (wave == 0 || wave < rest)
+      if (q < nq && (wave == 0 || wave < rest))
         chol_strip_32(S, rowbuf, ubuf0 + 1024 * (q & 1), c0, wave < rest ? c0 + 32 * (wave + 1) : -1,
                       wave == 0, r0, info + m.out);
     } else if (q > 0) {
@@ -324,6 +347,7 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
       backsub_32(ubuf0 + 1024 * ((q - 1) & 1), Yb, c0 - 32);
     }
     __syncthreads();
+    if (q == nq) break;
     if (wave == 0 && (t & 32) == 0) {
       // the factored leaf replaces A[q][q] now that no wave reads the original any more
       const lds_f* ub = ubuf0 + 1024 * (q & 1);
@@ -343,8 +367,6 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
       __syncthreads();
     }
   }
-  if (wave == 3) backsub_32(ubuf0 + 1024 * ((nq - 1) & 1), Yb, 32 * (nq - 1));
-  __syncthreads();
 
   // inverse of the whole block by doubling: 32 -> 64 -> 128
   if (nq > 1) {

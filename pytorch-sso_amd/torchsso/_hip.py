@@ -81,6 +81,9 @@ _SIGNATURES = {
     'kfac_scale_rows': (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_int, c_ptr, c_ptr]),
     'kfac_rowsq_sum': (c_int, [c_ptr, c_i64, c_int, c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     'kfac_bn_diag_combine': (c_int, [c_ptr, c_ptr, c_int, c_int, c_f32, c_ptr, c_ptr, c_ptr]),
+    'kfac_bn_diag_cov_workspace_bytes': (c_size, [c_int, c_int]),
+    'kfac_bn_diag_cov': (c_int, [c_ptr, c_int, c_int, c_int, c_ptr, c_f32, c_ptr, c_ptr, c_ptr,
+                                 c_size, c_ptr]),
 }
 
 

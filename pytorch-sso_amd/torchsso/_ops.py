@@ -423,6 +423,30 @@ def bn_diag_combine(sx, sg, alpha, bias):
     return w, b
 
 
+def bn_diag_cov(grad_output, channels, sx, alpha, bias):
+    """(w_curv, b_curv) of a BatchNorm layer from the output gradient and the forward
+    hook's [n, c] sums sx: alpha * sum_n sx * sum_hw g^2 and alpha * sum_n sum_hw g^2."""
+    lib = _hip.load()
+    g = grad_output.contiguous()
+    n = g.shape[0]
+    if g.shape[1] != channels or tuple(sx.shape) != (n, channels):
+        raise _hip.KfacHipError('bn_diag_cov: grad_output %s, sums %s, %d channels'
+                                % (tuple(g.shape), tuple(sx.shape), channels))
+    length = g.numel() // (n * channels)
+    w = torch.empty(channels, dtype=torch.float32, device=g.device)
+    b = torch.empty(channels, dtype=torch.float32, device=g.device) if bias else None
+    # the row sums of long rows pass through memory
+    ws = (torch.empty((n, channels), dtype=torch.float32, device=g.device)
+          if length > 256 or n > 2048 else None)
+    st = lib.kfac_bn_diag_cov(_hip.dev_ptr(g, 'grad_output'), n, channels, length,
+                              _hip.dev_ptr(sx, 'sx'), float(alpha), w.data_ptr(),
+                              None if b is None else b.data_ptr(),
+                              None if ws is None else ws.data_ptr(),
+                              0 if ws is None else ws.numel() * 4, _hip.stream_ptr(g.device))
+    _hip.check(st, 'kfac_bn_diag_cov')
+    return w, b
+
+
 def scale_rows(x, w, use_sqrt):
     """x[r] * (sqrt(w[r]) if use_sqrt else w[r]) for every row r = index along dim 0 (new tensor)."""
     lib = _hip.load()

@@ -41,8 +41,8 @@ class _DiagCovBatchNorm(DiagCurvature):
 
     def update_in_backward(self, grad_output):
         n = grad_output.shape[0]
-        sg = _ops.rowsq_sum(grad_output, self._module.num_features)
-        w, b = _ops.bn_diag_combine(self._sx, sg, float(n), self.bias)   # n^2 / n
+        w, b = _ops.bn_diag_cov(grad_output, self._module.num_features, self._sx, float(n),
+                                self.bias)                                # n^2 / n
         self._data = [w] if b is None else [w, b]
 
 

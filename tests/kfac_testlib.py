@@ -262,6 +262,9 @@ class OracleOps(object):
         b = alpha * sg.sum(dim=0) if bias else None
         return w, b
 
+    def bn_diag_cov(self, grad_output, channels, sx, alpha, bias):
+        return self.bn_diag_combine(sx, self.rowsq_sum(grad_output, channels), alpha, bias)
+
 
 def _oracle_sqrt_batched(self, xs, ys):
     for x, y in zip(xs, ys):

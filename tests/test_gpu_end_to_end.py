@@ -268,25 +268,32 @@ def test_bottleneck_residual_network_with_batchnorm():
     worst = _config_parity(SmallResNet, x, y, 2, shapes)
     print('bottleneck net worst rel. Frobenius errors:', {k: '%.2e' % v for k, v in worst.items()})
     dev = torch.device('cuda:0')
+    # torch's default convolution backward is not run-to-run deterministic, and a ReLU that
+    # flips under a 1e-7 perturbation changes the next gradient by far more than that:
+    # compare runs under deterministic convolution algorithms
     runs = []
-    for cls in (SmallResNet, SmallResNetInplace, SmallResNetInplace):
-        torch.manual_seed(1)
-        model = cls().to(dev)
-        opt = torchsso.optim.SecondOrderOptimizer(
-            model, 'Cov', shapes, {'damping': 1e-3, 'ema_decay': 0.95}, lr=0.01, momentum=0.9)
-        opt.step(closure=_closure(model, x.to(dev), y.to(dev)))
-        factors = [d.clone() for g in opt.param_groups for d in g['curv'].data]
-        opt.step(closure=_closure(model, x.to(dev), y.to(dev)))
-        runs.append((factors, [p.detach().clone() for p in model.parameters()]))
-    # the factors of the first step see the same parameters in every run: they may differ
-    # by the rounding of torch's own (not run-to-run deterministic) backward kernels only
+    det = torch.backends.cudnn.deterministic
+    torch.backends.cudnn.deterministic = True
+    try:
+        for cls in (SmallResNet, SmallResNetInplace, SmallResNetInplace):
+            torch.manual_seed(1)
+            model = cls().to(dev)
+            opt = torchsso.optim.SecondOrderOptimizer(
+                model, 'Cov', shapes, {'damping': 1e-3, 'ema_decay': 0.95}, lr=0.01, momentum=0.9)
+            opt.step(closure=_closure(model, x.to(dev), y.to(dev)))
+            factors = [d.clone() for g in opt.param_groups for d in g['curv'].data]
+            opt.step(closure=_closure(model, x.to(dev), y.to(dev)))
+            runs.append((factors, [p.detach().clone() for p in model.parameters()]))
+    finally:
+        torch.backends.cudnn.deterministic = det
     f_err = max(O.rel_fro(a, b) for a, b in zip(runs[0][0], runs[1][0]))
     p_err = max(O.rel_fro(a, b) for a, b in zip(runs[0][1], runs[1][1]))
     p_noise = max(O.rel_fro(a, b) for a, b in zip(runs[1][1], runs[2][1]))
     print('in-place against out-of-place activations: factors %.2e, parameters after 2 steps '
           '%.2e (two identical runs: %.2e)' % (f_err, p_err, p_noise))
     assert f_err < 1e-5
-    assert p_err < 1e-3
+    assert p_err < 1e-4
+    assert p_noise < 1e-4      # the kernels of this library are deterministic
 
 
 def test_config5_noisy_kfac_step_runs_and_samples():

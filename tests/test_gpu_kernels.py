@@ -286,19 +286,32 @@ def test_elementwise_tails(ops, dev):
     assert O.rel_fro(dgr[0], g.double() * inv[0].cpu().double()) < 1e-6
 
 
-@pytest.mark.parametrize('shape', [(6, 10, 5, 5), (4, 3, 1, 1), (32, 64, 56, 56), (16, 7)])
-def test_batchnorm_diag(ops, dev, shape):
+# row lengths: 1 (BatchNorm1d), up to 64 / 128 / 256 loads per row with and without
+# float4 alignment, the ResNet-50 shapes 7x7, 14x14 and 28x28, a ragged channel count,
+# and rows beyond 1024 elements (general kernels)
+@pytest.mark.parametrize('shape', [(6, 10, 5, 5), (4, 3, 1, 1), (32, 64, 56, 56), (16, 7),
+                                   (32, 96, 7, 7), (32, 130, 14, 14), (8, 70, 28, 28),
+                                   (5, 33, 10, 13), (3, 300, 9, 9), (7, 18, 16, 20),
+                                   (2, 9, 33, 33), (40, 6, 2, 2)])
+@pytest.mark.parametrize('bias', [True, False])
+def test_batchnorm_diag(ops, dev, shape, bias):
     torch.manual_seed(5)
     c = shape[1]
     out = torch.randn(*shape)
     w = torch.rand(c) + 0.5
     b = torch.randn(c)
     g = torch.randn(*shape) * 1e-2
-    ref = O.bn_diag(O.bn_restore_input(out.double(), w.double(), b.double()), g, True, D)
+    ref = O.bn_diag(O.bn_restore_input(out.double(), w.double(), b.double()), g, bias, D)
     sx = ops.rowsq_sum(out.to(dev), c, w.to(dev), b.to(dev))
+    xhat = O.bn_restore_input(out.double(), w.double(), b.double())
+    assert O.rel_fro(sx, (xhat * xhat).reshape(shape[0], c, -1).sum(2)) < TOL
     sg = ops.rowsq_sum(g.to(dev), c)
-    wc, bc = ops.bn_diag_combine(sx, sg, float(shape[0]), True)
-    assert O.rel_fro(wc, ref[0]) < TOL and O.rel_fro(bc, ref[1]) < TOL
+    wc, bc = ops.bn_diag_combine(sx, sg, float(shape[0]), bias)
+    assert O.rel_fro(wc, ref[0]) < TOL and (not bias or O.rel_fro(bc, ref[1]) < TOL)
+    # the backward half in one call
+    wf, bf = ops.bn_diag_cov(g.to(dev), c, sx, float(shape[0]), bias)
+    assert O.rel_fro(wf, ref[0]) < TOL and (not bias or O.rel_fro(bf, ref[1]) < TOL)
+    assert (bf is None) == (not bias)
 
 
 # ---- size-independent properties at the benchmark's sizes ---------------------
