@@ -166,6 +166,71 @@ __global__ __launch_bounds__(256) void syrk_reduce_kernel(const float* ws, int d
   }
 }
 
+// The same reduction for few splits and many tiles: one workgroup owns 32 rows x 64
+// columns of a tile, a thread two float4 groups, and walks the splits with four
+// loads in flight.  The mirrored block goes through LDS, so that it is written in
+// runs of 32 elements as well.
+template <int TS>
+__global__ __launch_bounds__(256) void syrk_reduce_tile_kernel(const float* ws, int d, int T,
+                                                                int ntiles, int splits, float* C,
+                                                                const float* Cin, float alpha,
+                                                                float beta) {
+  __shared__ float mir[32][65];
+  const int tile = blockIdx.x;
+  int bi, bj;
+  upper_tile(tile, T, bi, bj);
+  const int r0 = blockIdx.y * 32, c0 = blockIdx.z * 64;      // inside the tile
+  if (bi * TS + r0 >= d || bj * TS + c0 >= d) return;
+  const int g = threadIdx.x & 15, rr = threadIdx.x >> 4;
+  const size_t stride = (size_t)ntiles * (TS * TS);
+  const float* base = ws + (size_t)tile * (TS * TS) + (size_t)(r0 + rr) * TS + c0 + 4 * g;
+  float4 acc[2] = {make_float4(0.f, 0.f, 0.f, 0.f), make_float4(0.f, 0.f, 0.f, 0.f)};
+#pragma unroll 2
+  for (int sp = 0; sp < splits; ++sp) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const float4 v = *reinterpret_cast<const float4*>(base + (size_t)sp * stride + h * 16 * TS);
+      acc[h].x += v.x;
+      acc[h].y += v.y;
+      acc[h].z += v.z;
+      acc[h].w += v.w;
+    }
+  }
+  const float* prev = Cin ? Cin : C;
+  float o[2][4];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const float vals[4] = {acc[h].x, acc[h].y, acc[h].z, acc[h].w};
+    const int row = bi * TS + r0 + rr + 16 * h;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int col = bj * TS + c0 + 4 * g + k;
+      const bool in = row < d && col < d;
+      o[h][k] = alpha * vals[k] + ((beta != 0.f && in) ? beta * prev[(size_t)row * d + col] : 0.f);
+    }
+  }
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int row = bi * TS + r0 + rr + 16 * h;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int col = bj * TS + c0 + 4 * g + k;
+      if (row < d && col < d) C[(size_t)row * d + col] = o[h][k];
+      mir[rr + 16 * h][4 * g + k] = o[h][k];
+    }
+  }
+  if (bi == bj) return;
+  __syncthreads();
+  // element (c, r) of the mirrored block: 8 of its rows per pass, 32 elements each
+  const int mr = threadIdx.x & 31;
+#pragma unroll
+  for (int pass = 0; pass < 8; ++pass) {
+    const int mc = (threadIdx.x >> 5) + 8 * pass;
+    const int row = bi * TS + r0 + mr, col = bj * TS + c0 + mc;
+    if (row < d && col < d) C[(size_t)col * d + row] = mir[mr][mc];
+  }
+}
+
 template <class OP, int W>
 static void launch_syrk_cfg(const OP& op, const SyrkPlan& p, int d, int64_t K, float alpha,
                             float beta, const float* Cin, float* C, void* workspace,
@@ -176,10 +241,14 @@ static void launch_syrk_cfg(const OP& op, const SyrkPlan& p, int d, int64_t K, f
   hipLaunchKernelGGL((syrk_kernel<OP, W>), dim3(p.ntiles, p.splits), dim3(64 * W * W), lds_bytes,
                      stream, op, d, (int)K, p.T, p.ntiles, p.splits, p.cps, C, Cin, alpha, beta,
                      (float*)workspace);
-  if (p.splits > 1) {
+  if (p.splits > 16) {
     hipLaunchKernelGGL((syrk_reduce_kernel<TS>), dim3(p.ntiles, TS * (TS / 64)), dim3(256), 0,
                        stream, (const float*)workspace, d, p.T, p.ntiles, p.splits, C, Cin, alpha,
                        beta);
+  } else if (p.splits > 1) {
+    hipLaunchKernelGGL((syrk_reduce_tile_kernel<TS>), dim3(p.ntiles, TS / 32, TS / 64), dim3(256),
+                       0, stream, (const float*)workspace, d, p.T, p.ntiles, p.splits, C, Cin,
+                       alpha, beta);
   }
 }
 
