@@ -123,7 +123,8 @@ constexpr int DIAG_SMEM_BYTES = (2 * DB * DLD + 64 * WLD) * (int)sizeof(float);
 // are software-pipelined: step c first finishes element c+1 of the column, publishes
 // it (two buffers alternate) and issues the reads of row c+1, and only then applies
 // row c to the rest of the column, so the LDS round trip of the next row runs under
-// those FMAs; the pivot itself comes through v_readlane and does not wait for LDS.
+// those FMAs (scheduling barriers keep the compiler from moving them in front of the
+// store); the pivot itself comes through v_readlane and does not wait for LDS.
 // The panel columns see the same eliminations as the leaf columns, so the strip ends
 // up holding U[q][*] without a triangular solve.  Several waves may run this on the
 // same leaf with different panel blocks (the leaf is then factored redundantly; only
@@ -161,27 +162,39 @@ __device__ __forceinline__ void chol_strip_32(lds_f* S, lds_f* rowbuf, lds_f* ub
   rowbuf[lane] = a[0];
   __builtin_amdgcn_wave_barrier();
   read_row(rowbuf, 0, row);
+  float piv = lane_value(a[0], 0);
+  // 1/sqrt in one instruction: the next step's pivot waits on this chain
+  float rd = __builtin_amdgcn_rsqf(piv);
+  float f = a[0] * (rd * rd);
 #pragma unroll
   for (int c = 0; c < 32; ++c) {
-    const float piv = lane_value(a[c], c);
     if (!(piv > 0.f) && bad == 0) bad = row_base + c0 + c + 1;
-    // 1/sqrt in one instruction: the next step's pivot waits on this chain
-    const float rd = __builtin_amdgcn_rsqf(piv);
-    const float f = a[c] * (rd * rd);
     float next[32];
+    float pivn = 0.f, rdn = 0.f, fn = 0.f;
     if (c + 1 < 32) {
+      // the chain from step to step: element c+1, its store, the reads of row c+1
       a[c + 1] = fmaf(-row[c + 1], f, a[c + 1]);
       lds_f* const nb = rowbuf + 64 * ((c + 1) & 1);
       nb[lane] = a[c + 1];
       __builtin_amdgcn_wave_barrier();
       read_row(nb, c + 1, next);
+      // nothing may be scheduled in front of that store: the rest of this step is
+      // what runs while the row travels through LDS
+      __builtin_amdgcn_sched_barrier(0);
+      pivn = lane_value(a[c + 1], c + 1);
+      rdn = __builtin_amdgcn_rsqf(pivn);
+      fn = a[c + 1] * (rdn * rdn);
     }
 #pragma unroll
     for (int i = c + 2; i < 32; ++i) a[i] = fmaf(-row[i], f, a[i]);   // A[i][col] -= U[c][i] U[c][col]
     const float u = a[c] * rd;
     a[c] = leaf ? (j > c ? u : (j == c ? piv * rd : 0.f)) : u;
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = c + 1; i < 32; ++i) row[i] = next[i];
+    piv = pivn;
+    rd = rdn;
+    f = fn;
   }
   if (owner && bad != 0 && lane == 0) {
     if (*info == 0) *info = bad;
@@ -233,7 +246,7 @@ __device__ __forceinline__ void backsub_32(const lds_f* ubuf, lds_f* Yb, int c0)
 }
 
 // One wave: acc(32x32) = sum_{k<K} A(k, i) * B(k, j) with operands in LDS,
-//   A(k, i) = a[k*a_ks + i*a_is],  B(k, j) = b[k*b_ks + j*b_js]   (K even).
+//   A(k, i) = a[k*a_ks + i*a_is],  B(k, j) = b[k*b_ks + j*b_js]   (K a multiple of 32).
 // Result element t of lane (r, h): row 8*(t/4) + 4h + t%4, column r.
 __device__ __forceinline__ v16f lds_mma32(const lds_f* a, int a_ks, int a_is, const lds_f* b,
                                           int b_ks, int b_js, int K) {
@@ -244,9 +257,17 @@ __device__ __forceinline__ v16f lds_mma32(const lds_f* a, int a_ks, int a_is, co
   for (int t = 0; t < 16; ++t) acc[t] = 0.f;
   const lds_f* pa = a + h * a_ks + r * a_is;
   const lds_f* pb = b + h * b_ks + r * b_js;
-#pragma unroll 4
-  for (int k = 0; k < K; k += 2) {
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[k * a_ks], pb[k * b_ks], acc, 0, 0, 0);
+  // 32 deep at a time: the 32 operand reads are issued together, ahead of the 16 MFMAs
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    float av[16], bv[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      av[i] = pa[(k0 + 2 * i) * a_ks];
+      bv[i] = pb[(k0 + 2 * i) * b_ks];
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[i], acc, 0, 0, 0);
   }
   return acc;
 }
@@ -306,6 +327,9 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
   // load the upper triangle; pad with the identity up to 128.  32 loads are
   // issued before the first is used, so the block costs 2 memory round trips
   // instead of 64.
+  // (raw buffer loads: no 64-bit address per element, and the elements outside the
+  // triangle cost no memory access)
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(m.U + (size_t)r0 * n + r0);
   for (int e0 = 0; e0 < DB * DB; e0 += 256 * 32) {
     float v[32];
 #pragma unroll
@@ -313,7 +337,7 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
       const int e = e0 + u * 256 + t;
       const int i = e >> 7, j = e & 127;
       const bool in = i < nb && j < nb && j >= i;
-      v[u] = m.U[in ? (size_t)(r0 + i) * n + r0 + j : (size_t)r0 * n + r0];
+      v[u] = buffer_load(rs, in ? (unsigned)(i * n + j) * 4u : INV_M);
     }
 #pragma unroll
     for (int u = 0; u < 32; ++u) {
@@ -382,6 +406,9 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
   if (nq > 2) tri_pair(S, Yb, Wt, 0, 64, 0, 4);
 
   // write U_pp and Y_pp back, 16 LDS reads in flight per thread
+  typedef __attribute__((address_space(1))) float global_f;
+  global_f* const gU = (global_f*)(m.U + (size_t)r0 * n + r0);
+  global_f* const gY = (global_f*)(m.Y + (size_t)r0 * n + r0);
   for (int e0 = 0; e0 < DB * DB; e0 += 256 * 16) {
     float u[16], y[16];
 #pragma unroll
@@ -396,8 +423,8 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
       const int e = e0 + k * 256 + t;
       const int i = e >> 7, j = e & 127;
       if (i < nb && j < nb) {
-        m.U[(size_t)(r0 + i) * n + r0 + j] = u[k];
-        m.Y[(size_t)(r0 + i) * n + r0 + j] = y[k];
+        gU[i * n + j] = u[k];
+        gY[i * n + j] = y[k];
       }
     }
   }
