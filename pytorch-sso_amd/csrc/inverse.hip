@@ -447,6 +447,28 @@ __global__ __launch_bounds__(NTHREADS) void potrf_panel_kernel(const MatDesc* ta
   gemm_tile(P, Q, 0, bj * BN, 0, DB, false, epi, smem);
 }
 
+// Tile (bi <= bj) number `local` of the trailing update of block rows [row_lo, row_hi).
+__device__ __forceinline__ bool trail_tile(int T, int row_lo, int row_hi, int local, int& bi,
+                                           int& bj) {
+  const int hi = min(row_hi, T);
+  if (row_lo >= hi) return false;
+  if (row_hi >= T) {
+    // all remaining rows: walk the upper triangle of the (T - row_lo)^2 block grid
+    const int Tr = T - row_lo;
+    if (local >= Tr * (Tr + 1) / 2) return false;
+    upper_tile(xcd_remap(local, Tr * (Tr + 1) / 2), Tr, bi, bj);
+    bi += row_lo;
+    bj += row_lo;
+    return true;
+  }
+  // a few rows: rectangular walk, tiles left of the diagonal exit
+  const int width = T - row_lo;
+  const int rr = local / width;
+  bi = row_lo + rr;
+  bj = row_lo + (local - rr * width);
+  return bi < hi && bj >= bi;
+}
+
 // trailing update with the block rows [kb0, kb0 + nk) of U:
 //   A[i, j] -= sum_k U[k, i]^T U[k, j]   for block rows row_lo <= i < row_hi, j >= i.
 // The Cholesky runs in outer panels of OUTER_BLOCKS diagonal blocks: inside an
@@ -462,29 +484,86 @@ __global__ __launch_bounds__(NTHREADS, 3) void potrf_trail_kernel(const MatDesc*
   int mat, local;
   work_find(wl, mat, local);
   const MatDesc m = table[mat];
-  const int T = m.T;
-  const int hi = min(row_hi, T);
-  if (row_lo >= hi) return;
   int bi, bj;
-  if (row_hi >= T) {
-    // all remaining rows: walk the upper triangle of the (T - row_lo)^2 block grid
-    const int Tr = T - row_lo;
-    if (local >= Tr * (Tr + 1) / 2) return;
-    upper_tile(xcd_remap(local, Tr * (Tr + 1) / 2), Tr, bi, bj);
-    bi += row_lo;
-    bj += row_lo;
-  } else {
-    // a few rows: rectangular walk, tiles left of the diagonal exit
-    const int width = T - row_lo;
-    const int rr = local / width;
-    bi = row_lo + rr;
-    bj = row_lo + (local - rr * width);
-    if (bi >= hi || bj < bi) return;
-  }
+  if (!trail_tile(m.T, row_lo, row_hi, local, bi, bj)) return;
   const int n = m.n;
   DenseKM P{m.U + (size_t)kb0 * DB * n, nullptr, n, n, 0};
   EpiStore epi{m.U, n, n, n, -1.f, 1.f, false};
   gemm_tile(P, P, bi * BM, bj * BN, 0, nk * DB, bi == bj, epi, smem);
+}
+
+// The row panel (near == 0) or the near update with one block row (near == 1) for
+// launches of few tiles: the same 128x128x128 product, but by 16 waves with one
+// 32x32 block each instead of 4 waves with four.  A tile is a chain of dependent-issue
+// MFMAs, 256 per wave (7.8 us) in the tile engine and 64 here, and at the end of a
+// factorisation nothing else runs beside it.  Both operands are fetched whole (32
+// loads per thread in flight, and the old values of C with them) into 128 KB of LDS.
+constexpr int FINE_THREADS = 1024;
+constexpr int FINE_SMEM_BYTES = 2 * DB * DB * (int)sizeof(float);
+constexpr int FINE_MAX_TILES = 256;      // one workgroup per CU
+
+__global__ __launch_bounds__(FINE_THREADS) void potrf_fine_kernel(const MatDesc* table, int p,
+                                                                  int near, int row_hi,
+                                                                  const WorkList wl) {
+  extern __shared__ __attribute__((aligned(16))) float fsm[];
+  lds_f* const tp = (lds_f*)fsm;
+  lds_f* const tq = tp + DB * DB;
+  int mat, local;
+  work_find(wl, mat, local);
+  const MatDesc m = table[mat];
+  const int n = m.n;
+  int bi, bj;
+  if (near) {
+    if (!trail_tile(m.T, p + 1, row_hi, local, bi, bj)) return;
+  } else {
+    bi = p;
+    bj = p + 1 + local;
+    if (bj >= m.T) return;
+  }
+  const float* kbase = m.U + (size_t)p * DB * n;            // block row p of U
+  // P(k, i), i < pw;  Q(k, j), j < qw;  C[i][j]
+  const float* P = near ? kbase + bi * DB : m.Y + (size_t)p * DB * n + p * DB;
+  const float* Q = kbase + bj * DB;
+  float* C = m.U + (size_t)bi * DB * n + bj * DB;
+  const int pw = near ? min(DB, n - bi * DB) : DB;
+  const int qw = min(DB, n - bj * DB);
+  const bool same = near && bi == bj;
+  const int t = threadIdx.x;
+  const int wave = t >> 6, lane = t & 63;
+  const int r = lane & 31, h = lane >> 5;
+  const int wr = wave >> 2, wc = wave & 3;
+
+  {
+    const int mm = t & (DB - 1), kq = t >> 7;
+    const __amdgpu_buffer_rsrc_t rp = make_rsrc(P), rq = make_rsrc(Q);
+    float vp[16], vq[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const unsigned off = (unsigned)((kq + 8 * i) * n + mm) * 4u;
+      vp[i] = buffer_load(rp, mm < pw ? off : INV_M);
+      vq[i] = same ? 0.f : buffer_load(rq, mm < qw ? off : INV_M);
+    }
+    float old[16];
+    if (near) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = 32 * wr + 8 * (e >> 2) + 4 * h + (e & 3), col = 32 * wc + r;
+        old[e] = (row < pw && col < qw) ? C[(size_t)row * n + col] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      tp[(kq + 8 * i) * DB + mm] = vp[i];
+      if (!same) tq[(kq + 8 * i) * DB + mm] = vq[i];
+    }
+    __syncthreads();
+    const v16f acc = lds_mma32(tp + 32 * wr, DB, 1, (same ? tp : tq) + 32 * wc, DB, 1, DB);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int row = 32 * wr + 8 * (e >> 2) + 4 * h + (e & 3), col = 32 * wc + r;
+      if (row < pw && col < qw) C[(size_t)row * n + col] = near ? old[e] - acc[e] : acc[e];
+    }
+  }
 }
 
 // ---- Y = U^-1 by balanced recursive halving over the 128-blocks ---------------
@@ -628,6 +707,10 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
                           hipFuncAttributeMaxDynamicSharedMemorySize,
                           DIAG_SMEM_BYTES) != hipSuccess)
     return KFAC_ERR_LAUNCH;
+  if (hipFuncSetAttribute((const void*)potrf_fine_kernel,
+                          hipFuncAttributeMaxDynamicSharedMemorySize,
+                          FINE_SMEM_BYTES) != hipSuccess)
+    return KFAC_ERR_LAUNCH;
 
   // descending size order; remember where each caller index went
   std::vector<int> order(nmat);
@@ -703,15 +786,23 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
       const int nb = active(p + 2);
       if (nb == 0) continue;
       for_worklists(nb, [&](int T) { return T - p - 1; }, [&](const WorkList& wl, int grid) {
-        KFAC_LAUNCH_TILE2(potrf_panel_kernel, dim3(grid), stream, table, p, wl);
+        if (grid <= FINE_MAX_TILES)
+          hipLaunchKernelGGL(potrf_fine_kernel, dim3(grid), dim3(FINE_THREADS), FINE_SMEM_BYTES,
+                             stream, table, p, 0, 0, wl);
+        else
+          KFAC_LAUNCH_TILE2(potrf_panel_kernel, dim3(grid), stream, table, p, wl);
       });
       if (p + 1 < Pend) {
         // rows (p, Pend) of the outer panel, all columns to the right
         for_worklists(nb,
                       [&](int T) { return (std::min(Pend, T) - p - 1) * (T - p - 1); },
                       [&](const WorkList& wl, int grid) {
-                        KFAC_LAUNCH_TILE2(potrf_trail_kernel, dim3(grid), stream, table, p, 1,
-                                          p + 1, Pend, wl);
+                        if (grid <= FINE_MAX_TILES)
+                          hipLaunchKernelGGL(potrf_fine_kernel, dim3(grid), dim3(FINE_THREADS),
+                                             FINE_SMEM_BYTES, stream, table, p, 1, Pend, wl);
+                        else
+                          KFAC_LAUNCH_TILE2(potrf_trail_kernel, dim3(grid), stream, table, p, 1,
+                                            p + 1, Pend, wl);
                       });
       }
     }
