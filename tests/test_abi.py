@@ -60,5 +60,8 @@ def test_argument_errors_are_codes_not_crashes():
     assert lib.kfac_factor_linear(None, 8, 4, 4, 1, 1.0, 0.0, None, None, None, 0, None) == 1
     assert lib.kfac_factor_conv_g(None, 1, 1, 1, 1, 1.0, 0.0, None, None, None, 0, None) == 1
     assert lib.kfac_rowsq_sum(None, 1, 1, 1, None, None, None, None) == 1
+    assert lib.kfac_bn_diag_cov(None, 1, 1, 1, None, 1.0, None, None, None, 0, None) == 1
+    assert lib.kfac_bn_diag_cov_workspace_bytes(32, 64) == 32 * 64 * 4
+    assert lib.kfac_bn_diag_cov_workspace_bytes(0, 64) == 0
     with pytest.raises(_hip.KfacHipError):
         _hip.check(2, 'x')
