@@ -121,8 +121,11 @@ def test_factor_conv_a_by_correlations(ops, dev, shape, k, p, d):
     assert O.rel_fro(nxt, 0.9 * ref + 0.1 * old.double()) < TOL and torch.equal(prev.cpu(), old)
 
 
+# the last three: few k-splits over many tiles (tile-wise reduction, mirrored blocks
+# through LDS), with a ragged last tile in one of them
 @pytest.mark.parametrize('shape', [(1, 1, 1, 1), (2, 3, 4, 4), (8, 64, 7, 7), (4, 130, 14, 14),
-                                   (16, 64, 56, 56), (3, 257, 5, 3)])
+                                   (16, 64, 56, 56), (3, 257, 5, 3), (32, 1024, 14, 14),
+                                   (32, 2048, 7, 7), (8, 1500, 10, 10)])
 def test_factor_conv_g(ops, dev, shape):
     torch.manual_seed(sum(shape))
     g = torch.randn(*shape) * 1e-2
