@@ -291,11 +291,11 @@ def test_elementwise_tails(ops, dev):
 
 # row lengths: 1 (BatchNorm1d), up to 64 / 128 / 256 loads per row with and without
 # float4 alignment, the ResNet-50 shapes 7x7, 14x14 and 28x28, a ragged channel count,
-# and rows beyond 1024 elements (general kernels)
+# rows beyond 1024 elements and a batch beyond 2048 samples (general kernels)
 @pytest.mark.parametrize('shape', [(6, 10, 5, 5), (4, 3, 1, 1), (32, 64, 56, 56), (16, 7),
                                    (32, 96, 7, 7), (32, 130, 14, 14), (8, 70, 28, 28),
                                    (5, 33, 10, 13), (3, 300, 9, 9), (7, 18, 16, 20),
-                                   (2, 9, 33, 33), (40, 6, 2, 2)])
+                                   (2, 9, 33, 33), (40, 6, 2, 2), (2100, 3, 2, 2)])
 @pytest.mark.parametrize('bias', [True, False])
 def test_batchnorm_diag(ops, dev, shape, bias):
     torch.manual_seed(5)
