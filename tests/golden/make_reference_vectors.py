@@ -10,8 +10,9 @@ the GPU box):
 What it pins (behaviour that is convention rather than mathematics, so that a
 restatement could silently disagree): the order of operations inside
 SecondOrderOptimizer.step when l2_reg, damping, momentum and weight decay
-interact; what the hooks take as layer input / output gradient on current
-torch; the accumulation scales of VIOptimizer's MC loop.  The numerical kernels
+interact (momentum type, gradient EMA, bias correction, LARS, weight normalisation,
+accumulation over micro-steps, running max); what the hooks take as layer input /
+output gradient on current torch; the accumulation scales of VIOptimizer's MC loop.  The numerical kernels
 themselves are pinned by mathematics in tests/test_oracle.py.
 
 The reference imports `chainer` at module level for its multi-GPU communicator
@@ -74,6 +75,8 @@ def snapshot(optimizer, out, tag):
             out['%s.g%d.grad%d' % (tag, gi, pi)] = p.grad.detach().numpy().copy()
         for name in ('ema', 'inv'):
             val = getattr(curv, name)
+            if val is None:          # a micro-step of an accumulation: nothing updated yet
+                continue
             for k, t in enumerate(val):
                 out['%s.g%d.%s%d' % (tag, gi, name, k)] = t.detach().numpy().copy()
         out['%s.g%d.damping' % (tag, gi)] = np.float64(curv.damping)
@@ -160,6 +163,34 @@ def main():
              torchsso.optim.VOGN,
              dict(dataset_size=60, lr=0.01, num_mc_samples=2, warmup_kl_weighting_steps=None,
                   prior_variance=0, curv_kwargs={'ema_decay': 0.1, 'damping': 1e-3}), steps=3)
+
+    # 6. the tails of the update: gradient EMA on the preconditioned gradient, bias
+    #    correction, LARS, weight normalisation, no regularisation for BatchNorm, running
+    #    max of the curvature (orders of operations that no formula fixes)
+    torch.manual_seed(0)
+    x = torch.randn(6, 2, 8, 8)
+    y = torch.randint(0, 5, (6,))
+    run_case(torchsso, torch, nn, F, 'ref_convnet_kfac_tails', build_convnet(torch, nn), x, y,
+             torchsso.optim.SecondOrderOptimizer,
+             dict(curv_type='Cov',
+                  curv_shapes={'Linear': 'Kron', 'Conv2d': 'Kron', 'BatchNorm2d': 'Diag'},
+                  curv_kwargs={'damping': 1e-2, 'ema_decay': 0.9, 'use_max_ema': True},
+                  lr=0.02, momentum=0.5, grad_ema_decay=0.8, grad_ema_type='preconditioned',
+                  l2_reg=1e-4, weight_decay=1e-3, bias_correction=True, lars=True,
+                  normalizing_weights=True, non_reg_for_bn=True), steps=3)
+
+    # 7. accumulation over 2 micro-steps, raw momentum, LARS on the raw gradient, a
+    #    fixed weight scale; 6 calls = 3 updates
+    torch.manual_seed(0)
+    x = torch.randn(8, 12)
+    y = torch.randint(0, 5, (8,))
+    run_case(torchsso, torch, nn, F, 'ref_mlp_kfac_accumulate', build_mlp(torch, nn), x, y,
+             torchsso.optim.SecondOrderOptimizer,
+             dict(curv_type='Cov', curv_shapes={'Linear': 'Kron'},
+                  curv_kwargs={'damping': 1e-3, 'ema_decay': 0.95},
+                  lr=0.05, momentum=0.9, momentum_type='raw', l2_reg=1e-3, acc_steps=2,
+                  lars=True, lars_type='raw', normalizing_weights=True, weight_scale=1.5),
+             steps=6)
 
 
 if __name__ == '__main__':

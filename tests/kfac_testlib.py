@@ -149,8 +149,8 @@ def snapshot_optimizer(optimizer, target='params'):
         curv = group['curv']
         snap.append({'params': [p.detach().cpu().clone() for p in group['params']],
                      'grads': [p.grad.detach().cpu().clone() for p in group['params']],
-                     'ema': [e.detach().cpu().clone() for e in curv.ema],
-                     'inv': [i.detach().cpu().clone() for i in curv.inv]})
+                     'ema': [e.detach().cpu().clone() for e in (curv.ema or [])],
+                     'inv': [i.detach().cpu().clone() for i in (curv.inv or [])]})
     return snap
 
 

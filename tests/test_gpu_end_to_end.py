@@ -73,6 +73,29 @@ def test_reference_golden_vogn_diagonal_curvature():
                 skip={(0, 'grad', 1)})
 
 
+def test_reference_golden_update_tails():
+    # gradient EMA on the preconditioned gradient, bias correction, LARS, weight
+    # normalisation, no regularisation for BatchNorm, running max of the curvature
+    _run_golden('ref_convnet_kfac_tails', T.build_convnet, 'SecondOrderOptimizer',
+                dict(curv_type='Cov',
+                     curv_shapes={'Linear': 'Kron', 'Conv2d': 'Kron', 'BatchNorm2d': 'Diag'},
+                     curv_kwargs={'damping': 1e-2, 'ema_decay': 0.9, 'use_max_ema': True},
+                     lr=0.02, momentum=0.5, grad_ema_decay=0.8, grad_ema_type='preconditioned',
+                     l2_reg=1e-4, weight_decay=1e-3, bias_correction=True, lars=True,
+                     normalizing_weights=True, non_reg_for_bn=True), 3,
+                # zero gradient of the conv bias in front of the BatchNorm: rounding noise,
+                # which LARS scales up to the norm of the bias
+                skip={(0, 'grad', 1), (0, 'param', 1)})
+
+
+def test_reference_golden_accumulation_raw_momentum_lars():
+    _run_golden('ref_mlp_kfac_accumulate', T.build_mlp, 'SecondOrderOptimizer',
+                dict(curv_type='Cov', curv_shapes={'Linear': 'Kron'},
+                     curv_kwargs={'damping': 1e-3, 'ema_decay': 0.95},
+                     lr=0.05, momentum=0.9, momentum_type='raw', l2_reg=1e-3, acc_steps=2,
+                     lars=True, lars_type='raw', normalizing_weights=True, weight_scale=1.5), 6)
+
+
 class MLP(nn.Module):
     """BASELINE config 1: 784-1000-1000-10."""
 

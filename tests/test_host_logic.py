@@ -68,6 +68,50 @@ def test_second_order_optimizer_matches_reference_convnet(oracle_ops):
     T.compare_with_golden(snaps, gold, 2e-4)
 
 
+TAILS_ARGS = dict(curv_type='Cov',
+                  curv_shapes={'Linear': 'Kron', 'Conv2d': 'Kron', 'BatchNorm2d': 'Diag'},
+                  curv_kwargs={'damping': 1e-2, 'ema_decay': 0.9, 'use_max_ema': True},
+                  lr=0.02, momentum=0.5, grad_ema_decay=0.8, grad_ema_type='preconditioned',
+                  l2_reg=1e-4, weight_decay=1e-3, bias_correction=True, lars=True,
+                  normalizing_weights=True, non_reg_for_bn=True)
+ACCUMULATE_ARGS = dict(curv_type='Cov', curv_shapes={'Linear': 'Kron'},
+                       curv_kwargs={'damping': 1e-3, 'ema_decay': 0.95},
+                       lr=0.05, momentum=0.9, momentum_type='raw', l2_reg=1e-3, acc_steps=2,
+                       lars=True, lars_type='raw', normalizing_weights=True, weight_scale=1.5)
+
+
+def test_update_tails_match_reference(oracle_ops):
+    """Gradient EMA on the preconditioned gradient, bias correction, LARS, weight
+    normalisation, no regularisation for BatchNorm, running max of the curvature."""
+    gold = T.load_golden('ref_convnet_kfac_tails')
+    model = T.load_init(T.build_convnet(), gold)
+    x, y = torch.from_numpy(gold['x']), torch.from_numpy(gold['y'])
+    opt = torchsso.optim.SecondOrderOptimizer(model, **TAILS_ARGS)
+    snaps = []
+    for s in range(3):
+        loss, _ = opt.step(closure=_closure(model, x, y))
+        assert abs(loss.item() - float(gold['step%d.loss' % s])) < 1e-4
+        snaps.append(T.snapshot_optimizer(opt))
+    # the conv bias in front of the BatchNorm has a zero gradient (rounding noise, which
+    # LARS then scales up to the norm of the bias)
+    T.compare_with_golden(snaps, gold, 2e-4, skip={(0, 'grad', 1), (0, 'param', 1)})
+
+
+def test_accumulation_with_raw_momentum_and_lars_matches_reference(oracle_ops):
+    """acc_steps = 2: the odd calls only accumulate, the even ones update."""
+    gold = T.load_golden('ref_mlp_kfac_accumulate')
+    model = T.load_init(T.build_mlp(), gold)
+    x, y = torch.from_numpy(gold['x']), torch.from_numpy(gold['y'])
+    opt = torchsso.optim.SecondOrderOptimizer(model, **ACCUMULATE_ARGS)
+    snaps = []
+    for s in range(6):
+        loss, _ = opt.step(closure=_closure(model, x, y))
+        assert abs(loss.item() - float(gold['step%d.loss' % s])) < 1e-4
+        snaps.append(T.snapshot_optimizer(opt))
+        assert opt.optim_state == {'step': (s + 1) // 2, 'acc_step': (s + 1) % 2}
+    T.compare_with_golden(snaps, gold, 2e-4)
+
+
 def test_vi_optimizer_accumulation_matches_reference(oracle_ops):
     gold = T.load_golden('ref_mlp_vi_nosample')
     model = T.load_init(T.build_mlp(), gold)
