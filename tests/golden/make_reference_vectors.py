@@ -192,6 +192,19 @@ def main():
                   lars=True, lars_type='raw', normalizing_weights=True, weight_scale=1.5),
              steps=6)
 
+    # 8. diagonal curvature everywhere with the square root of the running average, a
+    #    gradient EMA on the raw gradient and bias correction: the Adam-like setting
+    torch.manual_seed(0)
+    x = torch.randn(6, 2, 8, 8)
+    y = torch.randint(0, 5, (6,))
+    run_case(torchsso, torch, nn, F, 'ref_convnet_diag_sqrt', build_convnet(torch, nn), x, y,
+             torchsso.optim.SecondOrderOptimizer,
+             dict(curv_type='Cov',
+                  curv_shapes={'Linear': 'Diag', 'Conv2d': 'Diag', 'BatchNorm2d': 'Diag'},
+                  curv_kwargs={'damping': 1e-8, 'ema_decay': 0.001, 'use_sqrt_ema': True},
+                  lr=1e-3, grad_ema_decay=0.1, grad_ema_type='raw', bias_correction=True),
+             steps=4)
+
 
 if __name__ == '__main__':
     main()

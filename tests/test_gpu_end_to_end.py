@@ -96,6 +96,16 @@ def test_reference_golden_accumulation_raw_momentum_lars():
                      lars=True, lars_type='raw', normalizing_weights=True, weight_scale=1.5), 6)
 
 
+def test_reference_golden_diagonal_sqrt_bias_correction():
+    # the Adam-like setting: diagonal curvature with the square root of the running average
+    _run_golden('ref_convnet_diag_sqrt', T.build_convnet, 'SecondOrderOptimizer',
+                dict(curv_type='Cov',
+                     curv_shapes={'Linear': 'Diag', 'Conv2d': 'Diag', 'BatchNorm2d': 'Diag'},
+                     curv_kwargs={'damping': 1e-8, 'ema_decay': 0.001, 'use_sqrt_ema': True},
+                     lr=1e-3, grad_ema_decay=0.1, grad_ema_type='raw', bias_correction=True), 4,
+                skip={(0, k, 1) for k in ('grad', 'param', 'ema', 'inv')})
+
+
 class MLP(nn.Module):
     """BASELINE config 1: 784-1000-1000-10."""
 

@@ -112,6 +112,29 @@ def test_accumulation_with_raw_momentum_and_lars_matches_reference(oracle_ops):
     T.compare_with_golden(snaps, gold, 2e-4)
 
 
+DIAG_SQRT_ARGS = dict(curv_type='Cov',
+                      curv_shapes={'Linear': 'Diag', 'Conv2d': 'Diag', 'BatchNorm2d': 'Diag'},
+                      curv_kwargs={'damping': 1e-8, 'ema_decay': 0.001, 'use_sqrt_ema': True},
+                      lr=1e-3, grad_ema_decay=0.1, grad_ema_type='raw', bias_correction=True)
+
+
+def test_diagonal_sqrt_curvature_with_bias_correction_matches_reference(oracle_ops):
+    """The Adam-like setting: diagonal curvature, sqrt of the running average, gradient
+    EMA on the raw gradient, bias correction with the square root."""
+    gold = T.load_golden('ref_convnet_diag_sqrt')
+    model = T.load_init(T.build_convnet(), gold)
+    x, y = torch.from_numpy(gold['x']), torch.from_numpy(gold['y'])
+    opt = torchsso.optim.SecondOrderOptimizer(model, **DIAG_SQRT_ARGS)
+    snaps = []
+    for s in range(4):
+        loss, _ = opt.step(closure=_closure(model, x, y))
+        assert abs(loss.item() - float(gold['step%d.loss' % s])) < 1e-4
+        snaps.append(T.snapshot_optimizer(opt))
+    # the conv bias in front of the BatchNorm has a zero gradient: g / sqrt(g^2) of rounding noise
+    T.compare_with_golden(snaps, gold, 2e-4,
+                          skip={(0, k, 1) for k in ('grad', 'param', 'ema', 'inv')})
+
+
 def test_vi_optimizer_accumulation_matches_reference(oracle_ops):
     gold = T.load_golden('ref_mlp_vi_nosample')
     model = T.load_init(T.build_mlp(), gold)
