@@ -205,6 +205,41 @@ def main():
                   lr=1e-3, grad_ema_decay=0.1, grad_ema_type='raw', bias_correction=True),
              steps=4)
 
+    # 9. the iteration-based learning-rate schedules (host arithmetic only)
+    if len(sys.argv) == 1 or 'ref_lr_schedules' in sys.argv[1:]:
+        L = torchsso.optim.lr_scheduler
+        out = {}
+
+        def sgd(lr=0.4, momentum=0.9):
+            return torch.optim.SGD(nn.Linear(3, 2).parameters(), lr=lr, momentum=momentum)
+
+        def run(tag, opt, sched, steps):
+            lrs, moms = [], []
+            for _ in range(steps):
+                sched.step()
+                lrs.append(opt.param_groups[0]['lr'])
+                moms.append(opt.param_groups[0]['momentum'])
+            out[tag + '.lr'] = np.array(lrs, dtype=np.float64)
+            out[tag + '.momentum'] = np.array(moms, dtype=np.float64)
+
+        opt = sgd()
+        run('poly_start2', opt, L.PolynomialDecayIterLR(opt, rate=2, max_count=10, start_iter=2), 12)
+        opt = sgd()
+        run('poly_target', opt, L.PolynomialDecayIterLR(opt, rate=1, max_count=10, target=0.1), 10)
+        opt = sgd()
+        run('poly_negative_rate', opt,
+            L.PolynomialDecayIterLR(opt, rate=-0.5, max_count=10, target=0.8), 9)
+        opt = sgd()
+        run('warmup_momentum', opt,
+            L.MomentumCorrectionLR(L.GradualWarmupIterLR(opt, initial_lr=0.1, max_count=4)), 7)
+        opt = sgd()
+        opt.param_groups[0]['initial_lr'] = 0.4
+        run('poly_resumed', opt,
+            L.PolynomialDecayIterLR(opt, rate=2, max_count=10, last_iter=5), 4)
+        path = os.path.join(HERE, 'ref_lr_schedules.npz')
+        np.savez_compressed(path, **out)
+        print('wrote', path, os.path.getsize(path), 'bytes')
+
 
 if __name__ == '__main__':
     main()

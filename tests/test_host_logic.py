@@ -322,6 +322,38 @@ def test_iteration_lr_schedules():
         L.GradualWarmupIterLR(fresh, 0.0, 4, last_iter=3)
 
 
+def test_iteration_lr_schedules_match_reference():
+    """The same schedules, stepped by the reference itself (golden sequences)."""
+    from torchsso.optim import lr_scheduler as L
+    gold = T.load_golden('ref_lr_schedules')
+
+    def sgd():
+        return torch.optim.SGD(nn.Linear(3, 2).parameters(), lr=0.4, momentum=0.9)
+
+    def check(tag, opt, sched):
+        want_lr, want_m = gold[tag + '.lr'], gold[tag + '.momentum']
+        for k in range(len(want_lr)):
+            sched.step()
+            assert opt.param_groups[0]['lr'] == pytest.approx(want_lr[k], rel=1e-14, abs=1e-300), (tag, k)
+            assert opt.param_groups[0]['momentum'] == pytest.approx(want_m[k], rel=1e-14), (tag, k)
+
+    opt = sgd()
+    check('poly_start2', opt, L.PolynomialDecayIterLR(opt, rate=2, max_count=10, start_iter=2))
+    opt = sgd()
+    sched = L.PolynomialDecayIterLR(opt, rate=1, max_count=10, target=0.1)
+    check('poly_target', opt, sched)
+    with pytest.raises(ZeroDivisionError):      # the reference divides by the decayed rate
+        sched.step()
+    opt = sgd()
+    check('poly_negative_rate', opt, L.PolynomialDecayIterLR(opt, rate=-0.5, max_count=10, target=0.8))
+    opt = sgd()
+    check('warmup_momentum', opt,
+          L.MomentumCorrectionLR(L.GradualWarmupIterLR(opt, initial_lr=0.1, max_count=4)))
+    opt = sgd()
+    opt.param_groups[0]['initial_lr'] = 0.4
+    check('poly_resumed', opt, L.PolynomialDecayIterLR(opt, rate=2, max_count=10, last_iter=5))
+
+
 def test_running_average_written_by_the_factor_kernels(oracle_ops):
     """With acc_steps == 1 the hooks build beta*factor + (1-beta)*ema straight into
     a second buffer and update_ema swaps buffers.  Same numbers as the unfused
