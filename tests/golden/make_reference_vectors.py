@@ -205,6 +205,17 @@ def main():
                   lr=1e-3, grad_ema_decay=0.1, grad_ema_type='raw', bias_correction=True),
              steps=4)
 
+    # 10. VOGN with a KL warm-up, a prior variance other than 1 and an initial precision:
+    #     the l2 / std scale bookkeeping of VIOptimizer, with sampling from the first step
+    torch.manual_seed(0)
+    x = torch.randn(6, 2, 8, 8)
+    y = torch.randint(0, 5, (6,))
+    run_case(torchsso, torch, nn, F, 'ref_convnet_vogn_warmup', build_convnet(torch, nn), x, y,
+             torchsso.optim.VOGN,
+             dict(dataset_size=60, lr=0.01, num_mc_samples=2, warmup_kl_weighting_steps=3,
+                  warmup_kl_weighting_init=0.1, kl_weighting=0.5, prior_variance=2,
+                  init_precision=8e-3, curv_kwargs={'ema_decay': 0.1, 'damping': 1e-3}), steps=5)
+
     # 9. the iteration-based learning-rate schedules (host arithmetic only)
     if len(sys.argv) == 1 or 'ref_lr_schedules' in sys.argv[1:]:
         L = torchsso.optim.lr_scheduler

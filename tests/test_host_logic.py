@@ -174,6 +174,29 @@ def test_vogn_matches_reference_with_sampling(oracle_ops):
     T.compare_with_golden(snaps, gold, 2e-4)
 
 
+def test_vogn_kl_warmup_prior_and_initial_precision_match_reference(oracle_ops):
+    """KL warm-up over 3 steps, prior variance 2, initial precision: the l2_reg /
+    std_scale bookkeeping of VIOptimizer (optim/vi.py:77-78, 98-106, 141-162), with a
+    posterior to sample from before the first step."""
+    gold = T.load_golden('ref_convnet_vogn_warmup')
+    model = T.load_init(T.build_convnet(), gold)
+    x, y = torch.from_numpy(gold['x']), torch.from_numpy(gold['y'])
+    opt = torchsso.optim.VOGN(model, 60, lr=0.01, num_mc_samples=2, warmup_kl_weighting_steps=3,
+                              warmup_kl_weighting_init=0.1, kl_weighting=0.5, prior_variance=2,
+                              init_precision=8e-3,
+                              curv_kwargs={'ema_decay': 0.1, 'damping': 1e-3})
+    snaps = []
+    for s in range(5):
+        loss, _ = opt.step(closure=_closure(model, x, y))
+        assert abs(loss.item() - float(gold['step%d.loss' % s])) < 1e-3 * max(1, abs(loss.item()))
+        snaps.append(T.snapshot_optimizer(opt))
+        for gi, g in enumerate(opt.param_groups):
+            assert abs(g['curv'].damping - float(gold['step%d.g%d.damping' % (s, gi)])) < 1e-9
+    # the bias of the conv in front of the BatchNorm has a zero gradient (rounding noise
+    # over its tiny curvature); everything else, sampled parameters included, must agree
+    T.compare_with_golden(snaps, gold, 2e-4, skip={(0, 'grad', 1)})
+
+
 def test_vi_sampling_consumes_generator_in_group_order(oracle_ops):
     """With a std present, params = mean + std_scale * U_G E U_A with E drawn by
     torch.randn in param_group order after manual_seed(step + seed)."""
