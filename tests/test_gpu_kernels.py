@@ -351,6 +351,29 @@ def test_large_inverse_at_benchmark_sizes(ops, dev):
         del Xd, Y, R
 
 
+def test_precondition_at_benchmark_sizes_against_float64_on_device(ops, dev):
+    """G^-1 [dW | db] A^-1 for the largest layers of configs 3 and 4 (ResNet-50
+    layer4 3x3 conv: 512 x 4608, no bias; AlexNet fc6: 4096 x 9216 + bias) against
+    the same product in float64 on the device (torch.matmul, a library routine)."""
+    for dg, da, bias in [(512, 4608, False), (4096, 9217, True)]:
+        g = torch.Generator(device='cpu').manual_seed(dg + da)
+        Gi = torch.randn(dg, dg, generator=g).to(dev)
+        Gi = Gi @ Gi.t() / dg + torch.eye(dg, device=dev)
+        Ai = torch.randn(da, da // 4, generator=g).to(dev)
+        Ai = Ai @ Ai.t() / (da // 4) + torch.eye(da, device=dev)
+        W = torch.randn(dg, da - (1 if bias else 0), generator=g).to(dev)
+        b = torch.randn(dg, generator=g).to(dev) if bias else None
+        V = W.double() if b is None else torch.cat([W.double(), b.double()[:, None]], 1)
+        ref = Gi.double() @ V @ Ai.double()
+        gw, gb = W.clone(), None if b is None else b.clone()
+        ops.precondition_batched([Gi], [Ai], [gw], [gb])
+        got = gw.double() if gb is None else torch.cat([gw.double(), gb.double()[:, None]], 1)
+        err = ((got - ref).norm() / ref.norm()).item()
+        print('precondition %d x %d: rel err %.2e' % (dg, da, err))
+        assert err < TOL
+        del Gi, Ai, V, ref, got
+
+
 def test_factor_linearity_at_full_size(ops, dev):
     """factor(x stacked with y) = factor(x) + factor(y) (sums of outer products),
     on the ResNet-50 layer1 3x3 shape (c=64, 56x56, batch 32)."""
