@@ -351,6 +351,26 @@ def test_large_inverse_at_benchmark_sizes(ops, dev):
         del Xd, Y, R
 
 
+def test_cholesky_factor_at_benchmark_size(ops, dev):
+    """std = upper Cholesky factor of a 4608^2 inverse (posterior of the largest
+    ResNet-50 factor): U^T U reproduces the matrix (float64 product on the device), U is
+    upper triangular with a positive diagonal, and agrees with torch.linalg.cholesky in
+    float64 (a library routine)."""
+    n = 4608
+    g = torch.Generator(device='cpu').manual_seed(n)
+    x = torch.randn(1568, n, generator=g).to(dev)
+    X = ops.factor_linear(x, False, 1.0 / 1568)
+    X.diagonal().add_(0.05 * X.diagonal().mean().item())
+    outs, info = ops.cholesky_upper_batched([X])
+    assert info.cpu().tolist() == [0]
+    U = outs[0]
+    assert torch.equal(U, torch.triu(U)) and (U.diagonal() > 0).all()
+    Ud = U.double()
+    assert ((Ud.t() @ Ud - X.double()).norm() / X.double().norm()).item() < 1e-5
+    ref = torch.linalg.cholesky(X.double()).t()
+    assert ((Ud - ref).norm() / ref.norm()).item() < TOL
+
+
 def test_precondition_at_benchmark_sizes_against_float64_on_device(ops, dev):
     """G^-1 [dW | db] A^-1 for the largest layers of configs 3 and 4 (ResNet-50
     layer4 3x3 conv: 512 x 4608, no bias; AlexNet fc6: 4096 x 9216 + bias) against
