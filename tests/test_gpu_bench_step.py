@@ -1,0 +1,102 @@
+"""One step of bench.py's own workload (BASELINE config 3: the ResNet-50 layer set at
+batch 32) checked at full size: for a sample of layers, the largest included, the
+running average after the first step, the pi-damped inverses and the preconditioned
+gradient are recomputed in float64 on the device with library routines (unfold,
+matmul, torch.linalg.inv).  Nothing in the timed step is skipped or cached."""
+import os
+import sys
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+def rel(a, b):
+    return ((a.double() - b).norm() / b.norm()).item()
+
+
+def conv_a_float64(x, s):
+    """sum over the batch of unfold(x) unfold(x)^T / n, image by image."""
+    k = s['k']
+    d = s['cin'] * k * k
+    A = torch.zeros(d, d, dtype=torch.float64, device=x.device)
+    for i in range(x.shape[0]):
+        u = F.unfold(x[i:i + 1].double(), k, padding=s['pad'], stride=s['stride'])[0]
+        A += u @ u.t()
+    return A / x.shape[0]
+
+
+def test_resnet50_step_at_full_size_against_float64_on_device():
+    import bench
+    dev = torch.device('cuda:0')
+    specs, batch, _ = bench.WORKLOADS['resnet50']
+    specs = specs()
+    ls = bench.LayerSet(specs, batch, dev)
+    raw = ls.flat_raw.clone()
+    ls.step()
+    torch.cuda.synchronize()
+    names = [s['name'] for s in specs]
+    picked = ['conv1', 'layer1.0.conv1', 'layer1.0.conv2', 'layer2.0.conv2', 'layer3.0.downsample',
+              'layer4.0.conv2', 'layer4.2.conv2', 'layer4.2.conv3', 'fc', 'layer3.1.bn2']
+    offs = {}
+    total = 0
+    for m in ls.model:
+        for p in m.parameters():
+            offs[id(p)] = total
+            total += (p.numel() + 63) // 64 * 64
+    worst = {}
+    for name in picked:
+        i = names.index(name)
+        s, m, curv, x, g = specs[i], ls.model[i], ls.curvs[i], ls.inputs[i], ls.gouts[i]
+        n = x.shape[0]
+        if s['kind'] == 'bn':
+            xhat = (x.double() - m.bias.detach().double().view(1, -1, 1, 1)) / \
+                m.weight.detach().double().view(1, -1, 1, 1)
+            sx = (xhat * xhat).sum((2, 3))
+            sg = (g.double() ** 2).sum((2, 3))
+            want = [(sx * sg).mean(0) * n * n, sg.mean(0) * n * n]
+            for k in range(2):
+                worst['bn ema'] = max(worst.get('bn ema', 0.), rel(curv.ema[k], want[k]))
+                worst['bn inv'] = max(worst.get('bn inv', 0.),
+                                      rel(curv.inv[k], 1. / (curv.ema[k].double() + 1e-3)))
+            continue
+        if s['kind'] == 'conv':
+            A = conv_a_float64(x, s)
+            hw = g.shape[2] * g.shape[3]
+            gm = g.double().permute(1, 0, 2, 3).reshape(g.shape[1], -1)
+            G = gm @ gm.t() * (float(n) / hw)
+        else:
+            xa = torch.cat([x.double(), torch.ones(n, 1, dtype=torch.float64, device=dev)], 1)
+            A = xa.t() @ xa / n
+            G = g.double().t() @ g.double() * float(n)
+        worst['A'] = max(worst.get('A', 0.), rel(curv.ema[0], A))
+        worst['G'] = max(worst.get('G', 0.), rel(curv.ema[1], G))
+        # pi-damped inverses of the running averages the step produced
+        eA, eG = curv.ema[0].double(), curv.ema[1].double()
+        pi = ((eA.diagonal().sum() / eA.shape[0]) / (eG.diagonal().sum() / eG.shape[0])).sqrt()
+        r = 1e-3 ** 0.5
+        Ai = torch.linalg.inv(eA + torch.eye(eA.shape[0], dtype=torch.float64, device=dev) * (r * pi))
+        Gi = torch.linalg.inv(eG + torch.eye(eG.shape[0], dtype=torch.float64, device=dev) * (r / pi))
+        worst['A inverse'] = max(worst.get('A inverse', 0.), rel(curv.inv[0], Ai))
+        worst['G inverse'] = max(worst.get('G inverse', 0.), rel(curv.inv[1], Gi))
+        assert curv.info.cpu().tolist() == [0, 0]
+        # preconditioned gradient (first step: the momentum buffer equals it)
+        ps = list(m.parameters())
+        V = raw[offs[id(ps[0])]:offs[id(ps[0])] + ps[0].numel()].view(ps[0].shape[0], -1).double()
+        got = ps[0].grad.reshape(ps[0].shape[0], -1).double()
+        if len(ps) > 1:
+            V = torch.cat([V, raw[offs[id(ps[1])]:offs[id(ps[1])] + ps[1].numel()].double()[:, None]], 1)
+            got = torch.cat([got, ps[1].grad.double()[:, None]], 1)
+        want = curv.inv[1].double() @ V @ curv.inv[0].double()
+        worst['preconditioned gradient'] = max(worst.get('preconditioned gradient', 0.), rel(got, want))
+        del A, G, Ai, Gi, eA, eG
+    print('config 3 step at full size, worst rel. Frobenius errors:',
+          {k: '%.2e' % v for k, v in worst.items()})
+    for k, v in worst.items():
+        assert v < TOL, (k, v)
