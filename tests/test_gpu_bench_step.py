@@ -1,5 +1,6 @@
-"""One step of bench.py's own workload (BASELINE config 3: the ResNet-50 layer set at
-batch 32) checked at full size: for a sample of layers, the largest included, the
+"""One step of bench.py's own workloads (BASELINE config 3: the ResNet-50 layer set at
+batch 32; config 4: AlexNet fc6-fc8 at batch 256) checked at full size: for a sample of
+layers, the largest included, the
 running average after the first step, the pi-damped inverses and the preconditioned
 gradient are recomputed in float64 on the device with library routines (unfold,
 matmul, torch.linalg.inv).  Nothing in the timed step is skipped or cached."""
@@ -21,6 +22,21 @@ def rel(a, b):
     return ((a.double() - b).norm() / b.norm()).item()
 
 
+def inverse_error(X, shift, Y):
+    """Relative error of Y as the inverse of X + shift*I, in float64 on the device:
+    against torch.linalg.inv up to 3000 rows, beyond that (where the library routine
+    can run out of workspace here) through one Newton step,
+    Y_true = Y + Y (I - X Y) + O(|I - X Y|^2)."""
+    n = X.shape[0]
+    Xd = X + torch.eye(n, dtype=torch.float64, device=X.device) * shift
+    Yd = Y.double()
+    if n <= 3000:
+        ref = torch.linalg.inv(Xd)
+        return ((Yd - ref).norm() / ref.norm()).item()
+    R = torch.eye(n, dtype=torch.float64, device=X.device) - Xd @ Yd
+    return ((Yd @ R).norm() / Yd.norm()).item()
+
+
 def conv_a_float64(x, s):
     """sum over the batch of unfold(x) unfold(x)^T / n, image by image."""
     k = s['k']
@@ -32,18 +48,26 @@ def conv_a_float64(x, s):
     return A / x.shape[0]
 
 
-def test_resnet50_step_at_full_size_against_float64_on_device():
+PICKED = {
+    'resnet50': ['conv1', 'layer1.0.conv1', 'layer1.0.conv2', 'layer2.0.conv2',
+                 'layer3.0.downsample', 'layer4.0.conv2', 'layer4.2.conv2', 'layer4.2.conv3', 'fc',
+                 'layer3.1.bn2'],
+    'alexnet_fc': ['fc6', 'fc7', 'fc8'],
+}
+
+
+@pytest.mark.parametrize('workload', ['resnet50', 'alexnet_fc'])
+def test_benchmark_step_at_full_size_against_float64_on_device(workload):
     import bench
     dev = torch.device('cuda:0')
-    specs, batch, _ = bench.WORKLOADS['resnet50']
+    specs, batch, _ = bench.WORKLOADS[workload]
     specs = specs()
     ls = bench.LayerSet(specs, batch, dev)
     raw = ls.flat_raw.clone()
     ls.step()
     torch.cuda.synchronize()
     names = [s['name'] for s in specs]
-    picked = ['conv1', 'layer1.0.conv1', 'layer1.0.conv2', 'layer2.0.conv2', 'layer3.0.downsample',
-              'layer4.0.conv2', 'layer4.2.conv2', 'layer4.2.conv3', 'fc', 'layer3.1.bn2']
+    picked = PICKED[workload]
     offs = {}
     total = 0
     for m in ls.model:
@@ -81,10 +105,8 @@ def test_resnet50_step_at_full_size_against_float64_on_device():
         eA, eG = curv.ema[0].double(), curv.ema[1].double()
         pi = ((eA.diagonal().sum() / eA.shape[0]) / (eG.diagonal().sum() / eG.shape[0])).sqrt()
         r = 1e-3 ** 0.5
-        Ai = torch.linalg.inv(eA + torch.eye(eA.shape[0], dtype=torch.float64, device=dev) * (r * pi))
-        Gi = torch.linalg.inv(eG + torch.eye(eG.shape[0], dtype=torch.float64, device=dev) * (r / pi))
-        worst['A inverse'] = max(worst.get('A inverse', 0.), rel(curv.inv[0], Ai))
-        worst['G inverse'] = max(worst.get('G inverse', 0.), rel(curv.inv[1], Gi))
+        worst['A inverse'] = max(worst.get('A inverse', 0.), inverse_error(eA, r * pi, curv.inv[0]))
+        worst['G inverse'] = max(worst.get('G inverse', 0.), inverse_error(eG, r / pi, curv.inv[1]))
         assert curv.info.cpu().tolist() == [0, 0]
         # preconditioned gradient (first step: the momentum buffer equals it)
         ps = list(m.parameters())
@@ -95,8 +117,15 @@ def test_resnet50_step_at_full_size_against_float64_on_device():
             got = torch.cat([got, ps[1].grad.double()[:, None]], 1)
         want = curv.inv[1].double() @ V @ curv.inv[0].double()
         worst['preconditioned gradient'] = max(worst.get('preconditioned gradient', 0.), rel(got, want))
-        del A, G, Ai, Gi, eA, eG
-    print('config 3 step at full size, worst rel. Frobenius errors:',
+        del A, G, eA, eG
+    print(workload, 'step at full size, worst rel. Frobenius errors:',
           {k: '%.2e' % v for k, v in worst.items()})
     for k, v in worst.items():
-        assert v < TOL, (k, v)
+        # config 4's factors have rank 256 of 4096..9217 before damping; with the benchmark's
+        # damping of 1e-3 their condition number is 2e3 (fc7) and more (fc6), and a float32
+        # inverse of such a matrix is off by about cond * 2^-24 whoever computes it:
+        # scipy.linalg.inv in float32, which is what the reference calls on the CPU, is off
+        # by 1.3e-4 on factors of fc7's shape and spectrum.  What is built from the inverses
+        # (the preconditioned gradient) is exact relative to them.
+        bound = 5e-4 if (workload == 'alexnet_fc' and k.endswith('inverse')) else TOL
+        assert v < bound, (k, v)
