@@ -125,7 +125,10 @@ def test_factor_conv_a_by_correlations(ops, dev, shape, k, p, d):
 # through LDS), with a ragged last tile in one of them
 @pytest.mark.parametrize('shape', [(1, 1, 1, 1), (2, 3, 4, 4), (8, 64, 7, 7), (4, 130, 14, 14),
                                    (16, 64, 56, 56), (3, 257, 5, 3), (32, 1024, 14, 14),
-                                   (32, 2048, 7, 7), (8, 1500, 10, 10)])
+                                   (32, 2048, 7, 7), (8, 1500, 10, 10),
+                                   # small factors over long reductions, ragged sizes
+                                   (32, 128, 28, 28), (24, 100, 30, 31), (20, 40, 30, 31),
+                                   (6, 64, 112, 112)])
 def test_factor_conv_g(ops, dev, shape):
     torch.manual_seed(sum(shape))
     g = torch.randn(*shape) * 1e-2
