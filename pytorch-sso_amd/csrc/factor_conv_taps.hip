@@ -338,7 +338,11 @@ static TapPlanHost plan_taps(int n, int c, int H, int Wd, int kh, int kw, int ph
   double total = 0;
   auto job_k = [&](const JobDesc& jd) { return (long)n * jd.hh * jd.ww; };
   for (int j = 0; j < pd.njobs; ++j) total += (double)job_k(pd.jobs[j]);
-  const double target_items = hp.w == 1 ? 3072.0 : 1024.0;
+  // All workgroups of a launch that fits the chip are resident at once (3 four-wave
+  // workgroups per CU: 768) and share the matrix cores of their CU, so the launch lasts as
+  // long as the fullest CU: a little under one full round (the split counts round up) beats
+  // 1.3 rounds by a quarter.  The one-wave workgroups (8 per CU) do best at 1.5 rounds.
+  const double target_items = hp.w == 1 ? 3072.0 : 700.0;
   int item = 0, part = 0;
   for (int j = 0; j < pd.njobs; ++j) {
     JobDesc& jd = pd.jobs[j];
