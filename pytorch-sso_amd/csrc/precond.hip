@@ -121,7 +121,7 @@ __global__ __launch_bounds__(NTHREADS) void precond_second_kernel(const LayerDes
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 static size_t precond_workspace(int layers, const int* dG, const int* dA) {
-  size_t bytes = align256((size_t)layers * sizeof(LayerDesc));
+  size_t bytes = 2 * align256((size_t)layers * sizeof(LayerDesc));     // one table per product
   for (int l = 0; l < layers; ++l) bytes += align256((size_t)dG[l] * dA[l] * sizeof(float));
   return bytes;
 }
@@ -133,49 +133,61 @@ static int run_layers(int layers, const int* dG, const int* dA, const float* con
                       void* workspace, size_t workspace_bytes, hipStream_t stream) {
   if (layers == 0) return KFAC_OK;
   if (!workspace || workspace_bytes < precond_workspace(layers, dG, dA)) return KFAC_ERR_WORKSPACE;
-  LayerDesc* table = (LayerDesc*)workspace;
-  char* tbase = (char*)workspace + align256((size_t)layers * sizeof(LayerDesc));
+  // Longest tiles first, so that the tail of a launch is made of short tiles: each of
+  // the two products walks the layers in the order of ITS reduction length (dG for the
+  // first, dA for the second), through a descriptor table of its own.
+  const size_t table_bytes = align256((size_t)layers * sizeof(LayerDesc));
+  LayerDesc* tables[2] = {(LayerDesc*)workspace, (LayerDesc*)((char*)workspace + table_bytes)};
+  char* tbase = (char*)workspace + 2 * table_bytes;
+  std::vector<size_t> toff(layers);
   size_t off = 0;
-  // longest tiles first: the table (= grid.y) is ordered by the reduction length of
-  // the second, larger product so that the tail of the launch is made of short tiles
-  std::vector<int> order(layers);
-  for (int l = 0; l < layers; ++l) order[l] = l;
-  std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return dA[a] > dA[b]; });
-  for (int s0 = 0; s0 < layers; s0 += LAYER_CHUNK) {
-    LayerChunk chunk;
-    const int cnt = std::min(LAYER_CHUNK, layers - s0);
-    for (int k = 0; k < cnt; ++k) {
-      const int l = order[s0 + k];
-      LayerDesc& d = chunk.d[k];
-      d.L = L[l];
-      d.R = R[l];
-      d.V = V[l];
-      d.vb = vb ? vb[l] : nullptr;
-      d.meanW = meanW ? meanW[l] : nullptr;
-      d.meanb = meanb ? meanb[l] : nullptr;
-      d.outW = outW[l];
-      d.outb = outb ? outb[l] : nullptr;
-      d.Tt = (float*)(tbase + off);
-      off += align256((size_t)dG[l] * dA[l] * sizeof(float));
-      d.dG = dG[l];
-      d.dA = dA[l];
-      d.dAw = dA[l] - (has_bias[l] ? 1 : 0);
-      d.scale = scale;
-      d.pad = 0;
+  for (int l = 0; l < layers; ++l) {
+    toff[l] = off;
+    off += align256((size_t)dG[l] * dA[l] * sizeof(float));
+  }
+  std::vector<int> order[2];
+  for (int pass = 0; pass < 2; ++pass) {
+    const int* key = pass == 0 ? dG : dA;
+    order[pass].resize(layers);
+    for (int l = 0; l < layers; ++l) order[pass][l] = l;
+    std::stable_sort(order[pass].begin(), order[pass].end(),
+                     [&](int a, int b) { return key[a] > key[b]; });
+    for (int s0 = 0; s0 < layers; s0 += LAYER_CHUNK) {
+      LayerChunk chunk;
+      const int cnt = std::min(LAYER_CHUNK, layers - s0);
+      for (int k = 0; k < cnt; ++k) {
+        const int l = order[pass][s0 + k];
+        LayerDesc& d = chunk.d[k];
+        d.L = L[l];
+        d.R = R[l];
+        d.V = V[l];
+        d.vb = vb ? vb[l] : nullptr;
+        d.meanW = meanW ? meanW[l] : nullptr;
+        d.meanb = meanb ? meanb[l] : nullptr;
+        d.outW = outW[l];
+        d.outb = outb ? outb[l] : nullptr;
+        d.Tt = (float*)(tbase + toff[l]);
+        d.dG = dG[l];
+        d.dA = dA[l];
+        d.dAw = dA[l] - (has_bias[l] ? 1 : 0);
+        d.scale = scale;
+        d.pad = 0;
+      }
+      hipLaunchKernelGGL(layer_setup_kernel, dim3(1), dim3(LAYER_CHUNK), 0, stream, chunk,
+                         tables[pass], s0, cnt);
     }
-    hipLaunchKernelGGL(layer_setup_kernel, dim3(1), dim3(LAYER_CHUNK), 0, stream, chunk, table, s0,
-                       cnt);
   }
   // both products have one tile per 128 x 128 block of the [dG, dA] result; every
   // first product is enqueued before any second one (stream order is the dependency)
   for (int pass = 0; pass < 2; ++pass) {
+    LayerDesc* const table = tables[pass];
     for (int s0 = 0; s0 < layers; s0 += WL_MAX) {
       WorkList wl;
       wl.first = s0;
       wl.n = std::min(WL_MAX, layers - s0);
       wl.cum[0] = 0;
       for (int i = 0; i < wl.n; ++i) {
-        const int l = order[s0 + i];
+        const int l = order[pass][s0 + i];
         wl.cum[i + 1] = wl.cum[i] + cdiv(dG[l], BM) * cdiv(dA[l], BN);
       }
       for (int i = wl.n + 1; i <= WL_MAX; ++i) wl.cum[i] = wl.cum[wl.n];
