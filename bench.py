@@ -29,9 +29,9 @@ METRIC = 'K-FAC step ms (factor+invert+precondition) & fp32 MFMA TFLOP/s, 1 MI35
 PEAK_FP32_MFMA_TFLOPS = 157.3
 # HBM bytes per launch of the factor-build kernels (syrk_kernel, corr_kernel and their reduce /
 # assemble kernels), averaged over the 226 launches of a resnet50 step, from two rocprofv3 --pmc runs
-# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration with a 1 GiB copy): 52.7 MB read + 15.5 MB
+# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration with a 1 GiB copy): 48.0 MB read + 14.6 MB
 # written (the reads include the previous running average, which the epilogues fold in).
-RESNET50_FACTOR_TRAFFIC_BYTES = 68.2e6
+RESNET50_FACTOR_TRAFFIC_BYTES = 62.6e6
 # flops the matrix cores execute for the factor products of one resnet50 step
 # (512 x SQ_INSTS_VALU_MFMA_MOPS_F32 from a rocprofv3 --pmc run): the symmetric products run one
 # triangle, and the stride-1 3x3 layers take 13 spatial correlations instead of 45 block products
