@@ -582,14 +582,25 @@ __device__ __forceinline__ int seg_of(int b, int depth, int T) {
   return (int)((((long)(b + 1) << depth) - 1) / T);
 }
 
-__device__ __forceinline__ MergeTile merge_tile(const MatDesc& m, int depth, int local) {
+__device__ __forceinline__ MergeTile merge_tile(const MatDesc& m, int depth, int local,
+                                                bool last_column_first) {
   MergeTile t;
   t.valid = false;
   const int T = m.T;
   if (T < 2 || local >= (T - 1) * T / 2) return t;
   int bi, bj;
-  upper_tile(xcd_remap(local, (T - 1) * T / 2), T - 1, bi, bj);
+  // No XCD remapping here: the reduction length of a tile varies with its position, and
+  // a contiguous range of tiles per XCD would give one XCD all the long ones.  Dispatch
+  // order deals consecutive tiles to the 8 XCDs in turn, so walking the tiles longest
+  // first balances the XCDs and leaves the short tiles for the end of the launch.
+  upper_tile(local, T - 1, bi, bj);
   bj += 1;
+  if (last_column_first) {
+    // the same pairs, from the last column to the first
+    const int a = bi;
+    bi = T - 1 - bj;
+    bj = T - 1 - a;
+  }
   const int P = seg_of(bi, depth, T);
   if (seg_of(bj, depth, T) != P) return t;
   if (seg_of(bi, depth + 1, T) == seg_of(bj, depth + 1, T)) return t;
@@ -614,7 +625,8 @@ __global__ __launch_bounds__(NTHREADS) void trtri_w_kernel(const MatDesc* table,
   int mat, local;
   work_find(wl, mat, local);
   const MatDesc m = table[mat];
-  const MergeTile t = merge_tile(m, depth, local);
+  // the reduction grows with the column index of the tile
+  const MergeTile t = merge_tile(m, depth, local, true);
   if (!t.valid) return;
   const int n = m.n;
   DenseKM P{m.Y + (size_t)t.X2 * n + t.X2, nullptr, n, t.b2, 0};
@@ -630,7 +642,8 @@ __global__ __launch_bounds__(NTHREADS) void trtri_y_kernel(const MatDesc* table,
   int mat, local;
   work_find(wl, mat, local);
   const MatDesc m = table[mat];
-  const MergeTile t = merge_tile(m, depth, local);
+  // the reduction shrinks with the row index of the tile: row-major order is longest first
+  const MergeTile t = merge_tile(m, depth, local, false);
   if (!t.valid) return;
   const int n = m.n;
   DenseMK P{m.Y + (size_t)t.X1 * n + t.X1, n, t.b1};
@@ -646,8 +659,11 @@ __global__ __launch_bounds__(NTHREADS) void lauum_kernel(const MatDesc* table, c
   work_find(wl, mat, local);
   const MatDesc m = table[mat];
   const int ntiles = m.T * (m.T + 1) / 2;
-  int bi, bj;
-  upper_tile(xcd_remap(local, ntiles), m.T, bi, bj);   // a tile row per L2
+  // column by column from the first: the reduction runs over k >= the column block, so
+  // this is longest first (and no XCD remapping, for the reason given at merge_tile)
+  int a, b;
+  upper_tile(ntiles - 1 - local, m.T, a, b);
+  const int bi = m.T - 1 - b, bj = m.T - 1 - a;
   const int n = m.n;
   DenseMK P{m.Y, n, n};
   EpiStore epi{m.U, n, n, n, 1.f, 0.f, bi != bj};
