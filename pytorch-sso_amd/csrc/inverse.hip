@@ -569,50 +569,60 @@ __global__ __launch_bounds__(FINE_THREADS) void potrf_fine_kernel(const MatDesc*
 // ---- Y = U^-1 by balanced recursive halving over the 128-blocks ---------------
 // Depth d cuts the T blocks of a matrix into 2^d nearly equal segments
 // (boundaries floor(j*T/2^d)); the merge of the two children X1, X2 of a
-// depth-d segment computes  Y12 = -Y11 * U12 * Y22.  A pair of blocks
-// (bi < bj) belongs to the merge of the deepest segment that contains both, so
-// every launch below walks all strictly-upper block pairs and keeps those whose
-// merge is at its depth.
+// depth-d segment computes  Y12 = -Y11 * U12 * Y22, one tile per pair of a block of
+// X1 and a block of X2.  A launch walks the tiles of all merges of its depth.
 struct MergeTile {
   int X1, b1, X2, b2, it, jt;
   bool valid;
 };
 
-__device__ __forceinline__ int seg_of(int b, int depth, int T) {
-  return (int)((((long)(b + 1) << depth) - 1) / T);
+struct Segment {
+  int p0, mid, p1;
+  __host__ __device__ int tiles() const { return (mid - p0) * (p1 - mid); }
+};
+
+__host__ __device__ inline Segment segment(int P, int depth, int T) {
+  Segment s;
+  s.p0 = (int)(((long)P * T) >> depth);
+  s.p1 = (int)(((long)(P + 1) * T) >> depth);
+  s.mid = (int)(((long)(2 * P + 1) * T) >> (depth + 1));
+  return s;
 }
 
+__host__ __device__ inline int merge_tiles(int T, int depth) {
+  int total = 0;
+  for (int P = 0; P < (1 << depth); ++P) total += segment(P, depth, T).tiles();
+  return total;
+}
+
+// Tile `local` of the merges at `depth`.  Each XCD (own L2) takes a contiguous run of the
+// tiles, walked so that a run holds every reduction length in equal measure and
+// neighbouring tiles share an operand panel: the reduction of the first product grows
+// with the column of the tile, so its tiles go row by row (a row shares the U12 panel);
+// that of the second shrinks with the row, so its tiles go column by column (a column
+// shares the W panel); within a row / column the longest comes first.
 __device__ __forceinline__ MergeTile merge_tile(const MatDesc& m, int depth, int local,
-                                                bool last_column_first) {
+                                                bool by_column) {
   MergeTile t;
   t.valid = false;
   const int T = m.T;
-  if (T < 2 || local >= (T - 1) * T / 2) return t;
-  int bi, bj;
-  // No XCD remapping here: the reduction length of a tile varies with its position, and
-  // a contiguous range of tiles per XCD would give one XCD all the long ones.  Dispatch
-  // order deals consecutive tiles to the 8 XCDs in turn, so walking the tiles longest
-  // first balances the XCDs and leaves the short tiles for the end of the launch.
-  upper_tile(local, T - 1, bi, bj);
-  bj += 1;
-  if (last_column_first) {
-    // the same pairs, from the last column to the first
-    const int a = bi;
-    bi = T - 1 - bj;
-    bj = T - 1 - a;
+  const int total = merge_tiles(T, depth);
+  if (local >= total) return t;
+  int item = xcd_remap(local, total);
+  Segment sg = segment(0, depth, T);
+  for (int P = 0; item >= sg.tiles(); sg = segment(++P, depth, T)) item -= sg.tiles();
+  const int rows = sg.mid - sg.p0, cols = sg.p1 - sg.mid;
+  if (by_column) {
+    t.jt = item / rows;
+    t.it = item - t.jt * rows;
+  } else {
+    t.it = item / cols;
+    t.jt = cols - 1 - (item - t.it * cols);
   }
-  const int P = seg_of(bi, depth, T);
-  if (seg_of(bj, depth, T) != P) return t;
-  if (seg_of(bi, depth + 1, T) == seg_of(bj, depth + 1, T)) return t;
-  const int p0 = (int)(((long)P * T) >> depth);
-  const int p1 = (int)(((long)(P + 1) * T) >> depth);
-  const int mid = (int)(((long)(2 * P + 1) * T) >> (depth + 1));
-  t.X1 = p0 * DB;
-  t.b1 = (mid - p0) * DB;
-  t.X2 = mid * DB;
-  t.b2 = min((p1 - mid) * DB, m.n - t.X2);
-  t.it = bi - p0;
-  t.jt = bj - mid;
+  t.X1 = sg.p0 * DB;
+  t.b1 = rows * DB;
+  t.X2 = sg.mid * DB;
+  t.b2 = min(cols * DB, m.n - t.X2);
   t.valid = true;
   return t;
 }
@@ -625,8 +635,7 @@ __global__ __launch_bounds__(NTHREADS) void trtri_w_kernel(const MatDesc* table,
   int mat, local;
   work_find(wl, mat, local);
   const MatDesc m = table[mat];
-  // the reduction grows with the column index of the tile
-  const MergeTile t = merge_tile(m, depth, local, true);
+  const MergeTile t = merge_tile(m, depth, local, false);
   if (!t.valid) return;
   const int n = m.n;
   DenseKM P{m.Y + (size_t)t.X2 * n + t.X2, nullptr, n, t.b2, 0};
@@ -642,8 +651,7 @@ __global__ __launch_bounds__(NTHREADS) void trtri_y_kernel(const MatDesc* table,
   int mat, local;
   work_find(wl, mat, local);
   const MatDesc m = table[mat];
-  // the reduction shrinks with the row index of the tile: row-major order is longest first
-  const MergeTile t = merge_tile(m, depth, local, false);
+  const MergeTile t = merge_tile(m, depth, local, true);
   if (!t.valid) return;
   const int n = m.n;
   DenseMK P{m.Y + (size_t)t.X1 * n + t.X1, n, t.b1};
@@ -843,7 +851,7 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
     const int na = active(2);
     for (int depth = D - 1; depth >= 0 && na > 0; --depth) {
       // matrices with fewer than 2^depth blocks have no merge this deep
-      auto pairs = [&](int T) { return (1 << depth) < T ? (T - 1) * T / 2 : 0; };
+      auto pairs = [&](int T) { return (1 << depth) < T ? merge_tiles(T, depth) : 0; };
       for_worklists(na, pairs, [&](const WorkList& wl, int grid) {
         KFAC_LAUNCH_TILE2(trtri_w_kernel, dim3(grid), stream, table, depth, wl);
       });
