@@ -660,18 +660,77 @@ __global__ __launch_bounds__(NTHREADS) void trtri_y_kernel(const MatDesc* table,
   gemm_tile(P, Q, t.it * BM, t.jt * BN, t.it * DB, t.b1, false, epi, smem);
 }
 
+// Which upper tile (bi <= bj) of Y Y^T a workgroup takes.  The tiles of a column bj all
+// reduce over k >= bj*128 (same length) and share the operand panel Y[bj rows], and the
+// work of a column, (bj + 1) * (T - bj), varies smoothly with bj.  Workgroups go to the
+// 8 XCDs (one L2 each) in turn by dispatch index, so XCD x is given the columns
+// bj = x, x + 8, ... (equal work within 3 %, a panel is read by one L2 only), first
+// column (longest reduction) first.  The classes differ a little in tile count while every
+// XCD gets the same number of workgroups: the surplus tiles of a class, which are its
+// shortest, go to the workgroups that the smaller classes leave without a tile.
+__device__ __forceinline__ int column_class_size(int T, int x) {
+  if (x > T - 1) return 0;
+  const int c = (T - 1 - x) / 8 + 1;
+  return c * (x + 1) + 4 * c * (c - 1);
+}
+
+__device__ __forceinline__ void column_class_tile(int x, int t, int& bi, int& bj) {
+  bj = x;
+  while (t >= bj + 1) {
+    t -= bj + 1;
+    bj += 8;
+  }
+  bi = t;
+}
+
+__device__ __forceinline__ void lauum_tile(int T, int local, int& bi, int& bj) {
+  const int ntiles = T * (T + 1) / 2;
+  const int g = (int)blockIdx.x;
+  const int x = g & 7;
+  const int s8 = (g - local) & 7;                  // where the matrix starts in the grid, mod 8
+  int deficit_before = 0, slots_x = 0, size_x = 0, first_x = 0;
+  int slots[8], size[8];
+#pragma unroll
+  for (int y = 0; y < 8; ++y) {
+    const int first = (y - s8 + 8) & 7;            // first workgroup of this matrix on XCD y
+    slots[y] = max(0, (ntiles - first + 7) / 8);
+    size[y] = column_class_size(T, y);
+    if (y == x) {
+      slots_x = slots[y];
+      size_x = size[y];
+      first_x = first;
+    }
+  }
+  const int t = (local - first_x) / 8;
+  if (t < size_x) {
+    column_class_tile(x, t, bi, bj);
+    return;
+  }
+#pragma unroll
+  for (int y = 0; y < 8; ++y)
+    if (y < x) deficit_before += max(0, slots[y] - size[y]);
+  int r = deficit_before + (t - size_x);           // rank among the tiles without a workgroup
+  (void)slots_x;
+#pragma unroll
+  for (int z = 0; z < 8; ++z) {
+    const int excess = max(0, size[z] - slots[z]);
+    if (r >= 0 && r < excess) {
+      column_class_tile(z, slots[z] + r, bi, bj);
+      return;
+    }
+    r -= excess;
+  }
+  bi = bj = 0;       // not reached: the classes hold exactly ntiles tiles
+}
+
 // dst = Y Y^T over the upper tiles (k >= the later block), mirrored
 __global__ __launch_bounds__(NTHREADS) void lauum_kernel(const MatDesc* table, const WorkList wl) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   int mat, local;
   work_find(wl, mat, local);
   const MatDesc m = table[mat];
-  const int ntiles = m.T * (m.T + 1) / 2;
-  // column by column from the first: the reduction runs over k >= the column block, so
-  // this is longest first (and no XCD remapping, for the reason given at merge_tile)
-  int a, b;
-  upper_tile(ntiles - 1 - local, m.T, a, b);
-  const int bi = m.T - 1 - b, bj = m.T - 1 - a;
+  int bi, bj;
+  lauum_tile(m.T, local, bi, bj);
   const int n = m.n;
   DenseMK P{m.Y, n, n};
   EpiStore epi{m.U, n, n, n, 1.f, 0.f, bi != bj};
