@@ -223,6 +223,7 @@ class LayerSet(object):
         diagonal curvature / EMA / inversion / preconditioning / parameter update, bracketed by HIP
         events on the stream the kernels are launched on (torch's current stream)."""
         torch = self.torch
+        import torchsso
         from torchsso.curv import curvature as _curv
         ev = lambda: torch.cuda.Event(enable_timing=True)
         acc = [0.] * 6
@@ -232,6 +233,7 @@ class LayerSet(object):
             e = [ev() for _ in range(7)]
             e[0].record()
             self.build_factors(('conv', 'linear'))
+            torchsso.join_factor_streams()   # the products run on the library's side streams
             e[1].record()
             self.build_factors(('bn',))
             e[2].record()
@@ -362,6 +364,8 @@ def main():
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--workload', default='resnet50', choices=sorted(WORKLOADS))
+    ap.add_argument('--factor-streams', type=int, default=None,
+                    help='side streams for the factor products (library default: 3; 0 = none)')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run a plain 1 GiB device copy (reference for rocprofv3 --pmc '
@@ -383,6 +387,10 @@ def main():
     if not torch.cuda.is_available():
         print('no HIP device visible', file=sys.stderr)
         sys.exit(1)
+    import torchsso
+    if args.factor_streams is not None:
+        torchsso.set_factor_streams(args.factor_streams)
+    factor_streams = torchsso.factor_streams()
     ms, ev_ms, phases, resident, not_spd = run_gpu(args, specs, batch)
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device='cuda:0').normal_()
@@ -402,7 +410,7 @@ def main():
         'config': {'workload': label, 'batch': batch,
                    'kron_layers': sum(1 for s in specs if s['kind'] != 'bn'),
                    'bn_layers': sum(1 for s in specs if s['kind'] == 'bn'),
-                   'damping': 1e-3, 'ema_decay': 0.95, 'invert_every_step': True,
+                   'damping': 1e-3, 'ema_decay': 0.95, 'invert_every_step': True, 'factor_side_streams': factor_streams,
                    'inputs_resident_GB': round(resident / 1e9, 3)},
         'tflops': round(total_flops / (ms * 1e-3) / 1e12, 2),
         'algorithmic_gflop': {k: round(v / 1e9, 1) for k, v in work.items() if not k.endswith('bytes')},

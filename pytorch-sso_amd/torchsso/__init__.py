@@ -5,7 +5,7 @@ The Python surface is the one of cybertronai/pytorch-sso for the K-FAC path
 up by name on this namespace, torchsso.utils.inv / cholesky); the arithmetic
 runs in hand-written HIP kernels behind the C ABI of libkfac_hip.so.
 """
-from torchsso import _hip, _ops  # NOQA
+from torchsso import _hip, _lanes, _ops  # NOQA
 from torchsso import utils  # NOQA
 
 from torchsso.curv.curvature import Curvature, DiagCurvature, KronCurvature  # NOQA
@@ -18,5 +18,10 @@ from torchsso.curv.fisher import KronFisherLinear, KronFisherConv2d, DiagFisherB
 from torchsso.curv.fisher import DiagFisherLinear, DiagFisherConv2d  # NOQA
 
 from torchsso import optim  # NOQA
+
+# side streams for the factor products (see torchsso._lanes); 0 = caller's stream only
+set_factor_streams = _lanes.set_count
+factor_streams = _lanes.count
+join_factor_streams = _lanes.join
 
 __version__ = '0.1.0'

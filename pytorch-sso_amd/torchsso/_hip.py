@@ -162,9 +162,10 @@ def stream_ptr(device=None):
 
 
 class _Workspace(threading.local):
-    """Per-thread, per-device scratch taken from torch's caching allocator and
-    grown on demand (forward hooks run on the caller's thread, backward hooks
-    on autograd's worker thread; each gets its own buffer)."""
+    """Per-thread, per-device, per-stream scratch taken from torch's caching
+    allocator and grown on demand (forward hooks run on the caller's thread,
+    backward hooks on autograd's worker thread; each gets its own buffer, and so
+    does each stream: kernels of two streams may run at the same time)."""
 
     def __init__(self):
         self.bufs = {}
@@ -173,7 +174,10 @@ class _Workspace(threading.local):
         nbytes = int(nbytes)
         if nbytes == 0:
             return None, 0
-        key = (device.type, device.index)
+        if device.type != 'cuda':
+            raise KfacHipError('scratch requested on %s: the K-FAC kernels run on a HIP device '
+                               'only (no CPU path exists in this package)' % device)
+        key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
         buf = self.bufs.get(key)
         if buf is None or buf.numel() < nbytes:
             # round up so that a slowly growing request does not reallocate each time

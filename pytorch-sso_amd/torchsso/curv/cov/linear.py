@@ -44,7 +44,7 @@ class KronCovLinear(KronCurvature):
         # A = [a,1]^T [a,1] / n                       (reference: linear.py:50-59)
         a = input_data.reshape(-1, input_data.shape[-1]) if input_data.dim() != 2 else input_data
         n = input_data.shape[0]
-        self._build_factor(0, lambda scale, out, beta, prev: _ops.factor_linear(
+        self._build_factor(0, a, lambda scale, out, beta, prev: _ops.factor_linear(
             a, self.bias, scale / n, out=out, beta=beta, prev=prev))
 
     def update_in_backward(self, grad_output):
@@ -52,7 +52,7 @@ class KronCovLinear(KronCurvature):
         #                                              curvature.py:154-155,299-300)
         g = grad_output.reshape(-1, grad_output.shape[-1]) if grad_output.dim() != 2 else grad_output
         n = grad_output.shape[0]
-        self._build_factor(1, lambda scale, out, beta, prev: _ops.factor_linear(
+        self._build_factor(1, g, lambda scale, out, beta, prev: _ops.factor_linear(
             g, False, scale * n, out=out, beta=beta, prev=prev))
 
     def _get_shape(self):

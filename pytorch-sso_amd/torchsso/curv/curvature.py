@@ -12,6 +12,8 @@ mechanics, none in results:
   engine routine is launched once per step, not once per layer;
 * `ema` is updated in place and `inv` / `std` buffers are reused from step to
   step (the reference allocates new tensors each time);
+* the Kronecker factor products are enqueued on side streams (torchsso._lanes) and
+  joined by whoever reads factor data first;
 * the output gradient is taken with a tensor hook on the module output instead
   of the deprecated module backward hook (same tensor, and it also works with
   an in-place activation after the module).
@@ -21,7 +23,7 @@ import math
 import torch
 import torch.nn as nn
 
-from torchsso import _ops
+from torchsso import _lanes, _ops
 
 PI_TYPE_TRACENORM = 'tracenorm'
 
@@ -156,6 +158,7 @@ class Curvature(object):
         (lists of tensors or None) and the two l2 scalars.  (The reference has no
         such method: its optimizer checkpoint pickles the Curvature objects, hooks
         and module included.)"""
+        _lanes.join()
         out = {'l2_reg': float(self._l2_reg), 'l2_reg_ema': float(self._l2_reg_ema)}
         for name in self._STATE_LISTS:
             val = getattr(self, name)
@@ -163,6 +166,7 @@ class Curvature(object):
         return out
 
     def load_state_dict(self, state):
+        _lanes.join()
         device = self.device
         self._l2_reg = state['l2_reg']
         self._l2_reg_ema = state['l2_reg_ema']
@@ -232,34 +236,41 @@ class KronCurvature(Curvature):
     stored; `data`, `A` and `G` rebuild it on demand from the two averages."""
 
     kind = 'kron'
+    _lanes_dealt = 0
 
     def __init__(self, *args, **kwargs):
         super(KronCurvature, self).__init__(*args, **kwargs)
         self._A = None
         self._G = None
         self.fuse_ema = False
+        self._lane = KronCurvature._lanes_dealt   # the side stream its factor products use
+        KronCurvature._lanes_dealt += 1
         self._next = [None, None]        # receives the next running average
         self._fresh = [False, False]     # _next[i] holds the next average (hook ran since the last step)
         self._prev_ok = [False, False]   # _next[i] holds the average before the current one
 
     # ---- raw factors ------------------------------------------------------------
 
-    def _build_factor(self, idx, build):
+    def _build_factor(self, idx, source, build):
         """Runs `build(scale, out, beta, prev)` (a factor kernel computing
-        out = scale * factor + beta * prev) either for the raw factor or, in
-        fused mode, for the next running average."""
+        out = scale * factor + beta * prev, reading the tensor `source`) either for
+        the raw factor or, in fused mode, for the next running average; on this
+        layer's side stream."""
         beta = self.ema_decay
+        device = source.device
+        lane = 2 * self._lane + idx    # A and G of a layer on different lanes, each always on its own
         if self.fuse_ema and self.ema is not None and beta != 1:
             ema = self.ema[idx]
             nxt = self._next[idx]
             if nxt is None or nxt.shape != ema.shape:
                 nxt = torch.empty_like(ema)
-            self._next[idx] = build(beta, nxt, 1. - beta, ema)
+            self._next[idx] = _lanes.run(device, lane, (source, ema),
+                                         lambda: build(beta, nxt, 1. - beta, ema))
             self._fresh[idx] = True
             self._prev_ok[idx] = False
             raw = None
         else:
-            raw = build(1., None, 0., None)
+            raw = _lanes.run(device, lane, (source,), lambda: build(1., None, 0., None))
             self._fresh[idx] = False
         if idx == 0:
             self._A = raw
@@ -267,6 +278,7 @@ class KronCurvature(Curvature):
             self._G = raw
 
     def _raw(self, idx):
+        _lanes.join()
         t = self._A if idx == 0 else self._G
         if t is None and self.ema is not None and (self._fresh[idx] or self._prev_ok[idx]):
             # factor = (newer average - (1 - beta) * older average) / beta
@@ -338,6 +350,7 @@ class KronCurvature(Curvature):
         return self._raw(1)
 
     def adjust_data_scale(self, scale):
+        _lanes.join()
         self._G.mul_(scale)
 
     def std_norm(self):
@@ -366,6 +379,7 @@ def add_value_to_diagonal(X, value):
 def update_ema_all(curvs):
     """Curvature.update_ema for every curvature in the list
     (reference: curvature.py:174-191).  ema_decay weighs the NEW data."""
+    _lanes.join()
     by_beta = {}
     stale = []
     for c in curvs:

@@ -1,0 +1,134 @@
+"""The side streams of the Kronecker factor products (torchsso._lanes): the results
+are the same bits with and without them, and a reader of factor data right after
+backward() sees the finished factors although the kernels run on other streams."""
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+import bench
+import kfac_testlib as T
+import torchsso
+from oracle import kfac_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def restore_stream_count():
+    before = torchsso.factor_streams()
+    yield
+    torchsso.set_factor_streams(before)
+
+
+def layer_set_state(count, specs, steps=3):
+    torchsso.set_factor_streams(count)
+    ls = bench.LayerSet(specs, 32, torch.device('cuda:0'), seed=3)
+    for _ in range(steps):
+        ls.step()
+    torch.cuda.synchronize()
+    out = [p.detach().clone() for p in ls.model.parameters()]
+    for c in ls.curvs:
+        out += [t.clone() for t in c.ema] + [t.clone() for t in c.inv]
+    return out
+
+
+@pytest.mark.parametrize('count', [1, 2, 3, 5])
+def test_layer_set_step_is_bit_identical_with_side_streams(count):
+    assert torchsso.factor_streams() == 3          # the default
+    base = layer_set_state(0, bench.convnet_specs())
+    got = layer_set_state(count, bench.convnet_specs())
+    assert len(base) == len(got)
+    for i, (a, b) in enumerate(zip(base, got)):
+        assert torch.equal(a, b), 'tensor %d differs with %d streams' % (i, count)
+
+
+class Net(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.c1 = nn.Conv2d(16, 64, 3, padding=1)
+        self.c2 = nn.Conv2d(64, 64, 3, padding=1, bias=False)
+        self.c3 = nn.Conv2d(64, 128, 1, stride=2)
+        self.fc = nn.Linear(128, 10)
+
+    def forward(self, x):
+        x = F.relu(self.c1(x))
+        x = F.relu(self.c2(x))
+        x = F.relu(self.c3(x))
+        return self.fc(x.mean(dim=(2, 3)))
+
+
+def test_factors_read_right_after_backward_are_complete():
+    """56x56 inputs at batch 32: the factor kernels of the last hooks are still running
+    when backward() returns.  `curv.data` must wait for them, and the memory of the
+    output gradients (freed by autograd as soon as the hook returns) must not be handed
+    out again under the kernels: fresh tensors are allocated and filled at once."""
+    torch.manual_seed(0)
+    dev = torch.device('cuda:0')
+    model = Net().to(dev)
+    opt = torchsso.optim.SecondOrderOptimizer(
+        model, 'Cov', {'Conv2d': 'Kron', 'Linear': 'Kron'}, {'damping': 1e-3, 'ema_decay': 1.},
+        lr=1e-2)
+    for g in opt.param_groups:
+        g['curv'].fuse_ema = False
+    x = torch.randn(32, 16, 56, 56, device=dev)
+    y = torch.randint(0, 10, (32,), device=dev)
+    model.zero_grad()
+    loss = F.cross_entropy(model(x), y)
+    loss.backward()
+    junk = [torch.full((32, 64, 56, 56), float('nan'), device=dev) for _ in range(4)]
+    got = {}
+    for g in opt.param_groups:
+        c = g['curv']
+        got[c.module] = [t.clone() for t in c.data]
+    torch.cuda.synchronize()
+    del junk
+    for mod, (A, G) in got.items():
+        rec = {'input': mod.data_input.cpu(), 'grad_output': mod.grad_output.cpu()}
+        _, (refA, refG) = T.oracle_factors(mod, rec, torch.float64)
+        for name, mine, ref in (('A', A, refA), ('G', G, refG)):
+            err = O.rel_fro(mine, ref)
+            assert err < 1e-4, (type(mod).__name__, name, err)
+
+
+def test_training_steps_match_single_stream_run():
+    """Three optimizer steps of an autograd model, side streams against none.  The
+    network's own kernels are made deterministic, so every bit must agree."""
+    dev = torch.device('cuda:0')
+    det = torch.backends.cudnn.deterministic
+    torch.backends.cudnn.deterministic = True
+    try:
+        runs = []
+        for count in (0, 3):
+            torchsso.set_factor_streams(count)
+            torch.manual_seed(1)
+            model = Net().to(dev)
+            opt = torchsso.optim.SecondOrderOptimizer(
+                model, 'Cov', {'Conv2d': 'Kron', 'Linear': 'Kron'},
+                {'damping': 1e-3, 'ema_decay': 0.9}, lr=1e-2, momentum=0.9)
+            gen = torch.Generator(device='cpu').manual_seed(5)
+            for _ in range(3):
+                x = torch.randn(16, 16, 28, 28, generator=gen).to(dev)
+                y = torch.randint(0, 10, (16,), generator=gen).to(dev)
+
+                def closure():
+                    opt.zero_grad()
+                    out = model(x)
+                    loss = F.cross_entropy(out, y)
+                    loss.backward()
+                    return loss, out
+                opt.step(closure=closure)
+            torch.cuda.synchronize()
+            runs.append([p.detach().clone() for p in model.parameters()]
+                        + [t.clone() for g in opt.param_groups for t in g['curv'].ema])
+        noise = max(((a - b).norm() / b.norm()).item() for a, b in zip(*runs))
+        assert noise < 1e-6, noise
+    finally:
+        torch.backends.cudnn.deterministic = det
+
+
+def test_stream_count_is_validated():
+    with pytest.raises(ValueError):
+        torchsso.set_factor_streams(-1)
+    with pytest.raises(ValueError):
+        torchsso.set_factor_streams(9)

@@ -517,6 +517,26 @@ def test_product_has_no_cpu_path():
         acc.update([1.0, 2.0])
 
 
+def test_factor_side_streams_host_logic():
+    """The stream count is validated, and tensors that are not on a HIP device never
+    reach a side stream (the launch runs where it is and raises there)."""
+    from torchsso import _lanes
+    before = torchsso.factor_streams()
+    try:
+        for bad in (-1, 9):
+            with pytest.raises(ValueError):
+                torchsso.set_factor_streams(bad)
+        torchsso.set_factor_streams(2)
+        assert torchsso.factor_streams() == 2
+        calls = []
+        out = _lanes.run(torch.device('cpu'), 5, (torch.zeros(1),), lambda: calls.append(1) or 'out')
+        assert out == 'out' and calls == [1]
+        torchsso.join_factor_streams()        # nothing pending: no device is touched
+    finally:
+        torchsso.set_factor_streams(before)
+    assert torchsso.factor_streams() == 3     # the default
+
+
 def test_fisher_closure_exact_and_mc(oracle_ops):
     """Exact Fisher: the G factor of the logits layer equals mean_n(diag(p) - p p^T);
     every layer (also the first) gets a G factor; gradients are those of the true
