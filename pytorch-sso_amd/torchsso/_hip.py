@@ -157,7 +157,10 @@ def dev_ptr(t, what='tensor'):
     return t.data_ptr()
 
 
-def stream_ptr(device=None):
+def stream_ptr(device=None, stream=None):
+    """Raw handle of `stream` (a torch.cuda.Stream), or of torch's current stream."""
+    if stream is not None:
+        return stream.cuda_stream
     return torch.cuda.current_stream(device).cuda_stream
 
 
@@ -170,16 +173,19 @@ class _Workspace(threading.local):
     def __init__(self):
         self.bufs = {}
 
-    def get(self, device, nbytes):
+    def get(self, device, nbytes, stream=None):
         nbytes = int(nbytes)
         if nbytes == 0:
             return None, 0
         if device.type != 'cuda':
             raise KfacHipError('scratch requested on %s: the K-FAC kernels run on a HIP device '
                                'only (no CPU path exists in this package)' % device)
-        key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
+        key = (device.type, device.index, stream_ptr(device, stream))
         buf = self.bufs.get(key)
         if buf is None or buf.numel() < nbytes:
+            if buf is not None and stream is not None:
+                # kernels of that stream may still use the buffer that is dropped here
+                buf.record_stream(stream)
             # round up so that a slowly growing request does not reallocate each time
             size = max(nbytes, 1 << 20)
             size = 1 << (size - 1).bit_length()
@@ -191,7 +197,8 @@ class _Workspace(threading.local):
 _workspace = _Workspace()
 
 
-def workspace(device, nbytes):
-    """(tensor-or-None, usable bytes); the tensor must stay referenced until the
-    kernels using it have been enqueued (stream order then protects it)."""
-    return _workspace.get(device, nbytes)
+def workspace(device, nbytes, stream=None):
+    """(tensor-or-None, usable bytes) of the scratch of `stream` (default: torch's
+    current stream); the tensor must stay referenced until the kernels using it have
+    been enqueued (stream order then protects it)."""
+    return _workspace.get(device, nbytes, stream)

@@ -29,7 +29,7 @@ import torch
 
 _count = 3
 _lock = threading.Lock()
-_streams = {}      # device index -> list of torch.cuda.Stream
+_streams = {}      # device index -> list of (torch.cuda.Stream, torch.cuda.Event for the fork)
 _pending = {}      # device index -> set of lane indices with work since the last join
 
 
@@ -49,36 +49,44 @@ def count():
 
 def _lane_streams(device):
     idx = device.index if device.index is not None else torch.cuda.current_device()
-    with _lock:
-        lst = _streams.setdefault(idx, [])
-        while len(lst) < _count:
-            lst.append(torch.cuda.Stream(device=device))   # default priority
+    lst = _streams.get(idx)
+    if lst is None or len(lst) < _count:
+        with _lock:
+            lst = _streams.setdefault(idx, [])
+            while len(lst) < _count:
+                # (default priority; the event is re-recorded before every product)
+                lst.append((torch.cuda.Stream(device=device), torch.cuda.Event()))
     return idx, lst
 
 
 def run(device, key, reads, launch):
-    """Runs `launch()` (which enqueues kernels on torch's current stream and returns
-    the output tensor) on lane `key % count` of `device`.  `reads`: the tensors the
-    kernels read."""
+    """Runs `launch(stream)` on lane `key % count` of `device`: `launch` enqueues its
+    kernels on the torch.cuda.Stream it is given (None: torch's current stream) and
+    returns the output tensor, allocated on the current stream.  `reads`: the
+    tensors the kernels read."""
     if _count == 0 or device.type != 'cuda':
-        return launch()
+        return launch(None)
     idx, lst = _lane_streams(device)
     lane = key % _count
-    side = lst[lane]
+    side, fork = lst[lane]
     cur = torch.cuda.current_stream(device)
     if side == cur:
-        return launch()
-    side.wait_stream(cur)
-    with torch.cuda.stream(side):
-        out = launch()
+        return launch(None)
+    # the lane waits for what the caller's stream holds now (a later record of the
+    # same event does not change what this wait refers to)
+    with _lock:   # (hooks of two host threads may share a lane)
+        fork.record(cur)
+        side.wait_event(fork)
+    out = launch(side)
     for t in reads:
         if t is not None:
             t.record_stream(side)
-    # the output may have been allocated on either stream and is used on both
     out.record_stream(side)
-    out.record_stream(cur)
-    with _lock:
-        _pending.setdefault(idx, set()).add(lane)
+    pending = _pending.get(idx)
+    if pending is None:
+        with _lock:
+            pending = _pending.setdefault(idx, set())
+    pending.add(lane)
     return out
 
 
@@ -91,8 +99,8 @@ def join(device=None):
         todo = [(i, sorted(l)) for i, l in _pending.items()
                 if l and (device is None or device.index is None or device.index == i)]
         for i, _ in todo:
-            _pending[i] = set()
+            _pending[i].clear()
     for i, lanes in todo:
         cur = torch.cuda.current_stream(i)
         for lane in lanes:
-            cur.wait_stream(_streams[i][lane])
+            cur.wait_stream(_streams[i][lane][0])

@@ -30,32 +30,42 @@ def _prev_ptr(prev):
     return None if prev is None else _hip.dev_ptr(prev, 'previous factor')
 
 
-def factor_linear(x, add_bias, alpha, out=None, beta=0., prev=None):
-    """out = alpha * [x,1]^T [x,1] + beta * (prev if given else out) for x of shape [rows, f]."""
+def _contiguous_for(x, stream, what):
+    """x.contiguous(); with an explicit stream the copy would run on another stream than
+    the kernels that read it, so the caller has to bring a contiguous tensor."""
+    if stream is not None and not x.is_contiguous():
+        raise _hip.KfacHipError('%s must be contiguous when a stream is given' % what)
+    return x.contiguous()
+
+
+def factor_linear(x, add_bias, alpha, out=None, beta=0., prev=None, stream=None):
+    """out = alpha * [x,1]^T [x,1] + beta * (prev if given else out) for x of shape [rows, f].
+    `stream`: a torch.cuda.Stream to enqueue on instead of the current one (the caller
+    orders it after the producers of x / prev and before the readers of out)."""
     lib = _hip.load()
     if x.dim() != 2:
         x = x.reshape(-1, x.shape[-1])
-    x = x.contiguous()
+    x = _contiguous_for(x, stream, 'input')
     rows, f = x.shape
     d = f + (1 if add_bias else 0)
     out = _out_square(out, d, x, beta, prev)
-    ws, ws_bytes = _hip.workspace(x.device, lib.kfac_factor_workspace_bytes(d, rows))
+    ws, ws_bytes = _hip.workspace(x.device, lib.kfac_factor_workspace_bytes(d, rows), stream)
     st = lib.kfac_factor_linear(_hip.dev_ptr(x, 'input'), rows, f, f, int(bool(add_bias)),
                                 float(alpha), float(beta), _prev_ptr(prev),
                                 _hip.dev_ptr(out, 'factor'),
                                 None if ws is None else ws.data_ptr(), ws_bytes,
-                                _hip.stream_ptr(x.device))
+                                _hip.stream_ptr(x.device, stream))
     _hip.check(st, 'kfac_factor_linear')
     return out
 
 
 def factor_conv_a(x, kernel_size, stride, padding, dilation, add_bias, alpha, out=None, beta=0.,
-                  prev=None):
+                  prev=None, stream=None):
     """out = alpha * M M^T + beta * (prev if given else out), M = implicit im2col of x [n, c, H, W]."""
     lib = _hip.load()
     if x.dim() != 4:
         raise _hip.KfacHipError('conv input must be [n, c, H, W], got %s' % (tuple(x.shape),))
-    x = x.contiguous()
+    x = _contiguous_for(x, stream, 'input')
     n, c, H, W = x.shape
     kh, kw = _pair(kernel_size)
     sh, sw = _pair(stride)
@@ -68,29 +78,29 @@ def factor_conv_a(x, kernel_size, stride, padding, dilation, add_bias, alpha, ou
     d = c * kh * kw + (1 if add_bias else 0)
     out = _out_square(out, d, x, beta, prev)
     ws, ws_bytes = _hip.workspace(x.device, lib.kfac_factor_conv_a_workspace_bytes(
-        n, c, H, W, kh, kw, sh, sw, ph, pw, dh, dw, int(bool(add_bias))))
+        n, c, H, W, kh, kw, sh, sw, ph, pw, dh, dw, int(bool(add_bias))), stream)
     st = lib.kfac_factor_conv_a(_hip.dev_ptr(x, 'input'), n, c, H, W, kh, kw, sh, sw, ph, pw,
                                 dh, dw, int(bool(add_bias)), float(alpha), float(beta),
                                 _prev_ptr(prev), _hip.dev_ptr(out, 'factor'),
                                 None if ws is None else ws.data_ptr(), ws_bytes,
-                                _hip.stream_ptr(x.device))
+                                _hip.stream_ptr(x.device, stream))
     _hip.check(st, 'kfac_factor_conv_a')
     return out
 
 
-def factor_conv_g(g, alpha, out=None, beta=0., prev=None):
+def factor_conv_g(g, alpha, out=None, beta=0., prev=None, stream=None):
     """out = alpha * m m^T + beta * (prev if given else out), m = g [n, c, h, w] as [c, n*h*w]."""
     lib = _hip.load()
     if g.dim() != 4:
         raise _hip.KfacHipError('conv output gradient must be [n, c, h, w]')
-    g = g.contiguous()
+    g = _contiguous_for(g, stream, 'grad_output')
     n, c, h, w = g.shape
     out = _out_square(out, c, g, beta, prev)
-    ws, ws_bytes = _hip.workspace(g.device, lib.kfac_factor_workspace_bytes(c, n * h * w))
+    ws, ws_bytes = _hip.workspace(g.device, lib.kfac_factor_workspace_bytes(c, n * h * w), stream)
     st = lib.kfac_factor_conv_g(_hip.dev_ptr(g, 'grad_output'), n, c, h, w, float(alpha),
                                 float(beta), _prev_ptr(prev), _hip.dev_ptr(out, 'factor'),
                                 None if ws is None else ws.data_ptr(), ws_bytes,
-                                _hip.stream_ptr(g.device))
+                                _hip.stream_ptr(g.device, stream))
     _hip.check(st, 'kfac_factor_conv_g')
     return out
 

@@ -47,16 +47,18 @@ class KronCovConv2d(KronCurvature):
         # divided by n only                              (reference: conv.py:47-67)
         conv2d = self._module
         n = data_input.shape[0]
-        self._build_factor(0, data_input, lambda scale, out, beta, prev: _ops.factor_conv_a(
+        data_input = data_input.contiguous()
+        self._build_factor(0, data_input, lambda scale, out, beta, prev, stream: _ops.factor_conv_a(
             data_input, conv2d.kernel_size, conv2d.stride, conv2d.padding, conv2d.dilation,
-            self.bias, scale / n, out=out, beta=beta, prev=prev))
+            self.bias, scale / n, out=out, beta=beta, prev=prev, stream=stream))
 
     def update_in_backward(self, grad_output):
         # G = m m^T / (n h w), then * n^2                (reference: conv.py:69-74,
         #                                                 curvature.py:154-155,299-300)
         n, c, h, w = grad_output.shape
-        self._build_factor(1, grad_output, lambda scale, out, beta, prev: _ops.factor_conv_g(
-            grad_output, scale * n / (h * w), out=out, beta=beta, prev=prev))
+        grad_output = grad_output.contiguous()
+        self._build_factor(1, grad_output, lambda scale, out, beta, prev, stream: _ops.factor_conv_g(
+            grad_output, scale * n / (h * w), out=out, beta=beta, prev=prev, stream=stream))
 
     def _get_shape(self):
         c_out, c_in, k_h, k_w = self._module.weight.shape

@@ -43,17 +43,19 @@ class KronCovLinear(KronCurvature):
     def update_in_forward(self, input_data):
         # A = [a,1]^T [a,1] / n                       (reference: linear.py:50-59)
         a = input_data.reshape(-1, input_data.shape[-1]) if input_data.dim() != 2 else input_data
+        a = a.contiguous()
         n = input_data.shape[0]
-        self._build_factor(0, a, lambda scale, out, beta, prev: _ops.factor_linear(
-            a, self.bias, scale / n, out=out, beta=beta, prev=prev))
+        self._build_factor(0, a, lambda scale, out, beta, prev, stream: _ops.factor_linear(
+            a, self.bias, scale / n, out=out, beta=beta, prev=prev, stream=stream))
 
     def update_in_backward(self, grad_output):
         # G = g^T g / n, then * n^2                   (reference: linear.py:61-67,
         #                                              curvature.py:154-155,299-300)
         g = grad_output.reshape(-1, grad_output.shape[-1]) if grad_output.dim() != 2 else grad_output
+        g = g.contiguous()
         n = grad_output.shape[0]
-        self._build_factor(1, g, lambda scale, out, beta, prev: _ops.factor_linear(
-            g, False, scale * n, out=out, beta=beta, prev=prev))
+        self._build_factor(1, g, lambda scale, out, beta, prev, stream: _ops.factor_linear(
+            g, False, scale * n, out=out, beta=beta, prev=prev, stream=stream))
 
     def _get_shape(self):
         f_out, f_in = self._module.weight.shape

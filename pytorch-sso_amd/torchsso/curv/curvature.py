@@ -252,10 +252,10 @@ class KronCurvature(Curvature):
     # ---- raw factors ------------------------------------------------------------
 
     def _build_factor(self, idx, source, build):
-        """Runs `build(scale, out, beta, prev)` (a factor kernel computing
-        out = scale * factor + beta * prev, reading the tensor `source`) either for
-        the raw factor or, in fused mode, for the next running average; on this
-        layer's side stream."""
+        """Runs `build(scale, out, beta, prev, stream)` (a factor kernel computing
+        out = scale * factor + beta * prev on `stream`, reading the contiguous tensor
+        `source`) either for the raw factor or, in fused mode, for the next running
+        average; on this layer's side stream."""
         beta = self.ema_decay
         device = source.device
         lane = 2 * self._lane + idx    # A and G of a layer on different lanes, each always on its own
@@ -265,12 +265,12 @@ class KronCurvature(Curvature):
             if nxt is None or nxt.shape != ema.shape:
                 nxt = torch.empty_like(ema)
             self._next[idx] = _lanes.run(device, lane, (source, ema),
-                                         lambda: build(beta, nxt, 1. - beta, ema))
+                                         lambda st: build(beta, nxt, 1. - beta, ema, st))
             self._fresh[idx] = True
             self._prev_ok[idx] = False
             raw = None
         else:
-            raw = _lanes.run(device, lane, (source,), lambda: build(1., None, 0., None))
+            raw = _lanes.run(device, lane, (source,), lambda st: build(1., None, 0., None, st))
             self._fresh[idx] = False
         if idx == 0:
             self._A = raw

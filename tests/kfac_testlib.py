@@ -164,18 +164,18 @@ class OracleOps(object):
 
     dtype = torch.float32
 
-    def factor_linear(self, x, add_bias, alpha, out=None, beta=0., prev=None):
+    def factor_linear(self, x, add_bias, alpha, out=None, beta=0., prev=None, stream=None):
         n = x.shape[0]
         r = O.factor_linear_a(x, add_bias, self.dtype) * (n * alpha)
         return self._emit(r, out, beta, prev)
 
     def factor_conv_a(self, x, kernel_size, stride, padding, dilation, add_bias, alpha, out=None, beta=0.,
-                      prev=None):
+                      prev=None, stream=None):
         n = x.shape[0]
         r = O.factor_conv_a(x, kernel_size, stride, padding, dilation, add_bias, self.dtype) * (n * alpha)
         return self._emit(r, out, beta, prev)
 
-    def factor_conv_g(self, g, alpha, out=None, beta=0., prev=None):
+    def factor_conv_g(self, g, alpha, out=None, beta=0., prev=None, stream=None):
         n, c, h, w = g.shape
         r = O.factor_conv_g(g, self.dtype, scale_by_batch=False) * (n * h * w * alpha)
         return self._emit(r, out, beta, prev)

@@ -529,8 +529,8 @@ def test_factor_side_streams_host_logic():
         torchsso.set_factor_streams(2)
         assert torchsso.factor_streams() == 2
         calls = []
-        out = _lanes.run(torch.device('cpu'), 5, (torch.zeros(1),), lambda: calls.append(1) or 'out')
-        assert out == 'out' and calls == [1]
+        out = _lanes.run(torch.device('cpu'), 5, (torch.zeros(1),), lambda st: calls.append(st) or 'out')
+        assert out == 'out' and calls == [None]
         torchsso.join_factor_streams()        # nothing pending: no device is touched
     finally:
         torchsso.set_factor_streams(before)
