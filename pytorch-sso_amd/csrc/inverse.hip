@@ -566,6 +566,100 @@ __global__ __launch_bounds__(FINE_THREADS) void potrf_fine_kernel(const MatDesc*
   }
 }
 
+// The same products for launches of very few tiles (at most SUB_MAX_TILES): every tile is
+// dealt to four workgroups, so that four CUs' matrix cores work on it.  A workgroup
+// takes RB x CB blocks of 32x32 (RB * CB == 4) and 8 waves: a wave does one block over
+// half of the 128-deep reduction and the halves are added through LDS.  The near update
+// is cut into 64x64 quarters (2 x 2 blocks).  The row panel overwrites its own right-hand
+// operand, so its pieces must not share columns: four 128x32 column strips (4 x 1 blocks).
+constexpr int SUB_THREADS = 512;
+constexpr int SUB_SMEM_BYTES = DB * (128 + 32) * (int)sizeof(float);
+constexpr int SUB_MAX_TILES = 64;        // 4 workgroups per tile, one workgroup per CU
+
+template <int RB, int CB>
+__global__ __launch_bounds__(SUB_THREADS) void potrf_sub_kernel(const MatDesc* table, int p,
+                                                                int near, int row_hi,
+                                                                const WorkList wl) {
+  constexpr int WP = 32 * RB, WQ = 32 * CB;
+  static_assert(RB * CB == 4, "a workgroup takes four 32x32 blocks");
+  static_assert(DB * (WP + WQ) * (int)sizeof(float) <= SUB_SMEM_BYTES, "LDS");
+  extern __shared__ __attribute__((aligned(16))) float fsm[];
+  lds_f* const tp = (lds_f*)fsm;
+  lds_f* const tq = tp + DB * WP;
+  int mat, item;
+  work_find(wl, mat, item);
+  const int local = item >> 2, sub = item & 3;
+  const int si = sub / (4 / CB), sj = sub % (4 / CB);
+  const MatDesc m = table[mat];
+  const int n = m.n;
+  int bi, bj;
+  if (near) {
+    if (!trail_tile(m.T, p + 1, row_hi, local, bi, bj)) return;
+  } else {
+    bi = p;
+    bj = p + 1 + local;
+    if (bj >= m.T) return;
+  }
+  const float* kbase = m.U + (size_t)p * DB * n;            // block row p of U
+  const float* P = near ? kbase + bi * DB : m.Y + (size_t)p * DB * n + p * DB;
+  const float* Q = kbase + bj * DB;
+  float* C = m.U + (size_t)bi * DB * n + bj * DB;
+  const int pw = near ? min(DB, n - bi * DB) : DB;
+  const int qw = min(DB, n - bj * DB);
+  const int t = threadIdx.x;
+  const int wave = t >> 6, lane = t & 63;
+  const int r = lane & 31, h = lane >> 5;
+  const int blk = wave & 3, khalf = wave >> 2;
+  const int br = blk / CB, bc = blk % CB;
+  const int row0 = WP * si + 32 * br, col0 = WQ * sj + 32 * bc;   // of this wave's block in the tile
+
+  const __amdgpu_buffer_rsrc_t rp = make_rsrc(P), rq = make_rsrc(Q);
+  float vp[WP / 4], vq[WQ / 4];
+#pragma unroll
+  for (int i = 0; i < WP / 4; ++i) {
+    const int idx = t + SUB_THREADS * i;
+    const int k = idx / WP, col = WP * si + idx % WP;
+    vp[i] = buffer_load(rp, col < pw ? (unsigned)(k * n + col) * 4u : INV_M);
+  }
+#pragma unroll
+  for (int i = 0; i < WQ / 4; ++i) {
+    const int idx = t + SUB_THREADS * i;
+    const int k = idx / WQ, col = WQ * sj + idx % WQ;
+    vq[i] = buffer_load(rq, col < qw ? (unsigned)(k * n + col) * 4u : INV_M);
+  }
+  float old[16];
+  if (near && khalf == 0) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int row = row0 + 8 * (e >> 2) + 4 * h + (e & 3), col = col0 + r;
+      old[e] = (row < pw && col < qw) ? C[(size_t)row * n + col] : 0.f;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < WP / 4; ++i) tp[t + SUB_THREADS * i] = vp[i];
+#pragma unroll
+  for (int i = 0; i < WQ / 4; ++i) tq[t + SUB_THREADS * i] = vq[i];
+  __syncthreads();
+  const v16f acc = lds_mma32(tp + 64 * khalf * WP + 32 * br, WP, 1,
+                             tq + 64 * khalf * WQ + 32 * bc, WQ, 1, 64);
+  __syncthreads();
+  // the second halves of the reduction travel through LDS (the operands are spent)
+  lds_f* const red = tp + blk * 1024;
+  if (khalf == 1) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) red[e * 64 + lane] = acc[e];
+  }
+  __syncthreads();
+  if (khalf == 0) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int row = row0 + 8 * (e >> 2) + 4 * h + (e & 3), col = col0 + r;
+      const float v = acc[e] + red[e * 64 + lane];
+      if (row < pw && col < qw) C[(size_t)row * n + col] = near ? old[e] - v : v;
+    }
+  }
+}
+
 // ---- Y = U^-1 by balanced recursive halving over the 128-blocks ---------------
 // Depth d cuts the T blocks of a matrix into 2^d nearly equal segments
 // (boundaries floor(j*T/2^d)); the merge of the two children X1, X2 of a
@@ -795,6 +889,14 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
                           FINE_SMEM_BYTES) != hipSuccess)
     return KFAC_ERR_LAUNCH;
 
+  if (hipFuncSetAttribute((const void*)potrf_sub_kernel<2, 2>,
+                          hipFuncAttributeMaxDynamicSharedMemorySize,
+                          SUB_SMEM_BYTES) != hipSuccess ||
+      hipFuncSetAttribute((const void*)potrf_sub_kernel<4, 1>,
+                          hipFuncAttributeMaxDynamicSharedMemorySize,
+                          SUB_SMEM_BYTES) != hipSuccess)
+    return KFAC_ERR_LAUNCH;
+
   // descending size order; remember where each caller index went
   std::vector<int> order(nmat);
   for (int i = 0; i < nmat; ++i) order[i] = i;
@@ -868,7 +970,20 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
                          p, info);
       const int nb = active(p + 2);
       if (nb == 0) continue;
-      for_worklists(nb, [&](int T) { return T - p - 1; }, [&](const WorkList& wl, int grid) {
+      auto total_items = [&](int count, auto&& items) {
+        long sum = 0;
+        for (int i = 0; i < count; ++i) sum += std::max(0, (int)items(Ts[i]));
+        return sum;
+      };
+      auto panel_items = [&](int T) { return T - p - 1; };
+      if (total_items(nb, panel_items) <= SUB_MAX_TILES) {
+        for_worklists(nb, [&](int T) { return 4 * std::max(0, panel_items(T)); },
+                      [&](const WorkList& wl, int grid) {
+                        hipLaunchKernelGGL((potrf_sub_kernel<4, 1>), dim3(grid), dim3(SUB_THREADS),
+                                           SUB_SMEM_BYTES, stream, table, p, 0, 0, wl);
+                      });
+      } else
+      for_worklists(nb, panel_items, [&](const WorkList& wl, int grid) {
         if (grid <= FINE_MAX_TILES)
           hipLaunchKernelGGL(potrf_fine_kernel, dim3(grid), dim3(FINE_THREADS), FINE_SMEM_BYTES,
                              stream, table, p, 0, 0, wl);
@@ -877,8 +992,16 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
       });
       if (p + 1 < Pend) {
         // rows (p, Pend) of the outer panel, all columns to the right
-        for_worklists(nb,
-                      [&](int T) { return (std::min(Pend, T) - p - 1) * (T - p - 1); },
+        auto near_items = [&](int T) { return (std::min(Pend, T) - p - 1) * (T - p - 1); };
+        if (total_items(nb, near_items) <= SUB_MAX_TILES) {
+          for_worklists(nb, [&](int T) { return 4 * std::max(0, near_items(T)); },
+                        [&](const WorkList& wl, int grid) {
+                          hipLaunchKernelGGL((potrf_sub_kernel<2, 2>), dim3(grid),
+                                             dim3(SUB_THREADS), SUB_SMEM_BYTES, stream, table, p,
+                                             1, Pend, wl);
+                        });
+        } else
+        for_worklists(nb, near_items,
                       [&](const WorkList& wl, int grid) {
                         if (grid <= FINE_MAX_TILES)
                           hipLaunchKernelGGL(potrf_fine_kernel, dim3(grid), dim3(FINE_THREADS),
