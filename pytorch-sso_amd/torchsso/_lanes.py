@@ -82,11 +82,8 @@ def run(device, key, reads, launch):
         if t is not None:
             t.record_stream(side)
     out.record_stream(side)
-    pending = _pending.get(idx)
-    if pending is None:
-        with _lock:
-            pending = _pending.setdefault(idx, set())
-    pending.add(lane)
+    with _lock:
+        _pending.setdefault(idx, set()).add(lane)
     return out
 
 
