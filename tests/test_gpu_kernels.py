@@ -185,6 +185,32 @@ def test_cholesky_upper_batched(ops, dev):
         assert torch.equal(o, torch.triu(o))
 
 
+def test_inverse_and_cholesky_of_random_ragged_batches(ops, dev):
+    """Batches of one to seven matrices of random sizes up to 1500 (last blocks of every
+    width, few-tile launches of every shape) against float64 on the device."""
+    gen = torch.Generator().manual_seed(7)
+    for trial in range(10):
+        count = int(torch.randint(1, 7, (1,), generator=gen))
+        sizes = [int(torch.randint(1, 1500, (1,), generator=gen)) for _ in range(count)]
+        if trial % 3 == 0:   # a size next to a multiple of the block size
+            sizes.append(max(1, 128 * int(torch.randint(1, 12, (1,), generator=gen))
+                             + int(torch.randint(0, 3, (1,), generator=gen)) - 1))
+        mats = []
+        for n in sizes:
+            a = torch.randn(n, n + 8, generator=gen).to(dev)
+            mats.append(a @ a.t() / (n + 8) + 0.1 * torch.eye(n, device=dev))
+        outs, info = ops.damped_inverse_batched(mats, [1e-3] * len(mats))
+        chol, info2 = ops.cholesky_upper_batched(mats)
+        assert int(info.abs().sum()) == 0 and int(info2.abs().sum()) == 0, sizes
+        for m, o, u in zip(mats, outs, chol):
+            n = m.shape[0]
+            m64 = m.double()
+            ref = torch.linalg.inv(m64 + 1e-3 * torch.eye(n, device=dev, dtype=torch.float64))
+            assert ((o.double() - ref).norm() / ref.norm()).item() < TOL, (sizes, n)
+            assert ((u.double().t() @ u.double() - m64).norm() / m64.norm()).item() < 1e-5, (sizes, n)
+            assert torch.equal(u, torch.triu(u)), (sizes, n)
+
+
 SHAPES = [(10, 193, True), (64, 76, True), (1000, 785, True), (128, 1601, True),
           (512, 1152, False), (1, 2, True), (3, 1, False), (64, 64, False), (130, 257, True)]
 
