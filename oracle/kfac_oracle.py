@@ -27,7 +27,10 @@ which retypes the formula):
                        per-sample gradient would give the square of a sum, is pinned
                        by brute-force loops instead)
   fisher_*             prob == 1 reduces to the Cov factor; the exact sum over classes at the
-                       logits layer equals mean_n(diag(p_n) - p_n p_n^T) (closed form)
+                       logits layer equals mean_n(diag(p_n) - p_n p_n^T) (closed form);
+                       fisher_conv_g and fisher_bn_diag by explicit per-sample loops with
+                       prob != 1 on a 2x3x2x2 input, the h = w = 1 reduction to the linear
+                       case and linearity in prob
   cholesky_upper       U^T U == X, U upper, diag > 0
   sample               injected-noise Kronecker identity
   tri_pack / unpack    the reference's own index formula evaluated by loops

@@ -119,13 +119,16 @@ def oracle_kfac_run(model, x, y, steps, *, lr, damping, ema_decay, l2_reg=0., mo
     return history
 
 
-def compare_with_golden(history_or_optimizer_snapshots, golden, tol, what=('param', 'grad', 'ema', 'inv'),
-                        skip=()):
-    """Worst relative Frobenius error against the golden arrays; asserts <= tol.
+def compare_with_golden(history_or_optimizer_snapshots, golden, tol=1e-4,
+                        what=('param', 'grad', 'ema', 'inv'), skip=(), exceptions=None, label=''):
+    """Relative Frobenius error of every stored array against the golden arrays; prints the
+    worst entry and asserts each one <= tol (1e-4, the bar of the parity tests).
     `skip` lists (group, name, index) entries that are mathematically zero, whose
     stored value is rounding noise (e.g. the gradient of a bias in front of a
-    BatchNorm layer)."""
-    worst = 0.
+    BatchNorm layer).  `exceptions` maps (group, name, index) to (bound, reason) for an
+    entry that is allowed a named, wider bound; every use is printed."""
+    worst, worst_at = 0., None
+    exceptions = exceptions or {}
     for s, snap in enumerate(history_or_optimizer_snapshots):
         for gi, layer in enumerate(snap):
             for key, name in (('params', 'param'), ('grads', 'grad'), ('ema', 'ema'), ('inv', 'inv')):
@@ -136,9 +139,16 @@ def compare_with_golden(history_or_optimizer_snapshots, golden, tol, what=('para
                         continue
                     ref = golden['step%d.g%d.%s%d' % (s, gi, name, k)]
                     err = O.rel_fro(torch.as_tensor(t).reshape(ref.shape), torch.from_numpy(ref))
-                    assert err <= tol, 'step %d layer %d %s%d: rel err %.3e > %.1e' % (
-                        s, gi, name, k, err, tol)
-                    worst = max(worst, err)
+                    where = 'step %d layer %d %s%d' % (s, gi, name, k)
+                    bound = tol
+                    if (gi, name, k) in exceptions:
+                        bound, reason = exceptions[(gi, name, k)]
+                        print('golden %s: %s held to %.1e instead of %.1e (%s): %.3e'
+                              % (label, where, bound, tol, reason, err))
+                    assert err <= bound, '%s: rel err %.3e > %.1e' % (where, err, bound)
+                    if err > worst:
+                        worst, worst_at = err, where
+    print('golden %s: worst rel. Frobenius error %.3e at %s (bar %.0e)' % (label, worst, worst_at, tol))
     return worst
 
 

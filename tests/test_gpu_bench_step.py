@@ -1,9 +1,12 @@
 """One step of bench.py's own workloads (BASELINE config 3: the ResNet-50 layer set at
 batch 32; config 4: AlexNet fc6-fc8 at batch 256) checked at full size: for a sample of
-layers, the largest included, the
-running average after the first step, the pi-damped inverses and the preconditioned
-gradient are recomputed in float64 on the device with library routines (unfold,
-matmul, torch.linalg.inv).  Nothing in the timed step is skipped or cached."""
+layers, the largest included, the running average after the first step, the pi-damped
+inverses and the preconditioned gradient are recomputed in float64 on the device with
+library routines (unfold, matmul, torch.linalg.inv).  The inverses of config 4 and of the
+largest ResNet-50 factors are also put beside the reference's own float32 result on the same
+damped matrix (scipy.linalg.inv through the oracle), with the condition number: where even
+that is further than 1e-4 from float64, the device result may be at most 1.5 x as far.
+Nothing in the timed step is skipped or cached."""
 import os
 import sys
 
@@ -48,12 +51,44 @@ def conv_a_float64(x, s):
     return A / x.shape[0]
 
 
+def norm2(M, iters=40):
+    """Largest singular value of a symmetric float64 matrix by power iteration."""
+    v = torch.ones(M.shape[0], dtype=torch.float64, device=M.device)
+    v /= v.norm()
+    lam = 0.
+    for _ in range(iters):
+        w = M @ v
+        lam = w.norm().item()
+        v = w / lam
+    return lam
+
+
+def inverse_record(name, X, shift, Y):
+    """The device's float32 inverse Y of X + shift*I next to the reference's own float32
+    result on the same matrix: torchsso.utils.inv on a CPU tensor is scipy.linalg.inv in
+    float32 (torchsso/utils/inv_cupy.py:32-34), which is what the oracle's float32 path calls.
+    Returns (condition number, device vs float64, reference float32 vs float64, device vs
+    reference float32); everything but the scipy call runs in float64 on the device."""
+    from oracle import kfac_oracle as O
+    ref32 = O.damped_inverse(X.float().cpu(), float(shift), torch.float32).to(X.device)
+    cond = norm2(X + torch.eye(X.shape[0], dtype=torch.float64, device=X.device) * shift) * \
+        norm2(Y.double())
+    e_dev = inverse_error(X, shift, Y)
+    e_ref = inverse_error(X, shift, ref32)
+    d = rel(Y, ref32.double())
+    print('%-22s n=%5d cond %.2e | device fp32 vs fp64 %.2e | reference fp32 (scipy) vs fp64 %.2e '
+          '| device vs reference fp32 %.2e' % (name, X.shape[0], cond, e_dev, e_ref, d), flush=True)
+    return cond, e_dev, e_ref, d
+
+
 PICKED = {
     'resnet50': ['conv1', 'layer1.0.conv1', 'layer1.0.conv2', 'layer2.0.conv2',
                  'layer3.0.downsample', 'layer4.0.conv2', 'layer4.2.conv2', 'layer4.2.conv3', 'fc',
                  'layer3.1.bn2'],
     'alexnet_fc': ['fc6', 'fc7', 'fc8'],
 }
+# layers whose inverses are also put beside the reference's float32 result
+BESIDE_REFERENCE = {'resnet50': ['layer4.2.conv2', 'fc'], 'alexnet_fc': ['fc6', 'fc7', 'fc8']}
 
 
 @pytest.mark.parametrize('workload', ['resnet50', 'alexnet_fc'])
@@ -62,6 +97,9 @@ def test_benchmark_step_at_full_size_against_float64_on_device(workload):
     dev = torch.device('cuda:0')
     specs, batch, _ = bench.WORKLOADS[workload]
     specs = specs()
+    if workload == 'alexnet_fc':
+        for s in specs:
+            s['relu_input'] = True      # as bench.py runs it: a = clamp(N(0,1), min=0)
     ls = bench.LayerSet(specs, batch, dev)
     raw = ls.flat_raw.clone()
     ls.step()
@@ -75,6 +113,7 @@ def test_benchmark_step_at_full_size_against_float64_on_device(workload):
             offs[id(p)] = total
             total += (p.numel() + 63) // 64 * 64
     worst = {}
+    inverse_bounds = {}     # entry of `worst` -> bound tied to the reference's own float32 error
     for name in picked:
         i = names.index(name)
         s, m, curv, x, g = specs[i], ls.model[i], ls.curvs[i], ls.inputs[i], ls.gouts[i]
@@ -101,12 +140,23 @@ def test_benchmark_step_at_full_size_against_float64_on_device(workload):
             G = g.double().t() @ g.double() * float(n)
         worst['A'] = max(worst.get('A', 0.), rel(curv.ema[0], A))
         worst['G'] = max(worst.get('G', 0.), rel(curv.ema[1], G))
+        del A, G
         # pi-damped inverses of the running averages the step produced
         eA, eG = curv.ema[0].double(), curv.ema[1].double()
         pi = ((eA.diagonal().sum() / eA.shape[0]) / (eG.diagonal().sum() / eG.shape[0])).sqrt()
         r = 1e-3 ** 0.5
-        worst['A inverse'] = max(worst.get('A inverse', 0.), inverse_error(eA, r * pi, curv.inv[0]))
-        worst['G inverse'] = max(worst.get('G inverse', 0.), inverse_error(eG, r / pi, curv.inv[1]))
+        if name in BESIDE_REFERENCE[workload]:
+            for tag, X, shift, Y in (('A', eA, r * pi, curv.inv[0]), ('G', eG, r / pi, curv.inv[1])):
+                key = '%s %s inverse' % (name, tag)
+                _, e_dev, e_ref, _ = inverse_record(key, X, shift.item(), Y)
+                worst[key] = e_dev
+                # 1e-4 where the reference's float32 inverse meets it too; where even
+                # scipy.linalg.inv in float32 is further than that from float64 (error of
+                # any float32 inverse ~ cond * 2^-24), at most 1.5 x the reference's error
+                inverse_bounds[key] = max(TOL, 1.5 * e_ref)
+        else:
+            worst['A inverse'] = max(worst.get('A inverse', 0.), inverse_error(eA, r * pi, curv.inv[0]))
+            worst['G inverse'] = max(worst.get('G inverse', 0.), inverse_error(eG, r / pi, curv.inv[1]))
         assert curv.info.cpu().tolist() == [0, 0]
         # preconditioned gradient (first step: the momentum buffer equals it)
         ps = list(m.parameters())
@@ -117,15 +167,9 @@ def test_benchmark_step_at_full_size_against_float64_on_device(workload):
             got = torch.cat([got, ps[1].grad.double()[:, None]], 1)
         want = curv.inv[1].double() @ V @ curv.inv[0].double()
         worst['preconditioned gradient'] = max(worst.get('preconditioned gradient', 0.), rel(got, want))
-        del A, G, eA, eG
+        del eA, eG
     print(workload, 'step at full size, worst rel. Frobenius errors:',
-          {k: '%.2e' % v for k, v in worst.items()})
+          {k: '%.2e' % v for k, v in worst.items()}, flush=True)
     for k, v in worst.items():
-        # config 4's factors have rank 256 of 4096..9217 before damping; with the benchmark's
-        # damping of 1e-3 their condition number is 2e3 (fc7) and more (fc6), and a float32
-        # inverse of such a matrix is off by about cond * 2^-24 whoever computes it:
-        # scipy.linalg.inv in float32, which is what the reference calls on the CPU, is off
-        # by 1.3e-4 on factors of fc7's shape and spectrum.  What is built from the inverses
-        # (the preconditioned gradient) is exact relative to them.
-        bound = 5e-4 if (workload == 'alexnet_fc' and k.endswith('inverse')) else TOL
-        assert v < bound, (k, v)
+        bound = inverse_bounds.get(k, TOL)
+        assert v <= bound, (k, v, bound)

@@ -36,7 +36,7 @@ def _run_golden(name, builder, opt_cls, opt_args, steps, skip=()):
         ret = opt.step(closure=_closure(model, x, y))
         assert abs(ret[0].item() - float(gold['step%d.loss' % s])) < 1e-4
         snaps.append(T.snapshot_optimizer(opt))
-    return T.compare_with_golden(snaps, gold, 2e-4, skip=skip)
+    return T.compare_with_golden(snaps, gold, skip=skip, label=name)
 
 
 def test_reference_golden_mlp():
@@ -483,7 +483,11 @@ def test_option_tails_and_checkpoint_on_gpu_match_cpu_oracle_path(monkeypatch):
         if not name.startswith('_') and callable(getattr(fake, name)) and hasattr(_ops, name):
             monkeypatch.setattr(_ops, name, getattr(fake, name))
     cpu_params, _ = run(torch.device('cpu'))
+    errs = {}
     for i, (a, b) in enumerate(zip(gpu_params, cpu_params)):
         if i == 1:
             continue        # bias in front of the BatchNorm: zero gradient, rounding noise
-        assert O.rel_fro(a, b) < 2e-4
+        errs[i] = O.rel_fro(a, b)
+    print('parameters after 3 updates, device vs CPU oracle path, rel. Frobenius error per '
+          'tensor:', {k: '%.2e' % v for k, v in errs.items()})
+    assert max(errs.values()) < TOL

@@ -48,7 +48,7 @@ def test_second_order_optimizer_matches_reference_mlp(oracle_ops):
         assert abs(loss.item() - float(gold['step%d.loss' % s])) < 1e-4
         snaps.append(T.snapshot_optimizer(opt))
         assert abs(opt.param_groups[0]['curv'].damping - float(gold['step%d.g0.damping' % s])) < 1e-12
-    T.compare_with_golden(snaps, gold, 2e-4)
+    T.compare_with_golden(snaps, gold)
     assert opt.optim_state == {'step': 3, 'acc_step': 0}
 
 
@@ -65,7 +65,7 @@ def test_second_order_optimizer_matches_reference_convnet(oracle_ops):
     for s in range(2):
         opt.step(closure=_closure(model, x, y))
         snaps.append(T.snapshot_optimizer(opt))
-    T.compare_with_golden(snaps, gold, 2e-4)
+    T.compare_with_golden(snaps, gold)
 
 
 TAILS_ARGS = dict(curv_type='Cov',
@@ -94,7 +94,7 @@ def test_update_tails_match_reference(oracle_ops):
         snaps.append(T.snapshot_optimizer(opt))
     # the conv bias in front of the BatchNorm has a zero gradient (rounding noise, which
     # LARS then scales up to the norm of the bias)
-    T.compare_with_golden(snaps, gold, 2e-4, skip={(0, 'grad', 1), (0, 'param', 1)})
+    T.compare_with_golden(snaps, gold, skip={(0, 'grad', 1), (0, 'param', 1)})
 
 
 def test_accumulation_with_raw_momentum_and_lars_matches_reference(oracle_ops):
@@ -109,7 +109,7 @@ def test_accumulation_with_raw_momentum_and_lars_matches_reference(oracle_ops):
         assert abs(loss.item() - float(gold['step%d.loss' % s])) < 1e-4
         snaps.append(T.snapshot_optimizer(opt))
         assert opt.optim_state == {'step': (s + 1) // 2, 'acc_step': (s + 1) % 2}
-    T.compare_with_golden(snaps, gold, 2e-4)
+    T.compare_with_golden(snaps, gold)
 
 
 DIAG_SQRT_ARGS = dict(curv_type='Cov',
@@ -131,7 +131,7 @@ def test_diagonal_sqrt_curvature_with_bias_correction_matches_reference(oracle_o
         assert abs(loss.item() - float(gold['step%d.loss' % s])) < 1e-4
         snaps.append(T.snapshot_optimizer(opt))
     # the conv bias in front of the BatchNorm has a zero gradient: g / sqrt(g^2) of rounding noise
-    T.compare_with_golden(snaps, gold, 2e-4,
+    T.compare_with_golden(snaps, gold,
                           skip={(0, k, 1) for k in ('grad', 'param', 'ema', 'inv')})
 
 
@@ -150,7 +150,7 @@ def test_vi_optimizer_accumulation_matches_reference(oracle_ops):
         # prob is accumulated with 1/acc_steps per MC sample (reference quirk, vi.py:209)
         assert abs(prob.sum().item() - 3 * x.shape[0]) < 1e-3
         snaps.append(T.snapshot_optimizer(opt))
-    T.compare_with_golden(snaps, gold, 2e-4)
+    T.compare_with_golden(snaps, gold)
 
 
 def test_vogn_matches_reference_with_sampling(oracle_ops):
@@ -171,7 +171,12 @@ def test_vogn_matches_reference_with_sampling(oracle_ops):
         loss, _ = opt.step(closure=_closure(model, x, y))
         assert abs(loss.item() - float(gold['step%d.loss' % s])) < 1e-3 * max(1, abs(loss.item()))
         snaps.append(T.snapshot_optimizer(opt))
-    T.compare_with_golden(snaps, gold, 2e-4)
+    # the raw gradient of the conv bias in front of the BatchNorm is zero up to rounding
+    # noise (1e-9), which the diagonal inverse (1 / damping = 1e3 for a curvature of g^2 ~
+    # 1e-18) scales up next to the prior term l2_reg * bias: that one entry carries the noise
+    # of two different summation orders and gets a named, wider bound
+    T.compare_with_golden(snaps, gold, label='ref_convnet_vogn', exceptions={
+        (0, 'grad', 1): (2e-4, 'zero raw gradient in front of BatchNorm, noise / damping')})
 
 
 def test_vogn_kl_warmup_prior_and_initial_precision_match_reference(oracle_ops):
@@ -194,7 +199,7 @@ def test_vogn_kl_warmup_prior_and_initial_precision_match_reference(oracle_ops):
             assert abs(g['curv'].damping - float(gold['step%d.g%d.damping' % (s, gi)])) < 1e-9
     # the bias of the conv in front of the BatchNorm has a zero gradient (rounding noise
     # over its tiny curvature); everything else, sampled parameters included, must agree
-    T.compare_with_golden(snaps, gold, 2e-4, skip={(0, 'grad', 1)})
+    T.compare_with_golden(snaps, gold, skip={(0, 'grad', 1)})
 
 
 def test_vi_sampling_consumes_generator_in_group_order(oracle_ops):

@@ -324,11 +324,11 @@ def test_oracle_step_matches_reference_mlp():
     hist = T.oracle_kfac_run(model, torch.from_numpy(gold['x']), torch.from_numpy(gold['y']), 3,
                              lr=0.05, damping=1e-3, ema_decay=0.95, l2_reg=1e-3, momentum=0.9,
                              weight_decay=1e-3)
-    worst = T.compare_with_golden(hist, gold, 2e-4)
+    worst = T.compare_with_golden(hist, gold)
     # effective damping = damping + EMA of l2_reg (curvature.py:102-104)
     for s in range(3):
         assert abs(hist[s][0]['damping'] - float(gold['step%d.g0.damping' % s])) < 1e-12
-    assert worst < 2e-4
+    assert worst < 1e-4
 
 
 def test_oracle_step_matches_reference_convnet_bn_raw_momentum():
@@ -337,7 +337,7 @@ def test_oracle_step_matches_reference_convnet_bn_raw_momentum():
     hist = T.oracle_kfac_run(model, torch.from_numpy(gold['x']), torch.from_numpy(gold['y']), 2,
                              lr=0.02, damping=1e-2, ema_decay=0.9, l2_reg=1e-4, momentum=0.5,
                              momentum_type='raw')
-    T.compare_with_golden(hist, gold, 2e-4)
+    T.compare_with_golden(hist, gold)
 
 
 def test_oracle_vi_accumulation_matches_reference():
@@ -345,7 +345,7 @@ def test_oracle_vi_accumulation_matches_reference():
     model = T.load_init(T.build_mlp(), gold)
     hist = T.oracle_kfac_run(model, torch.from_numpy(gold['x']), torch.from_numpy(gold['y']), 2,
                              lr=0.05, damping=1e-3, ema_decay=0.95, momentum=0.9, num_mc_samples=3)
-    T.compare_with_golden(hist, gold, 2e-4)
+    T.compare_with_golden(hist, gold)
 
 
 # ---- Fisher weighting ---------------------------------------------------------
@@ -371,6 +371,52 @@ def test_fisher_factors_reduce_to_cov_and_match_the_presoftmax_closed_form():
         G += O.fisher_linear_g(grad_k, p[:, k], D)
     closed = sum(torch.diag(p[i]) - torch.outer(p[i], p[i]) for i in range(n)) / n
     assert torch.allclose(G, closed, atol=1e-12)
+
+
+def test_fisher_conv_and_batchnorm_weighting_with_nontrivial_prob():
+    """G = sum_n prob[n] * (sum_hw g_n g_n^T) / (n h w)  (torchsso/curv/fisher/conv.py:61-70) and
+    the BatchNorm diagonal  mean_n[(sum_hw xhat^2) * prob[n] * (sum_hw g^2)]
+    (fisher/batchnorm.py:11-30), written as explicit per-sample loops on a 2x3x2x2 input with
+    prob != 1: a prob^2 weighting, a weight along the channel axis or a weight applied to
+    xhat as well would all fail here.  The batch^2 rescale is left out (scale_by_batch=False)
+    so that the loops state the reference formula literally."""
+    torch.manual_seed(13)
+    n, c, h, w = 2, 3, 2, 2
+    g = torch.randn(n, c, h, w, dtype=D)
+    xh = torch.randn(n, c, h, w, dtype=D)
+    prob = torch.tensor([0.3, 0.9], dtype=D)
+    G = torch.zeros(c, c, dtype=D)
+    for b in range(n):
+        for i in range(c):
+            for j in range(c):
+                for y in range(h):
+                    for x in range(w):
+                        G[i, j] += prob[b] * g[b, i, y, x] * g[b, j, y, x]
+    G /= n * h * w
+    assert torch.allclose(O.fisher_conv_g(g, prob, D, scale_by_batch=False), G, atol=1e-13)
+    assert torch.allclose(O.fisher_conv_g(g, prob, D), G * n * n, atol=1e-12)
+    wcurv, bcurv = torch.zeros(c, dtype=D), torch.zeros(c, dtype=D)
+    for b in range(n):
+        for i in range(c):
+            gg = sum(prob[b] * g[b, i, y, x] ** 2 for y in range(h) for x in range(w))
+            xx = sum(xh[b, i, y, x] ** 2 for y in range(h) for x in range(w))
+            wcurv[i] += xx * gg / n
+            bcurv[i] += gg / n
+    got = O.fisher_bn_diag(xh, g, prob, True, D, scale_by_batch=False)
+    assert torch.allclose(got[0], wcurv, atol=1e-13) and torch.allclose(got[1], bcurv, atol=1e-13)
+    got = O.fisher_bn_diag(xh, g, prob, False, D)
+    assert len(got) == 1 and torch.allclose(got[0], wcurv * n * n, atol=1e-12)
+    # h = w = 1 reduces the conv factor to the Linear one, which the closed form at the
+    # logits pins (test above)
+    g1 = torch.randn(5, c, 1, 1, dtype=D)
+    p5 = torch.rand(5, dtype=D)
+    assert torch.allclose(O.fisher_conv_g(g1, p5, D), O.fisher_linear_g(g1.reshape(5, c), p5, D),
+                          atol=1e-12)
+    # and the weight is linear in prob, not quadratic
+    assert torch.allclose(O.fisher_conv_g(g, 2 * prob, D), 2 * O.fisher_conv_g(g, prob, D), atol=1e-12)
+    a2 = O.fisher_bn_diag(xh, g, 2 * prob, True, D)
+    a1 = O.fisher_bn_diag(xh, g, prob, True, D)
+    assert all(torch.allclose(u, 2 * v, atol=1e-12) for u, v in zip(a2, a1))
 
 
 def test_triangular_wire_format_matches_the_reference_index_formula():
