@@ -3,20 +3,41 @@
 #include "common.h"
 #include "operands.h"
 
-#include <mutex>
-#include <set>
+#include <atomic>
 
 namespace kfac {
 
+// Which kernels already had their dynamic-LDS limit raised, per device.  A fixed table
+// of atomics: trivially destructible, so nothing of this library runs at process exit
+// (objects with destructors in a shared library are torn down in an order that other
+// libraries' exit handlers do not expect).
 bool enable_large_lds(const void* kernel, int bytes) {
-  static std::mutex mu;
-  static std::set<const void*> done;
-  std::lock_guard<std::mutex> lock(mu);
-  if (done.count(kernel)) return true;
-  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
-    return false;
-  done.insert(kernel);
-  return true;
+  constexpr int MAX_DEVICES = 64, CAP = 96;
+  static std::atomic<const void*> done[MAX_DEVICES][CAP];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  if (dev >= 0 && dev < MAX_DEVICES) {
+    for (int i = 0; i < CAP; ++i) {
+      const void* k = done[dev][i].load(std::memory_order_acquire);
+      if (k == kernel) return true;
+      if (k != nullptr) continue;
+      if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) !=
+          hipSuccess)
+        return false;
+      // publish in the first free slot from here on (two threads setting the attribute
+      // of one kernel at the same time both succeed; a duplicate entry is harmless)
+      for (; i < CAP; ++i) {
+        const void* expected = nullptr;
+        if (done[dev][i].compare_exchange_strong(expected, kernel, std::memory_order_acq_rel) ||
+            expected == kernel)
+          break;
+      }
+      return true;
+    }
+  }
+  // table full or device index out of its range: set the attribute on every call
+  return hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) ==
+         hipSuccess;
 }
 
 // Tile configuration and k-split of a symmetric d x d product reduced over K:

@@ -879,22 +879,11 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
   if (workspace == nullptr || workspace_bytes < inverse_workspace_bytes(dims))
     return KFAC_ERR_WORKSPACE;
 
-  // the diagonal-block kernel needs more than the default 64 KiB of LDS
-  if (hipFuncSetAttribute((const void*)potrf_diag_kernel,
-                          hipFuncAttributeMaxDynamicSharedMemorySize,
-                          DIAG_SMEM_BYTES) != hipSuccess)
-    return KFAC_ERR_LAUNCH;
-  if (hipFuncSetAttribute((const void*)potrf_fine_kernel,
-                          hipFuncAttributeMaxDynamicSharedMemorySize,
-                          FINE_SMEM_BYTES) != hipSuccess)
-    return KFAC_ERR_LAUNCH;
-
-  if (hipFuncSetAttribute((const void*)potrf_sub_kernel<2, 2>,
-                          hipFuncAttributeMaxDynamicSharedMemorySize,
-                          SUB_SMEM_BYTES) != hipSuccess ||
-      hipFuncSetAttribute((const void*)potrf_sub_kernel<4, 1>,
-                          hipFuncAttributeMaxDynamicSharedMemorySize,
-                          SUB_SMEM_BYTES) != hipSuccess)
+  // kernels that need more than the default 64 KiB of LDS (registered once per process)
+  if (!enable_large_lds((const void*)potrf_diag_kernel, DIAG_SMEM_BYTES) ||
+      !enable_large_lds((const void*)potrf_fine_kernel, FINE_SMEM_BYTES) ||
+      !enable_large_lds((const void*)potrf_sub_kernel<2, 2>, SUB_SMEM_BYTES) ||
+      !enable_large_lds((const void*)potrf_sub_kernel<4, 1>, SUB_SMEM_BYTES))
     return KFAC_ERR_LAUNCH;
 
   // descending size order; remember where each caller index went

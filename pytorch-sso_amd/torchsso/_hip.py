@@ -5,6 +5,7 @@ contiguous fp32 tensor on a HIP device, the call raises.  torch is used only
 for device memory (tensors, the caching allocator for scratch) and for the
 current stream handle.
 """
+import atexit
 import ctypes
 import os
 import threading
@@ -164,6 +165,9 @@ def stream_ptr(device=None, stream=None):
     return torch.cuda.current_stream(device).cuda_stream
 
 
+_all_workspaces = []     # the `bufs` dict of every thread's _Workspace
+
+
 class _Workspace(threading.local):
     """Per-thread, per-device, per-stream scratch taken from torch's caching
     allocator and grown on demand (forward hooks run on the caller's thread,
@@ -172,6 +176,8 @@ class _Workspace(threading.local):
 
     def __init__(self):
         self.bufs = {}
+        with _lock:
+            _all_workspaces.append(self.bufs)
 
     def get(self, device, nbytes, stream=None):
         nbytes = int(nbytes)
@@ -195,6 +201,28 @@ class _Workspace(threading.local):
 
 
 _workspace = _Workspace()
+
+
+def release_workspaces():
+    """Drops every cached scratch buffer (all threads).  Also runs at interpreter exit, after
+    a device synchronisation and before the HIP runtime and the libraries loaded beside it
+    (a profiler's tool library, for one) start their own teardown: nothing of this package
+    is then in flight or holds device memory while they unload."""
+    with _lock:
+        for bufs in _all_workspaces:
+            bufs.clear()
+
+
+def _at_exit():
+    try:
+        if _lib is not None and torch.cuda.is_initialized():
+            torch.cuda.synchronize()
+    except Exception:
+        pass
+    release_workspaces()
+
+
+atexit.register(_at_exit)
 
 
 def workspace(device, nbytes, stream=None):

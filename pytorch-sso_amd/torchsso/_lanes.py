@@ -23,6 +23,7 @@ All default-priority streams.  `set_count(0)` puts every product back on the
 caller's stream.  The results do not depend on the setting: the kernels are
 deterministic and each stream has its own scratch.
 """
+import atexit
 import threading
 
 import torch
@@ -101,3 +102,19 @@ def join(device=None):
         cur = torch.cuda.current_stream(i)
         for lane in lanes:
             cur.wait_stream(_streams[i][lane][0])
+
+
+def _at_exit():
+    """Interpreter exit: wait for the side streams and drop them (and their events) while the
+    HIP runtime is still whole."""
+    try:
+        for lst in _streams.values():
+            for side, _ in lst:
+                side.synchronize()
+    except Exception:
+        pass
+    _pending.clear()
+    _streams.clear()
+
+
+atexit.register(_at_exit)
