@@ -12,7 +12,8 @@
  *    nothing synchronises with the host;
  *  - no entry point allocates or frees memory; scratch comes in as
  *    (workspace, workspace_bytes) and the matching *_workspace_bytes() query
- *    tells the caller how much to bring;
+ *    tells the caller how much to bring (one entry point,
+ *    kfac_damped_inverse_batched_static, brings its own fixed scratch instead);
  *  - the return value is 0 on success or one of the KFAC_ERR_* codes; nothing
  *    throws and nothing keeps a caller pointer after returning;
  *  - sizes: any single matrix (factor, inverse, gradient viewed as 2-D) is at most
@@ -35,6 +36,7 @@ extern "C" {
 #define KFAC_ERR_ARG 1        /* null pointer, non-positive size, matrix above 16384 x 16384 */
 #define KFAC_ERR_WORKSPACE 2  /* workspace_bytes smaller than the query says */
 #define KFAC_ERR_LAUNCH 3     /* the HIP runtime refused a launch */
+#define KFAC_ERR_TOO_LARGE 4  /* the problem does not fit the library's built-in scratch */
 
 /* Version of this ABI (bumped when a signature changes). */
 int kfac_abi_version(void);
@@ -121,6 +123,24 @@ int kfac_pi_damped_inverse_batched(int layers, const int* dA, const int* dG,
 int kfac_damped_inverse_batched(int count, const int* dims, const float* const* src,
                                 const float* damp, float* const* dst, int* info,
                                 void* workspace, size_t workspace_bytes, void* stream);
+
+/* kfac_damped_inverse_batched for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid it).  It has no
+ * counterpart in the reference.  Same arguments and results as kfac_damped_inverse_batched
+ * without the workspace: the descriptor table and the n x n buffers live in an array that
+ * is part of the library's code object (kfac_static_workspace_bytes() = 8 MiB, held by
+ * every GPU the library runs on until the process ends), and the call makes no hipMalloc,
+ * hipFree or other allocating call.  A list that needs more than that
+ * (kfac_inverse_workspace_bytes(count, dims) > kfac_static_workspace_bytes(); e.g. one
+ * matrix above 1447 x 1447) is rejected with KFAC_ERR_TOO_LARGE before anything is
+ * launched.  The first call on a device looks up the array's address on that device (and
+ * raises the LDS limit of the kernels); make that call outside a capture.  All calls on one
+ * GPU share the array: calls that overlap in time on one GPU (two streams, two threads)
+ * race; calls in stream order on one stream do not. */
+size_t kfac_static_workspace_bytes(void);
+int kfac_damped_inverse_batched_static(int count, const int* dims, const float* const* src,
+                                       const float* damp, float* const* dst, int* info,
+                                       void* stream);
 
 /* dst[i] = U with src[i] = U^T U, U upper triangular (strictly lower part
  * written as zero).  Replaces torchsso.utils.cholesky(m, upper=True),

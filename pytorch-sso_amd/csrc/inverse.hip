@@ -17,6 +17,7 @@
 // so small factors ride along with the large ones instead of getting a launch
 // sequence each.
 #include <algorithm>
+#include <atomic>
 #include <vector>
 
 #include "common.h"
@@ -1037,11 +1038,57 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
   return launch_status();
 }
 
+// ---------------------------------------------------------------------------
+// Scratch for the entry point that allocates nothing: one array in device memory,
+// part of the code object, so every GPU this library runs on holds its own copy at
+// its own address until the process ends.  In host code the name `scratch` is only a
+// handle for hipGetSymbolAddress; kernels and memory calls get the address it returns.
+// ---------------------------------------------------------------------------
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)8 << 20;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+constexpr int SCRATCH_MAX_DEVICES = 64;
+static std::atomic<void*> scratch_ptr[SCRATCH_MAX_DEVICES];   // address on each device, once known
+
+// Device address of `scratch` on the current device (looked up on the first call on that
+// device); nullptr on failure.
+static void* static_scratch() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SCRATCH_MAX_DEVICES) return nullptr;
+  void* ptr = scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr != nullptr) return ptr;
+  if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr)
+    return nullptr;
+  scratch_ptr[dev].store(ptr, std::memory_order_release);
+  return ptr;
+}
+
 }  // namespace kfac
 
 using namespace kfac;
 
 extern "C" {
+
+size_t kfac_static_workspace_bytes(void) { return STATIC_SCRATCH_BYTES; }
+
+int kfac_damped_inverse_batched_static(int count, const int* dims, const float* const* src,
+                                       const float* damp, float* const* dst, int* info,
+                                       void* stream) {
+  if (count < 0 || (count > 0 && (!dims || !src || !dst || !info))) return KFAC_ERR_ARG;
+  std::vector<HostMat> mats(count);
+  std::vector<int> d(count);
+  for (int i = 0; i < count; ++i) {
+    if (dims[i] <= 0 || dims[i] > 16384 || !src[i] || !dst[i] || src[i] == dst[i])
+      return KFAC_ERR_ARG;
+    mats[i] = HostMat{src[i], dst[i], dims[i], damp ? damp[i] : 0.f, -1, 0, i};
+    d[i] = dims[i];
+  }
+  if (count == 0) return KFAC_OK;
+  if (inverse_workspace_bytes(d) > STATIC_SCRATCH_BYTES) return KFAC_ERR_TOO_LARGE;
+  void* ptr = static_scratch();
+  if (ptr == nullptr) return KFAC_ERR_LAUNCH;
+  return run_batched(mats, MODE_INVERSE, info, ptr, STATIC_SCRATCH_BYTES, (hipStream_t)stream);
+}
 
 size_t kfac_inverse_workspace_bytes(int count, const int* dims) {
   if (count <= 0 || !dims) return 0;

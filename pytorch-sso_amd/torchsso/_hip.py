@@ -22,7 +22,8 @@ c_f32 = ctypes.c_float
 c_ptr = ctypes.c_void_p
 c_size = ctypes.c_size_t
 
-ERRORS = {1: 'invalid argument', 2: 'workspace too small', 3: 'HIP launch failed'}
+ERRORS = {1: 'invalid argument', 2: 'workspace too small', 3: 'HIP launch failed',
+          4: 'problem too large for the built-in scratch'}
 
 
 class KfacHipError(RuntimeError):
@@ -48,6 +49,8 @@ _SIGNATURES = {
                                                c_ptr, c_ptr, c_ptr, c_size, c_ptr]),
     'kfac_damped_inverse_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
                                             c_ptr, c_size, c_ptr]),
+    'kfac_static_workspace_bytes': (c_size, []),
+    'kfac_damped_inverse_batched_static': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
     'kfac_cholesky_upper_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr,
                                             c_ptr, c_size, c_ptr]),
     'kfac_precondition_workspace_bytes': (c_size, [c_int, c_ptr, c_ptr]),
