@@ -27,6 +27,10 @@ class CovBatchNorm2d(Curvature):
 
 class _DiagCovBatchNorm(DiagCurvature):
 
+    # set to True (on the class or an instance) to have the forward hook store the
+    # normalised input x_hat = (out - bias) / weight as module.data_input
+    expose_normalized_input = False
+
     def forward_postprocess(self, module, input, output):
         assert self._module == module
         bn = module
@@ -35,6 +39,15 @@ class _DiagCovBatchNorm(DiagCurvature):
         out = output.detach()
         # [n, c] sums over the spatial positions of ((out - bias) / weight)^2
         self._sx = _ops.rowsq_sum(out, bn.num_features, bn.weight.detach(), bn.bias.detach())
+        # module.data_input: x_hat, as the reference keeps it (curvature.py:123-136), only
+        # on request: it costs a pass over the activation and a tensor of its size that
+        # nothing here reads
+        if self.expose_normalized_input:
+            shape = (1, -1) + (1,) * (out.dim() - 2)
+            x_hat = (out - bn.bias.detach().view(shape)) / bn.weight.detach().view(shape)
+        else:
+            x_hat = None
+        setattr(module, 'data_input', x_hat)
         setattr(module, 'data_output', output)
         if output.requires_grad:
             output.register_hook(self._on_grad_output)

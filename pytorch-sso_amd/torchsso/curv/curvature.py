@@ -54,7 +54,8 @@ class Curvature(object):
         self.ema_max = None
         self.inv = None
         self.std = None
-        self.info = None   # device int32 status of the last inversion (0 = ok)
+        self.info = None       # device int32 status of the last inversion (0 = ok)
+        self.std_info = None   # same for the last Cholesky factorisation of the inverses
 
         self.use_sqrt_ema = use_sqrt_ema
         self.use_max_ema = use_max_ema
@@ -131,9 +132,17 @@ class Curvature(object):
         self.backward_postprocess(self._module, None, (grad_output,))
 
     def backward_postprocess(self, module, grad_input, grad_output):
-        """Reference: curvature.py:141-155."""
+        """Reference: curvature.py:141-155.  `module.grad_input` is None here: the
+        gradient arrives through a tensor hook on the module output, which sees no
+        gradient with respect to the module input (nothing on the K-FAC path reads
+        it; the reference's value comes from the legacy module hook and may be None
+        as well)."""
         assert self._module == module
         grad_output = grad_output[0].detach()
+        if grad_input is not None:
+            index = 1 if self.bias else 0
+            grad_input = None if grad_input[index] is None else grad_input[index].detach()
+        setattr(module, 'grad_input', grad_input)
         setattr(module, 'grad_output', grad_output)
         self.update_in_backward(grad_output)
 
@@ -463,7 +472,9 @@ def update_std_all(curvs):
         mats.extend(c.inv)
         outs.extend(c.std)
     if mats:
-        _ops.cholesky_upper_batched(mats, outs)
+        _, info = _ops.cholesky_upper_batched(mats, outs)
+        for i, c in enumerate(kron):
+            c.std_info = info[2 * i:2 * i + 2]
     xs, ys = [], []
     for c in curvs:
         if c.kind == 'diag':
@@ -474,6 +485,40 @@ def update_std_all(curvs):
         elif c.kind == 'full':
             raise NotImplementedError
     _ops.sqrt_batched(xs, ys)
+
+
+class NotPositiveDefiniteError(RuntimeError):
+    """A damped curvature factor (or its inverse, for the Cholesky factor of the
+    posterior) had a non-positive pivot: its inverse / std holds garbage."""
+
+
+def check_spd_all(curvs):
+    """Reads the status words the batched inversion and Cholesky factorisation left on
+    the device for every Kronecker curvature in the list (ONE device-to-host copy, which
+    waits for the stream) and raises NotPositiveDefiniteError naming the layers whose
+    factors were not positive definite.  The reference never looks at the solver's
+    status (utils/inv_cupy.py:124,130) and carries NaNs forward instead."""
+    words, owners = [], []
+    for li, c in enumerate(curvs):
+        if c.kind != 'kron':
+            continue
+        for what, info in (('inverse', c.info), ('Cholesky factor of the inverse', c.std_info)):
+            if info is not None:
+                words.append(info.reshape(-1))
+                owners.append((li, c, what))
+    if not words:
+        return
+    flat = torch.cat(words).cpu().tolist()
+    bad = []
+    for k, (li, c, what) in enumerate(owners):
+        for side, code in zip(('A', 'G'), flat[2 * k:2 * k + 2]):
+            if code != 0:
+                bad.append('layer %d (%s): %s of factor %s failed, leading minor of order %d is '
+                           'not positive' % (li, type(c.module).__name__, what, side, code))
+    if bad:
+        raise NotPositiveDefiniteError(
+            'curvature factors that are not positive definite (raise `damping`):\n  '
+            + '\n  '.join(bad))
 
 
 def step_all(curvs, update_std=False, update_inv=True):

@@ -43,6 +43,8 @@ class SecondOrderOptimizer(Optimizer):
         grad_ema_decay, grad_ema_type, l2_reg, weight_decay,
         normalizing_weights, weight_scale, acc_steps, non_reg_for_bn,
         bias_correction, lars, lars_type, update_inv, precondition_grad
+        check_spd (bool, not in the reference): raise NotPositiveDefiniteError when the
+            inversion of a step met a factor that is not positive definite
     """
 
     def __init__(self, model: nn.Module, curv_type: str, curv_shapes: dict, curv_kwargs: dict,
@@ -50,7 +52,8 @@ class SecondOrderOptimizer(Optimizer):
                  grad_ema_decay=1., grad_ema_type='raw', l2_reg=0., weight_decay=0.,
                  normalizing_weights=False, weight_scale=None,
                  acc_steps=1, non_reg_for_bn=False, bias_correction=False,
-                 lars=False, lars_type='preconditioned', update_inv=True, precondition_grad=True):
+                 lars=False, lars_type='preconditioned', update_inv=True, precondition_grad=True,
+                 check_spd=False):
 
         if lr < 0:
             raise ValueError("Invalid learning rate: {}".format(lr))
@@ -86,6 +89,10 @@ class SecondOrderOptimizer(Optimizer):
         self.curv_shapes = {} if curv_shapes is None else curv_shapes
         self.update_inv = update_inv
         self.precondition_grad = precondition_grad
+        # opt-in (not in the reference): after the inversion of a step, read the solver's
+        # status words once (a host synchronisation) and raise if a factor was not
+        # positive definite; may also be switched on later as an attribute
+        self.check_spd = bool(check_spd)
         self.optim_state = {'step': 0, 'acc_step': 0}
 
         # one param_group per leaf module that owns parameters
@@ -215,12 +222,7 @@ class SecondOrderOptimizer(Optimizer):
             loss = closure()
 
             if n > 1:
-                for group in self.param_groups:
-                    grads = [p.grad.data for p in group['params']]
-                    group['acc_grads'].update(grads, scale=1 / n)
-                    curv = group['curv']
-                    if curv is not None:
-                        group['acc_curv'].update(curv.data, scale=1 / n)
+                self._accumulate(1 / n)
 
             self.optim_state['acc_step'] += 1
             if self.optim_state['acc_step'] < n:
@@ -238,6 +240,15 @@ class SecondOrderOptimizer(Optimizer):
                             precondition=self.precondition_grad)
         return loss
 
+    def _accumulate(self, weight):
+        """Adds weight * (current gradients, current curvature data) of every group to the
+        group's accumulators (reference: secondorder.py:175-182, vi.py:211-220)."""
+        for group in self.param_groups:
+            group['acc_grads'].update([p.grad.data for p in group['params']], scale=weight)
+            curv = group['curv']
+            if curv is not None:
+                group['acc_curv'].update(curv.data, scale=weight)
+
     def _update_groups(self, groups, target, update_inv, update_std, precondition):
         for group in groups:
             self.update_preprocess(group, target=target, grad_type='raw')
@@ -247,6 +258,8 @@ class SecondOrderOptimizer(Optimizer):
             if isinstance(update_std, (list, tuple)):
                 update_std = [u for g, u in zip(groups, update_std) if g['curv'] is not None]
             _curv.step_all(curvs, update_std=update_std, update_inv=update_inv)
+            if getattr(self, 'check_spd', False):
+                _curv.check_spd_all(curvs)
             if precondition:
                 _curv.precondition_all([(g['curv'], g[target]) for g in groups
                                         if g['curv'] is not None])

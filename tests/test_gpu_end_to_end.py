@@ -491,3 +491,44 @@ def test_option_tails_and_checkpoint_on_gpu_match_cpu_oracle_path(monkeypatch):
     print('parameters after 3 updates, device vs CPU oracle path, rel. Frobenius error per '
           'tensor:', {k: '%.2e' % v for k, v in errs.items()})
     assert max(errs.values()) < TOL
+
+
+def test_module_attributes_and_positive_definiteness_check_on_gpu():
+    """What the hooks leave on the modules (reference: curvature.py:118-155) and the
+    opt-in check of the solver status: a factor that is not positive definite raises
+    and names its layer."""
+    import torchsso
+    from torchsso.curv import curvature as _curv
+    dev = torch.device('cuda:0')
+    torch.manual_seed(4)
+    model = nn.Sequential(nn.Conv2d(3, 8, 3, padding=1), nn.BatchNorm2d(8), nn.ReLU(),
+                          nn.Flatten(), nn.Linear(8 * 5 * 5, 4)).to(dev)
+    x = torch.randn(6, 3, 5, 5, device=dev)
+    y = torch.randint(0, 4, (6,), device=dev)
+    opt = torchsso.optim.SecondOrderOptimizer(
+        model, 'Cov', {'Conv2d': 'Kron', 'Linear': 'Kron', 'BatchNorm2d': 'Diag'},
+        {'damping': 1e-3, 'ema_decay': 0.9}, check_spd=True)
+    bn_curv = opt.param_groups[1]['curv']
+    bn_curv.expose_normalized_input = True
+    opt.step(closure=_closure(model, x, y))
+    conv, bn, lin = model[0], model[1], model[4]
+    assert torch.equal(conv.data_input, x) and conv.grad_output.shape == (6, 8, 5, 5)
+    assert conv.grad_input is None and lin.grad_input is None
+    assert lin.data_input.shape == (6, 200) and lin.grad_output.shape == (6, 4)
+    # BatchNorm: x_hat on request, from the output the hook saw (parameters have moved since)
+    assert bn.data_input.shape == (6, 8, 5, 5)
+    var = bn.data_input.var(dim=(0, 2, 3), unbiased=False)
+    assert torch.allclose(bn.data_input.mean(dim=(0, 2, 3)), torch.zeros(8, device=dev), atol=1e-5)
+    assert torch.allclose(var, torch.ones(8, device=dev), atol=1e-3)
+    bn_curv.expose_normalized_input = False
+    opt.step(closure=_closure(model, x, y))
+    assert bn.data_input is None
+
+    kron = [g['curv'] for g in opt.param_groups if g['curv'].kind == 'kron']
+    _curv.check_spd_all(kron)                            # healthy
+    d = kron[1].ema[0].shape[0]
+    kron[1].ema[0].copy_(-torch.eye(d, device=dev))      # the Linear layer's A factor
+    _curv.update_inv_all(kron)
+    with pytest.raises(_curv.NotPositiveDefiniteError,
+                       match=r'layer 1 \(Linear\): inverse of factor A failed, leading minor of order 1'):
+        _curv.check_spd_all(kron)

@@ -202,6 +202,65 @@ def test_vogn_kl_warmup_prior_and_initial_precision_match_reference(oracle_ops):
     T.compare_with_golden(snaps, gold, skip={(0, 'grad', 1)})
 
 
+def test_kl_rate_follows_the_stateful_warmup_of_the_reference():
+    """The reference keeps l2_reg / std_scale in the param groups and moves them in
+    adjust_kl_weighting after every update (optim/vi.py:150-172): nothing while
+    step > warmup_steps, else rate = (init + step / warmup * (target - init)) / init.
+    Simulated here as that loop, against the closed function of the step."""
+    import math
+    from torchsso.optim.vi import kl_rate
+    for warmup, init, target in ((3, 0.1, 0.5), (1000, 0.01, 1.), (2.5, 0.2, 0.1), (0.5, 0.1, 1.),
+                                 (1, 0.3, 0.3)):
+        rate = 1.                                   # what the groups hold, relative to the start
+        for step in range(1, 12):
+            if not warmup < step:
+                rate = (init + step / warmup * (target - init)) / init
+            assert kl_rate(step, warmup, init, target) == rate, (warmup, step)
+    assert kl_rate(7, None, 0.01, 1.) == 1.
+    assert kl_rate(0, 5, 0.01, 1.) == 1.
+    # and the optimizer applies it to the groups that have a prior term only
+    model = nn.Sequential(nn.Linear(4, 3), nn.BatchNorm1d(3))
+    opt = torchsso.optim.VIOptimizer(model, 50, 'Cov', {'Linear': 'Kron', 'BatchNorm1d': 'Diag'},
+                                     {}, non_reg_for_bn=True, warmup_kl_weighting_steps=4,
+                                     warmup_kl_weighting_init=0.1, kl_weighting=0.5, prior_variance=2)
+    lin, bn = opt.param_groups
+    assert lin['l2_reg'] == 0.1 / 50 / 2 and lin['std_scale'] == math.sqrt(0.1 / 50)
+    assert bn['l2_reg'] == 0 and bn['std_scale'] == 0
+    opt.optim_state['step'] = 2
+    opt.adjust_kl_weighting()
+    r = kl_rate(2, 4, 0.1, 0.5)
+    assert lin['l2_reg'] == r * (0.1 / 50 / 2) and lin['std_scale'] == math.sqrt(r) * math.sqrt(0.1 / 50)
+    assert bn['l2_reg'] == 0 and bn['std_scale'] == 0
+    opt.optim_state['step'] = 9
+    lin['l2_reg'] = 123.                           # past the warm-up nothing is touched
+    opt.adjust_kl_weighting()
+    assert lin['l2_reg'] == 123.
+
+
+def test_check_spd_raises_and_names_the_layer(oracle_ops, monkeypatch):
+    """check_spd=True: the status words of the inversion are read once per step and a
+    factor that was not positive definite raises, naming the layer, instead of the
+    reference's silent NaNs (utils/inv_cupy.py:124,130 never read dev_info)."""
+    from torchsso.curv.curvature import NotPositiveDefiniteError
+    torch.manual_seed(2)
+    model = nn.Sequential(nn.Linear(4, 3), nn.ReLU(), nn.Linear(3, 2))
+    x, y = torch.randn(8, 4), torch.randint(0, 2, (8,))
+    opt = torchsso.optim.SecondOrderOptimizer(model, 'Cov', {'Linear': 'Kron'}, {'damping': 1e-3},
+                                              check_spd=True)
+    opt.step(closure=_closure(model, x, y))        # healthy factors: no complaint
+    real = oracle_ops.pi_damped_inverse_batched
+
+    def failing(As, Gs, dampings, A_invs=None, G_invs=None, info=None):
+        a, g, info = real(As, Gs, dampings, A_invs, G_invs, info)
+        info[3] = 2                                 # layer 1, factor G, leading minor 2
+        return a, g, info
+    monkeypatch.setattr(_ops, 'pi_damped_inverse_batched', failing)
+    with pytest.raises(NotPositiveDefiniteError, match=r'layer 1 \(Linear\): inverse of factor G.*order 2'):
+        opt.step(closure=_closure(model, x, y))
+    opt.check_spd = False                           # the default: nothing is read
+    opt.step(closure=_closure(model, x, y))
+
+
 def test_vi_sampling_consumes_generator_in_group_order(oracle_ops):
     """With a std present, params = mean + std_scale * U_G E U_A with E drawn by
     torch.randn in param_group order after manual_seed(step + seed)."""
