@@ -1,7 +1,8 @@
 """K-FAC step benchmark on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50|alexnet_fc|convnet|mlp]
-                    [--no-cpu-baseline] [--copy-calibration]
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+                    [--workload resnet50|alexnet_fc|convnet|mlp|noisy_kfac|resnet50_train]
+                    [--factor-streams N] [--no-cpu-baseline] [--copy-calibration]
 
 A "step" is one pass of the K-FAC hot path over one batch of synthetic input,
 driven through the public torchsso API: for every layer the two Kronecker
@@ -12,8 +13,14 @@ gradients and the parameter update.  The default workload is BASELINE config 3:
 the 53 convolutions + fc of a ResNet-50 at batch 32, 224x224 (real per-layer
 activation / gradient shapes, N(0,1) data), with diagonal curvature for the 53
 BatchNorm layers.  All inputs are resident in HBM before the timed region.
+`--workload noisy_kfac` is BASELINE config 5: VIOptimizer.step on config 2's
+network, 4 MC samples, timed from the second step (forward and backward of the
+network included: the factor products run inside its hooks).
+`--workload resnet50_train` times whole training steps of the ResNet-50 itself (forward,
+backward, K-FAC step on real activations) beside plain SGD steps of the same network.
 
-Prints ONE JSON line (see the keys below).  `value` is the step time in ms.
+Prints ONE JSON line.  `value` is the step time in ms; `host_enqueue_ms` the host's
+own time to enqueue a step; `roofline.executed_*` come from the library's tile plan.
 """
 import argparse
 import json
@@ -27,15 +34,28 @@ sys.path.insert(0, ROOT)
 
 METRIC = 'K-FAC step ms (factor+invert+precondition) & fp32 MFMA TFLOP/s, 1 MI355X'
 PEAK_FP32_MFMA_TFLOPS = 157.3
-# HBM bytes per launch of the factor-build kernels (syrk_kernel, corr_kernel and their reduce /
-# assemble kernels), averaged over the 226 launches of a resnet50 step, from two rocprofv3 --pmc runs
-# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration with a 1 GiB copy): 48.0 MB read + 14.6 MB
-# written (the reads include the previous running average, which the epilogues fold in).
-RESNET50_FACTOR_TRAFFIC_BYTES = 62.6e6
-# flops the matrix cores execute for the factor products of one resnet50 step
-# (512 x SQ_INSTS_VALU_MFMA_MOPS_F32 from a rocprofv3 --pmc run): the symmetric products run one
-# triangle, and the stride-1 3x3 layers take 13 spatial correlations instead of 45 block products
-RESNET50_FACTOR_EXECUTED_FLOP = 560.6e9
+# rocprofv3 --pmc readings of the factor-build kernels of a resnet50 step, kept with the
+# profile summary they come from (counter runs cannot be made from inside this script):
+#   traffic_bytes_per_launch   HBM bytes per launch (FETCH_SIZE, WRITE_SIZE, calibrated)
+#   executed_flop_per_step_pmc 512 x SQ_INSTS_VALU_MFMA_MOPS_F32
+# The second one is the check on the plan arithmetic below: if the flops this script
+# derives from the library's tile / split plan differ from it by more than 3 %, the plan
+# has changed since the counters were read, and the line says so instead of quoting them.
+PMC_SUMMARY = os.path.join(ROOT, 'profiles', 'factor_build_resnet50_b32_hbm_traffic.txt')
+
+
+def read_pmc_summary(path=PMC_SUMMARY):
+    vals = {}
+    try:
+        with open(path) as f:
+            for line in f:
+                parts = line.split('=')
+                if len(parts) == 2 and parts[0].strip() in ('traffic_bytes_per_launch',
+                                                            'executed_flop_per_step_pmc'):
+                    vals[parts[0].strip()] = float(parts[1].split()[0])
+    except OSError:
+        pass
+    return vals
 
 
 # ---------------------------------------------------------------------------
@@ -103,6 +123,59 @@ WORKLOADS = {
 }
 
 
+def build_resnet50(num_classes=1000):
+    """The network config 3's layer list comes from, as torch modules: ResNet-50 with
+    Bottleneck blocks [3, 4, 6, 3], the stride of a stage on its first block's 3x3
+    convolution, bias-free convolutions each followed by BatchNorm, a 1x1 projection on the
+    first block of every stage, global average pooling and a 2048 -> classes linear layer.
+    Module order = resnet50_specs() order (used by the tests that run the K-FAC step on
+    real activations and by --workload resnet50_train)."""
+    import torch.nn as nn
+    import torch.nn.functional as F
+
+    class Block(nn.Module):
+        def __init__(self, inplanes, planes, stride, project):
+            super(Block, self).__init__()
+            self.conv1 = nn.Conv2d(inplanes, planes, 1, bias=False)
+            self.bn1 = nn.BatchNorm2d(planes)
+            self.conv2 = nn.Conv2d(planes, planes, 3, stride, 1, bias=False)
+            self.bn2 = nn.BatchNorm2d(planes)
+            self.conv3 = nn.Conv2d(planes, 4 * planes, 1, bias=False)
+            self.bn3 = nn.BatchNorm2d(4 * planes)
+            if project:
+                self.downsample = nn.Conv2d(inplanes, 4 * planes, 1, stride, bias=False)
+                self.downsample_bn = nn.BatchNorm2d(4 * planes)
+            else:
+                self.downsample = None
+
+        def forward(self, x):
+            y = F.relu(self.bn1(self.conv1(x)))
+            y = F.relu(self.bn2(self.conv2(y)))
+            y = self.bn3(self.conv3(y))
+            skip = x if self.downsample is None else self.downsample_bn(self.downsample(x))
+            return F.relu(y + skip)
+
+    class Net(nn.Module):
+        def __init__(self):
+            super(Net, self).__init__()
+            self.conv1 = nn.Conv2d(3, 64, 7, 2, 3, bias=False)
+            self.bn1 = nn.BatchNorm2d(64)
+            blocks, inplanes = [], 64
+            for planes, count, stride in ((64, 3, 1), (128, 4, 2), (256, 6, 2), (512, 3, 2)):
+                for b in range(count):
+                    blocks.append(Block(inplanes, planes, stride if b == 0 else 1, b == 0))
+                    inplanes = 4 * planes
+            self.blocks = nn.Sequential(*blocks)
+            self.fc = nn.Linear(2048, num_classes)
+
+        def forward(self, x):
+            x = F.max_pool2d(F.relu(self.bn1(self.conv1(x))), 3, 2, 1)
+            x = self.blocks(x)
+            return self.fc(x.mean(dim=(2, 3)))
+
+    return Net()
+
+
 def spec_dims(s, batch):
     """(dA, dG, L) of a Kron layer."""
     if s['kind'] == 'conv':
@@ -125,6 +198,28 @@ def algorithmic_work(specs, batch):
         w['ema_bytes'] += 12. * (dA * dA + dG * dG)
         w['update_bytes'] += 20. * dG * dA
     return w
+
+
+def factor_executed_flops(specs, batch):
+    """fp32 MFMA flops the factor kernels execute for one step, from the same tile / split /
+    correlation plan the launches use (the library's plan queries): upper-triangular tiles x
+    whole reduction chunks x 2 * tile^2 * chunk depth; 13 shared correlations instead of 45
+    tap-pair products for a stride-1 3x3 layer."""
+    from torchsso import _hip
+    lib = _hip.load()
+    total = 0.
+    for s in specs:
+        if s['kind'] == 'bn':
+            continue
+        dA, dG, L = spec_dims(s, batch)
+        if s['kind'] == 'conv':
+            total += lib.kfac_factor_conv_a_executed_flops(
+                batch, s['cin'], s['hin'], s['hin'], s['k'], s['k'], s['stride'], s['stride'],
+                s['pad'], s['pad'], 1, 1, int(s['bias']))
+        else:
+            total += lib.kfac_factor_executed_flops(dA, L)
+        total += lib.kfac_factor_executed_flops(dG, L)
+    return total
 
 
 # ---------------------------------------------------------------------------
@@ -251,26 +346,250 @@ class LayerSet(object):
         return [a / iters for a in acc]
 
 
-def run_gpu(args, specs, batch):
+def time_steps(step, steps, warmup):
+    """(ms per step by the slower of HIP events and the host clock, ms by events, host
+    enqueue ms per step).  The third figure is the host's own time to enqueue a step with no
+    synchronisation in between (Python + ctypes + launch calls), taken over a second run of
+    the same steps; where it approaches the first, the step is bound by the host."""
     import torch
-    dev = torch.device('cuda:0')
-    ls = LayerSet(specs, batch, dev)
-    for _ in range(args.warmup):
-        ls.step()
+    for _ in range(warmup):
+        step()
     torch.cuda.synchronize()
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     start.record()
-    for _ in range(args.steps):
-        ls.step()
+    for _ in range(steps):
+        step()
     end.record()
     torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    ev_ms = start.elapsed_time(end) / args.steps
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev_ms = start.elapsed_time(end) / steps
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    host_ms = (time.perf_counter() - t0) * 1e3 / steps
+    torch.cuda.synchronize()
+    return max(wall_ms, ev_ms), ev_ms, host_ms
+
+
+def run_gpu(args, specs, batch):
+    import torch
+    dev = torch.device('cuda:0')
+    ls = LayerSet(specs, batch, dev)
+    ms, ev_ms, host_ms = time_steps(ls.step, args.steps, args.warmup)
     phases = ls.timed_phases(max(2, min(args.steps, 5)))
     infos = [c.info for c in ls.curvs if c.kind == 'kron']
     not_spd = int(sum(int((i != 0).sum().item()) for i in infos))
-    return max(wall_ms, ev_ms), ev_ms, phases, ls.bytes_resident(), not_spd
+    return ms, ev_ms, host_ms, phases, ls.bytes_resident(), not_spd
+
+
+# ---------------------------------------------------------------------------
+# BASELINE config 5: Noisy K-FAC (VIOptimizer) on config 2's network
+# ---------------------------------------------------------------------------
+
+class PhaseClock(object):
+    """Brackets named functions with HIP events on the current stream while a step runs and
+    sums the elapsed times per name; the functions are patched in place for the duration of
+    `with clock:` only (an instrumented run, separate from the timed one)."""
+
+    def __init__(self, targets):
+        self.targets = targets            # name -> (object, attribute)
+        self.pairs = {}
+        self.saved = []
+
+    def wrap(self, name, fn):
+        import torch
+
+        def timed(*a, **k):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            out = fn(*a, **k)
+            e1.record()
+            self.pairs.setdefault(name, []).append((e0, e1))
+            return out
+        return timed
+
+    def __enter__(self):
+        for name, (obj, attr) in self.targets.items():
+            fn = getattr(obj, attr)
+            self.saved.append((obj, attr, fn))
+            setattr(obj, attr, self.wrap(name, fn))
+        return self
+
+    def __exit__(self, *exc):
+        for obj, attr, fn in self.saved:
+            setattr(obj, attr, fn)
+        self.saved = []
+
+    def totals_ms(self):
+        import torch
+        torch.cuda.synchronize()
+        return {name: sum(a.elapsed_time(b) for a, b in pairs) for name, pairs in self.pairs.items()}
+
+
+class NoisyKfacJob(object):
+    """The network and data of BASELINE config 2 (conv 3->64 k5, pool, conv 64->128 k5, pool,
+    3200-384-192-10; batch 128 of 3x32x32) under VIOptimizer with 4 MC samples per step,
+    Kronecker curvature for Conv2d and Linear: per step 4 x (posterior sample, forward,
+    backward with the factor products in the hooks, accumulation), then the running average,
+    the pi-damped inversion, the Cholesky factors of the inverses, preconditioning and the
+    update of the posterior means (reference: optim/vi.py:174-258)."""
+
+    MC = 4
+
+    def __init__(self, device, batch=128):
+        import torch
+        import torch.nn as nn
+        import torch.nn.functional as F
+        import torchsso
+        torch.manual_seed(1)
+        self.model = nn.Sequential(
+            nn.Conv2d(3, 64, 5), nn.ReLU(), nn.MaxPool2d(2),
+            nn.Conv2d(64, 128, 5), nn.ReLU(), nn.MaxPool2d(2), nn.Flatten(),
+            nn.Linear(3200, 384), nn.ReLU(), nn.Linear(384, 192), nn.ReLU(),
+            nn.Linear(192, 10)).to(device)
+        gen = torch.Generator().manual_seed(0)
+        self.x = torch.randn(batch, 3, 32, 32, generator=gen).to(device)
+        self.y = torch.randint(0, 10, (batch,), generator=gen).to(device)
+        self.opt = torchsso.optim.VIOptimizer(
+            self.model, 50000, 'Cov', {'Conv2d': 'Kron', 'Linear': 'Kron'},
+            {'damping': 1e-3, 'ema_decay': 0.95}, lr=1e-3, momentum=0.9,
+            num_mc_samples=self.MC, prior_variance=1, kl_weighting=1, seed=1)
+        self.F = F
+
+    def closure(self):
+        self.model.zero_grad()
+        out = self.model(self.x)
+        loss = self.F.cross_entropy(out, self.y)
+        loss.backward()
+        return loss, out
+
+    def step(self):
+        self.opt.step(closure=self.closure)
+
+    def timed_phases(self, iters):
+        from torchsso.curv import curvature as _curv
+        clock = PhaseClock({
+            'sample': (_curv, 'sample_all'),
+            'forward_backward_factor': (self, 'closure'),
+            'accumulate': (self.opt, '_accumulate'),
+            'ema': (_curv, 'update_ema_all'),
+            'invert': (_curv, 'update_inv_all'),
+            'cholesky': (_curv, 'update_std_all'),
+            'precondition': (_curv, 'precondition_all'),
+            'update': (self.opt, '_fused_update'),
+        })
+        with clock:
+            for _ in range(iters):
+                self.step()
+        return {k: v / iters for k, v in clock.totals_ms().items()}
+
+
+def run_noisy_kfac(args):
+    import torch
+    dev = torch.device('cuda:0')
+    job = NoisyKfacJob(dev)
+    job.step()                     # the first step has no posterior to sample from yet
+    ms, ev_ms, host_ms = time_steps(job.step, args.steps, args.warmup)
+    phases = job.timed_phases(max(2, min(args.steps, 5)))
+    specs = convnet_specs()
+    work = algorithmic_work(specs, 128)
+    flops = {'factor': NoisyKfacJob.MC * work['factor'], 'inverse': work['inverse'],
+             'cholesky': work['inverse'] / 3., 'sample': NoisyKfacJob.MC * work['precondition'],
+             'precondition': work['precondition']}
+    info = [g['curv'].info for g in job.opt.param_groups] + \
+        [g['curv'].std_info for g in job.opt.param_groups]
+    not_spd = int(sum(int((i != 0).sum().item()) for i in info if i is not None))
+    total = sum(flops.values())
+    both = phases['invert'] + phases['cholesky']
+    out = {
+        'metric': METRIC, 'value': round(ms, 4), 'unit': 'ms', 'n_gpus': 1,
+        'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms, 4),
+        'higher_is_better': False, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'f32', 'data': 'synthetic',
+        'config': {'workload': 'noisy_kfac_convnet_batch128_mc4 (BASELINE config 5)', 'batch': 128,
+                   'kron_layers': 5, 'num_mc_samples': NoisyKfacJob.MC, 'dataset_size': 50000,
+                   'damping': 1e-3, 'ema_decay': 0.95, 'measured_from_step': 2,
+                   'step_includes': 'forward and backward of the network (torch) for every MC sample'},
+        'tflops': round(total / (ms * 1e-3) / 1e12, 2),
+        'algorithmic_gflop': {k: round(v / 1e9, 2) for k, v in flops.items()},
+        'phases_ms': {k: round(v, 4) for k, v in phases.items()},
+        'phases_tflops': {'invert': round(flops['inverse'] / phases['invert'] / 1e9, 2),
+                          'cholesky': round(flops['cholesky'] / phases['cholesky'] / 1e9, 2),
+                          'sample': round(flops['sample'] / phases['sample'] / 1e9, 2),
+                          'precondition': round(flops['precondition'] / phases['precondition'] / 1e9, 2)},
+        'host_enqueue_ms': round(host_ms, 4),
+        'not_spd_factors': not_spd,
+        'roofline': {'bound': 'mfma',
+                     'kernel': 'pi-damped inversion + Cholesky factors of the inverses, all layers '
+                               '(potrf_*, trtri_*, lauum kernels)',
+                     'achieved': round((flops['inverse'] + flops['cholesky']) / both / 1e9, 2),
+                     'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': round((flops['inverse'] + flops['cholesky']) / both / 1e9
+                                   / PEAK_FP32_MFMA_TFLOPS, 4),
+                     'traffic': None},
+    }
+    return out
+
+
+# ---------------------------------------------------------------------------
+# a real training step: ResNet-50 forward + backward + K-FAC step (and plain SGD beside it)
+# ---------------------------------------------------------------------------
+
+def run_resnet50_train(args):
+    """Whole training steps of the ResNet-50 itself (torch modules, batch 32, 224x224, fp32):
+    forward, backward with the factor products in the hooks, SecondOrderOptimizer.step with
+    every factor inverted every step; beside it the same network under torch.optim.SGD.
+    What the optimizer adds to a step is the difference."""
+    import torch
+    import torch.nn.functional as F
+    import torchsso
+    dev = torch.device('cuda:0')
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(32, 3, 224, 224, generator=gen).to(dev)
+    y = torch.randint(0, 1000, (32,), generator=gen).to(dev)
+
+    torch.manual_seed(1)
+    model = build_resnet50().to(dev)
+    sgd = torch.optim.SGD(model.parameters(), lr=1e-3, momentum=0.9)
+
+    def sgd_step():
+        sgd.zero_grad()
+        F.cross_entropy(model(x), y).backward()
+        sgd.step()
+    sgd_ms, _, _ = time_steps(sgd_step, args.steps, args.warmup)
+    del sgd, model
+
+    torch.manual_seed(1)
+    model = build_resnet50().to(dev)
+    opt = torchsso.optim.SecondOrderOptimizer(
+        model, 'Cov', {'Conv2d': 'Kron', 'Linear': 'Kron', 'BatchNorm2d': 'Diag'},
+        {'damping': 1e-3, 'ema_decay': 0.95}, lr=1e-3, momentum=0.9)
+
+    def closure():
+        opt.zero_grad()
+        out = model(x)
+        loss = F.cross_entropy(out, y)
+        loss.backward()
+        return loss, out
+    ms, ev_ms, host_ms = time_steps(lambda: opt.step(closure=closure), args.steps, args.warmup)
+    info = torch.cat([g['curv'].info for g in opt.param_groups if g['curv'].kind == 'kron'])
+    work = algorithmic_work(resnet50_specs(), 32)
+    total = work['factor'] + work['inverse'] + work['precondition']
+    return {
+        'metric': 'ResNet-50 training step ms with the K-FAC step inside (forward + backward + '
+                  'factor + invert + precondition + update), 1 MI355X',
+        'value': round(ms, 4), 'unit': 'ms', 'n_gpus': 1, 'steps': args.steps,
+        'warmup': args.warmup, 'ms_per_step': round(ms, 4), 'higher_is_better': False,
+        'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
+        'config': {'workload': 'resnet50_training_step_batch32_224x224 (real activations)',
+                   'batch': 32, 'invert_every_step': True,
+                   'factor_side_streams': torchsso.factor_streams()},
+        'sgd_step_ms': round(sgd_ms, 4), 'kfac_overhead_ms': round(ms - sgd_ms, 4),
+        'kfac_algorithmic_tflops_over_the_overhead': round(total / ((ms - sgd_ms) * 1e-3) / 1e12, 2),
+        'host_enqueue_ms': round(host_ms, 4),
+        'not_spd_factors': int((info != 0).sum().item()),
+    }
 
 
 # ---------------------------------------------------------------------------
@@ -278,13 +597,16 @@ def run_gpu(args, specs, batch):
 # ---------------------------------------------------------------------------
 
 def run_cpu_baseline(specs, batch, budget_s=30.0):
-    """Times the oracle on one layer of every distinct shape and weighs each by
-    how often that shape occurs in the workload (bounded sample of the same
-    step).  Largest shapes first; stops adding shapes when the budget is spent
-    and scales the remainder by algorithmic flops."""
+    """Times the oracle on one layer of every distinct shape and weighs each by how often
+    that shape occurs in the workload (a bounded sample of the same step).  Largest shapes
+    first; the shapes that carry the first 80 % of the step's algorithmic flops get one
+    untimed warm-up run and the median of two timed ones, the rest one timed run; shapes the
+    budget does not reach are scaled in by flops.  Threads: the job's share of the host
+    (OMP_NUM_THREADS where the environment sets it, else every core)."""
     import torch
     from oracle import kfac_oracle as O
-    threads = int(os.environ.get('OMP_NUM_THREADS', '0')) or min(os.cpu_count() or 1, 16)
+    cores = os.cpu_count() or 1
+    threads = int(os.environ.get('OMP_NUM_THREADS', '0')) or cores
     torch.set_num_threads(threads)
     groups = {}
     for s in specs:
@@ -298,16 +620,37 @@ def run_cpu_baseline(specs, batch, budget_s=30.0):
         return 2. * (dA * dA + dG * dG) * L + 2. * (float(dA) ** 3 + float(dG) ** 3) \
             + 2. * dG * dA * (dA + dG)
 
+    def one_layer(s, x, g, gw, gb):
+        if s['kind'] == 'bn':
+            w, b = torch.rand(s['c']) + 0.5, torch.randn(s['c'])
+            xhat = O.bn_restore_input(x, w, b)
+            data = O.bn_diag(xhat, g, True)
+            ema = O.ema_update(data, [d.clone() for d in data], 0.95)
+            inv = [O.diag_inverse(e, 1e-3) for e in ema]
+            return [i * torch.ones_like(i) for i in inv]
+        if s['kind'] == 'conv':
+            A = O.factor_conv_a(x, (s['k'], s['k']), (s['stride'],) * 2, (s['pad'],) * 2,
+                                (1, 1), s['bias'])
+            G = O.factor_conv_g(g)
+        else:
+            A = O.factor_linear_a(x, s['bias'])
+            G = O.factor_linear_g(g)
+        ema = O.ema_update([A, G], [A.clone(), G.clone()], 0.95)
+        Ai, Gi = O.pi_damped_inverse(ema[0], ema[1], 1e-3)
+        pw, pb = O.precondition(Gi, Ai, gw, gb)
+        return O.sgd_tail(torch.zeros_like(pw), pw, torch.zeros_like(pw), 1e-3, 0.9, 0.)
+
     order = sorted(groups.values(), key=lambda sc: -flops(sc[0]))
     total_flops = sum(flops(s) * c for s, c in order)
     done_flops = 0.
     total_s = 0.
     spent = 0.
-    measured = 0
+    measured = repeated = 0
     torch.manual_seed(0)
     for s, count in order:
         if spent > budget_s:
             break
+        gw = gb = None
         if s['kind'] == 'conv':
             x = torch.randn(batch, s['cin'], s['hin'], s['hin'])
             g = torch.randn(batch, s['cout'], s['hout'], s['hout']) * 1e-2
@@ -315,45 +658,42 @@ def run_cpu_baseline(specs, batch, budget_s=30.0):
             gb = torch.randn(s['cout']) * 1e-2 if s['bias'] else None
         elif s['kind'] == 'linear':
             x = torch.randn(batch, s['fin'])
+            if s.get('relu_input', False):
+                x.clamp_(min=0)
             g = torch.randn(batch, s['fout']) * 1e-2
             gw = torch.randn(s['fout'], s['fin']) * 1e-2
             gb = torch.randn(s['fout']) * 1e-2 if s['bias'] else None
         else:
             x = torch.randn(batch, s['c'], s['h'], s['h'])
             g = torch.randn(batch, s['c'], s['h'], s['h']) * 1e-2
-        t0 = time.perf_counter()
-        if s['kind'] == 'bn':
-            w, b = torch.rand(s['c']) + 0.5, torch.randn(s['c'])
-            xhat = O.bn_restore_input(x, w, b)
-            data = O.bn_diag(xhat, g, True)
-            ema = O.ema_update(data, [d.clone() for d in data], 0.95)
-            inv = [O.diag_inverse(e, 1e-3) for e in ema]
-            _ = [i * torch.ones_like(i) for i in inv]
-        else:
-            if s['kind'] == 'conv':
-                A = O.factor_conv_a(x, (s['k'], s['k']), (s['stride'],) * 2, (s['pad'],) * 2,
-                                    (1, 1), s['bias'])
-                G = O.factor_conv_g(g)
-            else:
-                A = O.factor_linear_a(x, s['bias'])
-                G = O.factor_linear_g(g)
-            ema = O.ema_update([A, G], [A.clone(), G.clone()], 0.95)
-            Ai, Gi = O.pi_damped_inverse(ema[0], ema[1], 1e-3)
-            pw, pb = O.precondition(Gi, Ai, gw, gb)
-            O.sgd_tail(torch.zeros_like(pw), pw, torch.zeros_like(pw), 1e-3, 0.9, 0.)
-        dt = time.perf_counter() - t0
-        spent += dt
+        heavy = done_flops < 0.8 * total_flops
+        times = []
+        for rep in range(3 if heavy else 1):
+            t0 = time.perf_counter()
+            one_layer(s, x, g, gw, gb)
+            dt = time.perf_counter() - t0
+            spent += dt
+            if not (heavy and rep == 0):     # the first run of a heavy shape is the warm-up
+                times.append(dt)
+            if heavy and spent > budget_s and times:
+                break
+        times.sort()
+        dt = times[len(times) // 2] if len(times) % 2 else 0.5 * (times[len(times) // 2 - 1]
+                                                                   + times[len(times) // 2])
         total_s += dt * count
         done_flops += flops(s) * count
         measured += 1
+        repeated += 1 if heavy else 0
     if done_flops < total_flops:      # extrapolate what the budget did not cover
         total_s *= total_flops / done_flops
-    sample = ('%d of %d distinct layer shapes timed once each (largest first, %.0f%% of the '
-              'step\'s algorithmic flops), weighted by multiplicity%s; torch CPU einsum/unfold/mm '
-              '+ scipy.linalg.inv, fp32' % (
+    sample = ('%d of %d distinct layer shapes (largest first, %.0f%% of the step\'s algorithmic '
+              'flops), weighted by multiplicity%s; the %d shapes carrying the first 80%% of the '
+              'flops: warm-up + median of 2, the rest once; torch CPU einsum/unfold/mm + '
+              'scipy.linalg.inv, fp32; %d threads = the job\'s share of a host with %d cores' % (
                   measured, len(order), 100. * done_flops / total_flops,
-                  '' if done_flops >= total_flops else ', rest scaled by flops'))
-    return total_s * 1e3, threads, sample
+                  '' if done_flops >= total_flops else ', rest scaled by flops', repeated,
+                  threads, cores))
+    return total_s * 1e3, cores, threads, sample
 
 
 # ---------------------------------------------------------------------------
@@ -363,7 +703,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workload', default='resnet50', choices=sorted(WORKLOADS))
+    ap.add_argument('--workload', default='resnet50', choices=sorted(WORKLOADS) + ['noisy_kfac', 'resnet50_train'])
     ap.add_argument('--factor-streams', type=int, default=None,
                     help='side streams for the factor products (library default: 3; 0 = none)')
     ap.add_argument('--no-cpu-baseline', action='store_true')
@@ -376,13 +716,6 @@ def main():
               '(no collectives are part of this build)', file=sys.stderr)
         sys.exit(2)
 
-    make, batch, label = WORKLOADS[args.workload]
-    specs = make()
-    if args.workload == 'alexnet_fc':
-        for s in specs:
-            s['relu_input'] = True
-    work = algorithmic_work(specs, batch)
-
     import torch
     if not torch.cuda.is_available():
         print('no HIP device visible', file=sys.stderr)
@@ -391,7 +724,37 @@ def main():
     if args.factor_streams is not None:
         torchsso.set_factor_streams(args.factor_streams)
     factor_streams = torchsso.factor_streams()
-    ms, ev_ms, phases, resident, not_spd = run_gpu(args, specs, batch)
+
+    if args.workload == 'resnet50_train':
+        print(json.dumps(run_resnet50_train(args)))
+        return
+    if args.workload == 'noisy_kfac':
+        out = run_noisy_kfac(args)
+        out['config']['factor_side_streams'] = factor_streams
+        if not args.no_cpu_baseline:
+            # the same step on the host: 4 x factors + inverse + Cholesky + 4 x sampling products
+            specs = convnet_specs()
+            cpu_ms, cores, threads, sample = run_cpu_baseline(specs, 128)
+            out['cpu_baseline'] = {
+                'value': round(cpu_ms, 1), 'unit': 'ms', 'cores': cores, 'threads': threads,
+                'kind': 'port',
+                'sample': 'ONE factor build + inversion + preconditioning of the same layers '
+                          '(config 2\'s K-FAC step, a lower bound for the Noisy K-FAC step, which '
+                          'builds the factors 4 times and adds the Cholesky factors and 4 '
+                          'sampling products; the reference has no CPU Cholesky at all, '
+                          'utils/cholesky_cupy.py is CuPy only); ' + sample}
+        print(json.dumps(out))
+        return
+
+    make, batch, label = WORKLOADS[args.workload]
+    specs = make()
+    if args.workload == 'alexnet_fc':
+        for s in specs:
+            s['relu_input'] = True
+    work = algorithmic_work(specs, batch)
+    executed = factor_executed_flops(specs, batch)
+
+    ms, ev_ms, host_ms, phases, resident, not_spd = run_gpu(args, specs, batch)
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device='cuda:0').normal_()
         dst = torch.empty_like(src)
@@ -421,26 +784,41 @@ def main():
         'phases_tflops': {'factor': round(work['factor'] / f_ms / 1e9, 2),
                           'invert': round(work['inverse'] / inv_ms / 1e9, 2),
                           'precondition': round(work['precondition'] / pre_ms / 1e9, 2)},
+        'host_enqueue_ms': round(host_ms, 4),
         'not_spd_factors': not_spd,
         'roofline': {'bound': 'mfma',
                      'kernel': 'Kronecker factor build, all layers (syrk_kernel, corr_kernel)',
                      'achieved': round(work['factor'] / f_ms / 1e9, 2),
                      'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
                      'frac': round(work['factor'] / f_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4),
-                     'traffic': RESNET50_FACTOR_TRAFFIC_BYTES if args.workload == 'resnet50' else None,
+                     'traffic': None,
                      'note': 'achieved counts the algorithmic flops 2*d^2*L of every factor (dense '
                              'convention); the kernels execute fewer (one triangle of each symmetric '
                              'product, shared spatial correlations for stride-1 kxk convolutions), so '
-                             'frac can exceed 1; executed_* is what the matrix cores really do'},
+                             'frac can exceed 1; executed_* prices what the matrix cores really do, '
+                             'derived from the library\'s tile / split plan',
+                     'executed_gflop': round(executed / 1e9, 1),
+                     'executed_tflops': round(executed / f_ms / 1e9, 2),
+                     'executed_frac': round(executed / f_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)},
     }
     if args.workload == 'resnet50':
-        ex = RESNET50_FACTOR_EXECUTED_FLOP / f_ms / 1e9
-        out['roofline']['executed_tflops'] = round(ex, 2)
-        out['roofline']['executed_frac'] = round(ex / PEAK_FP32_MFMA_TFLOPS, 4)
+        pmc = read_pmc_summary()
+        seen = pmc.get('executed_flop_per_step_pmc')
+        if seen and abs(executed - seen) <= 0.03 * seen:
+            out['roofline']['traffic'] = pmc.get('traffic_bytes_per_launch')
+            out['roofline']['executed_gflop_pmc'] = round(seen / 1e9, 1)
+        else:
+            msg = ('the factor plan executes %.1f GFLOP per step but the counter summary %s was '
+                   'taken at %s: the plan changed since, traffic and the PMC cross-check are '
+                   'left out until the counters are read again'
+                   % (executed / 1e9, os.path.relpath(PMC_SUMMARY, ROOT),
+                      'no reading' if not seen else '%.1f GFLOP' % (seen / 1e9)))
+            print('bench.py: WARNING: ' + msg, file=sys.stderr)
+            out['roofline']['pmc_check'] = 'STALE: ' + msg
     if not args.no_cpu_baseline:
-        cpu_ms, cores, sample = run_cpu_baseline(specs, batch)
+        cpu_ms, cores, threads, sample = run_cpu_baseline(specs, batch)
         out['cpu_baseline'] = {'value': round(cpu_ms, 1), 'unit': 'ms', 'cores': cores,
-                               'kind': 'port', 'sample': sample}
+                               'threads': threads, 'kind': 'port', 'sample': sample}
         out['speedup_vs_cpu'] = round(cpu_ms / ms, 1)
     print(json.dumps(out))
 

@@ -80,6 +80,17 @@ int kfac_factor_conv_a(const float* x, int n, int c, int H, int W,
                        int add_bias, float alpha, float beta, const float* C_prev, float* C,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* Plan queries (no device needed): the fp32 MFMA flops the factor builders execute for a
+ * d x d factor reduced over K terms (kfac_factor_linear, kfac_factor_conv_g and the
+ * pointwise case of kfac_factor_conv_a) and for a Conv2d input factor of the given
+ * geometry: whole tiles of the upper triangle, whole reduction chunks, the shared spatial
+ * correlations of a stride-1 k x k layer.  For utilisation figures next to the
+ * algorithmic 2*d*d*K. */
+double kfac_factor_executed_flops(int d, int64_t K);
+double kfac_factor_conv_a_executed_flops(int n, int c, int H, int W, int kh, int kw,
+                                         int sh, int sw, int ph, int pw, int dh, int dw,
+                                         int add_bias);
+
 /* C = alpha * m m^T + beta * C_prev with m = g viewed as [c, n*h*w]; g is
  * [n, c, h, w] and is read in place (no transpose copy).
  * Replaces torchsso/curv/cov/conv.py:69-74 plus the n^2 rescale of

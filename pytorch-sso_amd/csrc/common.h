@@ -28,6 +28,8 @@ bool enable_large_lds(const void* kernel, int bytes);
 bool conv_a_taps_applicable(int c, int kh, int kw, int sh, int sw, int add_bias);
 size_t conv_a_taps_workspace(int n, int c, int H, int W, int kh, int kw, int ph, int pw, int dh,
                              int dw);
+double conv_a_taps_executed_flops(int n, int c, int H, int W, int kh, int kw, int ph, int pw,
+                                  int dh, int dw);   // 0 when the geometry is not covered
 int conv_a_taps(const float* x, int n, int c, int H, int W, int kh, int kw, int ph, int pw, int dh,
                 int dw, float alpha, float beta, const float* A_prev, float* A, void* workspace,
                 size_t workspace_bytes, hipStream_t stream);

@@ -309,6 +309,51 @@ static int64_t slice_len(int64_t total, int64_t elems_per_unit) {
   return max_units < 1 ? 0 : (total < max_units ? total : max_units);
 }
 
+// MFMA flops one launch_syrk executes: every (tile, split) workgroup runs whole chunks of
+// KC reduction steps on a full ts x ts tile (padding and the k tail included).
+static double syrk_executed_flops(int d, int64_t K) {
+  const SyrkPlan p = plan_syrk(d, (long)K);
+  const int kc = p.w == 1 ? Cfg<1, 1>::KC : Cfg<2, 2>::KC;
+  const double chunks = (double)((K + kc - 1) / kc);
+  return (double)p.ntiles * chunks * kc * 2.0 * p.ts * p.ts;
+}
+
+double kfac_factor_executed_flops(int d, int64_t K) {
+  if (d <= 0 || K <= 0) return 0.;
+  return syrk_executed_flops(d, K);
+}
+
+double kfac_factor_conv_a_executed_flops(int n, int c, int H, int W, int kh, int kw, int sh,
+                                         int sw, int ph, int pw, int dh, int dw, int add_bias) {
+  if (n <= 0 || c <= 0 || H <= 0 || W <= 0 || kh <= 0 || kw <= 0 || sh <= 0 || sw <= 0 ||
+      ph < 0 || pw < 0 || dh <= 0 || dw <= 0)
+    return 0.;
+  const int OH = (H + 2 * ph - dh * (kh - 1) - 1) / sh + 1;
+  const int OW = (W + 2 * pw - dw * (kw - 1) - 1) / sw + 1;
+  if (OH <= 0 || OW <= 0) return 0.;
+  const int64_t image = (int64_t)c * H * W;
+  const int64_t step = slice_len(n, image);
+  if (step == 0) return 0.;
+  const int d = c * kh * kw + (add_bias ? 1 : 0);
+  double total = 0.;
+  for (int64_t n0 = 0; n0 < n; n0 += step) {
+    const int cnt = (int)(n - n0 < step ? n - n0 : step);
+    if (kh == 1 && kw == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && !add_bias) {
+      total += syrk_executed_flops(d, (int64_t)cnt * H * W);
+      continue;
+    }
+    if (conv_a_taps_applicable(c, kh, kw, sh, sw, add_bias)) {
+      const double t = conv_a_taps_executed_flops(cnt, c, H, W, kh, kw, ph, pw, dh, dw);
+      if (t > 0.) {
+        total += t;
+        continue;
+      }
+    }
+    total += syrk_executed_flops(d, (int64_t)cnt * OH * OW);
+  }
+  return total;
+}
+
 size_t kfac_factor_conv_a_workspace_bytes(int n, int c, int H, int W, int kh, int kw, int sh,
                                           int sw, int ph, int pw, int dh, int dw, int add_bias) {
   if (n <= 0 || c <= 0 || H <= 0 || W <= 0 || kh <= 0 || kw <= 0 || sh <= 0 || sw <= 0 ||

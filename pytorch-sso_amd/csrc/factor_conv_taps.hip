@@ -378,6 +378,24 @@ size_t conv_a_taps_workspace(int n, int c, int H, int W, int kh, int kw, int ph,
   return hp.ok ? hp.partial_floats * sizeof(float) : 0;
 }
 
+// MFMA flops corr_kernel executes for this geometry: whole chunks on full tiles, for every
+// (job, split, tile) work item.
+double conv_a_taps_executed_flops(int n, int c, int H, int W, int kh, int kw, int ph, int pw,
+                                  int dh, int dw) {
+  const TapPlanHost hp = plan_taps(n, c, H, W, kh, kw, ph, pw, dh, dw);
+  if (!hp.ok) return 0.;
+  const int ts = 64 * hp.w;
+  const int kc = hp.w == 1 ? Cfg<1, 1>::KC : Cfg<2, 2>::KC;
+  const double ntiles = (double)hp.tiles_side * hp.tiles_side;
+  double total = 0.;
+  for (int j = 0; j < hp.dev.njobs; ++j) {
+    const JobDesc& jd = hp.dev.jobs[j];
+    const long K = (long)n * jd.hh * jd.ww;
+    total += ntiles * (double)((K + kc - 1) / kc) * kc * 2.0 * ts * ts;
+  }
+  return total;
+}
+
 // returns KFAC_OK, an error, or -1 when the geometry is not covered (the caller
 // then uses the im2col kernel)
 int conv_a_taps(const float* x, int n, int c, int H, int W, int kh, int kw, int ph, int pw, int dh,

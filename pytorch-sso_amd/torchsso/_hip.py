@@ -38,6 +38,8 @@ _SIGNATURES = {
     'kfac_abi_version': (c_int, []),
     'kfac_factor_workspace_bytes': (c_size, [c_int, c_i64]),
     'kfac_factor_conv_a_workspace_bytes': (c_size, [c_int] * 13),
+    'kfac_factor_executed_flops': (ctypes.c_double, [c_int, c_i64]),
+    'kfac_factor_conv_a_executed_flops': (ctypes.c_double, [c_int] * 13),
     'kfac_factor_linear': (c_int, [c_ptr, c_i64, c_int, c_i64, c_int, c_f32, c_f32, c_ptr, c_ptr,
                                    c_ptr, c_size, c_ptr]),
     'kfac_factor_conv_a': (c_int, [c_ptr] + [c_int] * 13 + [c_f32, c_f32, c_ptr, c_ptr,
