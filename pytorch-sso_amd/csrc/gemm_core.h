@@ -122,8 +122,10 @@ struct Stager {
   float regs[CNT];
   unsigned onebits;    // element i is the constant 1 (and inside the k range)
 
+  // (thread index within a group of NT threads: a workgroup may hold several groups,
+  // each computing a tile of its own)
   __device__ __forceinline__ void init(const OP& op, int m0) {
-    const int t = threadIdx.x;
+    const int t = threadIdx.x & (NT - 1);
     if (OP::layout == KM) {
       ms[0] = op.mstate(m0 + (t % ROWS));
     } else {
@@ -137,7 +139,7 @@ struct Stager {
   // k range come back as 0 from the hardware's range check; the loaded values
   // are not touched until commit, so nothing here waits on memory.
   __device__ __forceinline__ void fetch(const OP& op, int k0, int kend) {
-    const int t = threadIdx.x;
+    const int t = threadIdx.x & (NT - 1);
     const __amdgpu_buffer_rsrc_t rs = op.rsrc();
     unsigned oneb = 0;
     if (OP::layout == KM) {
@@ -166,7 +168,7 @@ struct Stager {
   }
 
   __device__ __forceinline__ void commit(lds_f* tile) const {
-    const int t = threadIdx.x;
+    const int t = threadIdx.x & (NT - 1);
 #pragma unroll
     for (int i = 0; i < CNT; ++i) {
       float v = ((onebits >> i) & 1u) ? 1.f : regs[i];
@@ -233,7 +235,7 @@ template <int WM, int WN>
 __device__ __forceinline__ void acc_coords(int m0, int n0, int a, int b, int i, int& row,
                                            int& col) {
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = (threadIdx.x & (64 * WM * WN - 1)) >> 6;
   const int r = lane & 31, h = lane >> 5;
   row = m0 + (wave / WN) * 64 + 32 * a + 8 * (i >> 2) + 4 * h + (i & 3);
   col = n0 + (wave % WN) * 64 + 32 * b + r;
@@ -244,7 +246,7 @@ __device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0
                                               int kbeg, int kend, bool same, EPI& epi,
                                               float* smem) {
   typedef Cfg<WM, WN> C;
-  const int t = threadIdx.x;
+  const int t = threadIdx.x & (C::NT - 1);
   const int lane = t & 63;
   const int wave = t >> 6;
   const int r = lane & 31;
@@ -403,9 +405,9 @@ struct WorkList {
   int cum[WL_MAX + 1];
 };
 
-// matrix (table index) and local work item of the calling workgroup
-__device__ __forceinline__ void work_find(const WorkList& wl, int& mat, int& local) {
-  const int item = blockIdx.x;
+// matrix (table index) and local work item of work item `item` of the list
+__device__ __forceinline__ void work_find_item(const WorkList& wl, int item, int& mat,
+                                               int& local) {
   int lo = 0, hi = wl.n;
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
@@ -413,6 +415,11 @@ __device__ __forceinline__ void work_find(const WorkList& wl, int& mat, int& loc
   }
   mat = wl.first + lo;
   local = item - wl.cum[lo];
+}
+
+// ... of the calling workgroup, in a launch whose grid is the list
+__device__ __forceinline__ void work_find(const WorkList& wl, int& mat, int& local) {
+  work_find_item(wl, (int)blockIdx.x, mat, local);
 }
 
 // tile index t (0-based, row-major over the upper triangle incl. diagonal of a

@@ -7,7 +7,12 @@
 //   2. blocked right-looking Cholesky  S = U^T U  (upper, in place in dst) with
 //      128-wide panels: one workgroup factors AND inverts the 128x128 diagonal
 //      block in LDS; the row panel is a product with that small inverse; the
-//      trailing update is a symmetric rank-128 product on the MFMA tile engine;
+//      trailing update is a symmetric rank-128 product on the MFMA tile engine.
+//      Panels are grouped: the rows of the current group receive each panel's
+//      update at once (the next row before anything else, the others from tile
+//      workgroups that share a launch with the next diagonal block, so that the
+//      chip is not idle while that latency-bound block is factored), the rows
+//      beyond the group receive the whole group in one deeper product;
 //   3. Y = U^-1 by recursive doubling over the 128-blocks:
 //      Y12 = -Y11 * U12 * Y22, two MFMA products per level, log2(n/128) levels;
 //   4. dst = Y Y^T on the MFMA tile engine (upper tiles, mirrored).
@@ -313,12 +318,12 @@ __device__ __forceinline__ void tri_pair(const lds_f* S, lds_f* Yb, lds_f* Wt, i
   __syncthreads();
 }
 
-__global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, int p, int* info) {
-  extern __shared__ __attribute__((aligned(16))) float dsm[];
+// Factors and inverts diagonal block p of matrix m (one workgroup of 256 threads with
+// DIAG_SMEM_BYTES of LDS at dsm).
+__device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, float* dsm) {
   lds_f* const S = (lds_f*)dsm;
   lds_f* const Yb = S + DB * DLD;
   lds_f* const Wt = S + 2 * DB * DLD;
-  const MatDesc m = table[blockIdx.x];
   const int n = m.n;
   const int r0 = p * DB;
   const int nb = min(DB, n - r0);
@@ -431,6 +436,11 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, i
   }
 }
 
+__global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, int p, int* info) {
+  extern __shared__ __attribute__((aligned(16))) float dsm[];
+  diag_block(table[blockIdx.x], p, info, dsm);
+}
+
 // row panel of the blocked Cholesky: U[p, j] = Ypp^T * A[p, j], j > p
 __global__ __launch_bounds__(NTHREADS) void potrf_panel_kernel(const MatDesc* table, int p,
                                                                const WorkList wl) {
@@ -472,11 +482,17 @@ __device__ __forceinline__ bool trail_tile(int T, int row_lo, int row_hi, int lo
 
 // trailing update with the block rows [kb0, kb0 + nk) of U:
 //   A[i, j] -= sum_k U[k, i]^T U[k, j]   for block rows row_lo <= i < row_hi, j >= i.
-// The Cholesky runs in outer panels of OUTER_BLOCKS diagonal blocks: inside an
-// outer panel each step updates only the remaining rows of that panel (nk = 1),
-// and the rows beyond it receive the whole panel at once (nk = OUTER_BLOCKS),
-// which cuts the read-modify-write passes over the trailing matrix by that factor.
-constexpr int OUTER_BLOCKS = 4;
+// The Cholesky runs in groups of GROUP_BLOCKS diagonal blocks: inside a group each step
+// updates only the remaining rows of that group (nk = 1), and the rows beyond it receive
+// the whole group at once (nk = GROUP_BLOCKS), which cuts the read-modify-write passes over
+// the trailing matrix by that factor (a rank-128 update of a large trailing matrix is
+// bound by memory traffic, not by the matrix cores).  Taller groups run no faster (measured
+// up to 16: the tiles that ride along with a diagonal block are hidden either way) and
+// cost accuracy: the float32 error of the inverse of a 9217^2 factor with condition number
+// 9e2 grows from 2.2e-5 (height 1) over 5.2e-5 (4; scipy's float32 LU inverse: 4.7e-5) to
+// 1.0e-4 (16), because a deeper product accumulates more terms before it meets the
+// entry it nearly cancels.
+constexpr int GROUP_BLOCKS = 4;
 
 __global__ __launch_bounds__(NTHREADS, 3) void potrf_trail_kernel(const MatDesc* table, int kb0,
                                                                int nk, int row_lo, int row_hi,
@@ -491,6 +507,32 @@ __global__ __launch_bounds__(NTHREADS, 3) void potrf_trail_kernel(const MatDesc*
   DenseKM P{m.U + (size_t)kb0 * DB * n, nullptr, n, n, 0};
   EpiStore epi{m.U, n, n, n, -1.f, 1.f, false};
   gemm_tile(P, P, bi * BM, bj * BN, 0, nk * DB, bi == bj, epi, smem);
+}
+
+// Diagonal blocks p and, beside them, the part of panel p-1's update that nothing needs
+// before the next row panel:   A[i,j] -= U[p-1,i]^T U[p-1,j]   for block rows
+// row_lo <= i < row_hi (row_lo = p + 1: row p got its update in a launch of its own).
+// The first `ndiag` workgroups take one diagonal block each (potrf_diag_kernel's work),
+// the others one tile each.  The launch carries the diagonal block's LDS, so one
+// workgroup runs per CU: the tile workgroups use the CUs that the few diagonal blocks
+// leave idle, for about as long as a diagonal block takes.
+__global__ __launch_bounds__(NTHREADS) void potrf_step_kernel(const MatDesc* table, int p,
+                                                              int* info, int ndiag, int row_lo,
+                                                              int row_hi, const WorkList wl) {
+  extern __shared__ __attribute__((aligned(16))) float dsm[];
+  if ((int)blockIdx.x < ndiag) {
+    diag_block(table[blockIdx.x], p, info, dsm);
+    return;
+  }
+  int mat, local;
+  work_find_item(wl, (int)blockIdx.x - ndiag, mat, local);
+  const MatDesc m = table[mat];
+  int bi, bj;
+  if (!trail_tile(m.T, row_lo, row_hi, local, bi, bj)) return;
+  const int n = m.n;
+  DenseKM P{m.U + (size_t)(p - 1) * DB * n, nullptr, n, n, 0};
+  EpiStore epi{m.U, n, n, n, -1.f, 1.f, false};
+  gemm_tile(P, P, bi * BM, bj * BN, 0, DB, bi == bj, epi, dsm);
 }
 
 // The row panel (near == 0) or the near update with one block row (near == 1) for
@@ -882,6 +924,7 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
 
   // kernels that need more than the default 64 KiB of LDS (registered once per process)
   if (!enable_large_lds((const void*)potrf_diag_kernel, DIAG_SMEM_BYTES) ||
+      !enable_large_lds((const void*)potrf_step_kernel, DIAG_SMEM_BYTES) ||
       !enable_large_lds((const void*)potrf_fine_kernel, FINE_SMEM_BYTES) ||
       !enable_large_lds((const void*)potrf_sub_kernel<2, 2>, SUB_SMEM_BYTES) ||
       !enable_large_lds((const void*)potrf_sub_kernel<4, 1>, SUB_SMEM_BYTES))
@@ -952,19 +995,32 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
     hipLaunchKernelGGL(inv_copy_damp_kernel, dim3(grid), dim3(256), 0, stream, table, info, wl);
   });
 
-  for (int P0 = 0; P0 < Tmax; P0 += OUTER_BLOCKS) {
-    const int Pend = std::min(P0 + OUTER_BLOCKS, Tmax);
+  for (int P0 = 0, Pend = 0; P0 < Tmax; P0 = Pend) {
+    Pend = std::min(P0 + GROUP_BLOCKS, Tmax);
+    auto total_items = [&](int count, auto&& items) {
+      long sum = 0;
+      for (int i = 0; i < count; ++i) sum += std::max(0, (int)items(Ts[i]));
+      return sum;
+    };
     for (int p = P0; p < Pend; ++p) {
       const int na = active(p + 1);
-      hipLaunchKernelGGL(potrf_diag_kernel, dim3(na), dim3(256), DIAG_SMEM_BYTES, stream, table,
-                         p, info);
+      // diagonal block p; beside it, panel p-1's update of the group's rows beyond p
+      // (rows p+1 .. Pend-1; row p got it right after panel p-1)
+      auto rest_items = [&](int T) { return (std::min(Pend, T) - p - 1) * (T - p - 1); };
+      if (p == P0 || total_items(na, rest_items) == 0) {
+        hipLaunchKernelGGL(potrf_diag_kernel, dim3(na), dim3(256), DIAG_SMEM_BYTES, stream,
+                           table, p, info);
+      } else {
+        bool first = true;
+        for_worklists(na, rest_items, [&](const WorkList& wl, int grid) {
+          const int nd = first ? na : 0;
+          first = false;
+          hipLaunchKernelGGL(potrf_step_kernel, dim3(nd + grid), dim3(NTHREADS), DIAG_SMEM_BYTES,
+                             stream, table, p, info, nd, p + 1, Pend, wl);
+        });
+      }
       const int nb = active(p + 2);
       if (nb == 0) continue;
-      auto total_items = [&](int count, auto&& items) {
-        long sum = 0;
-        for (int i = 0; i < count; ++i) sum += std::max(0, (int)items(Ts[i]));
-        return sum;
-      };
       auto panel_items = [&](int T) { return T - p - 1; };
       if (total_items(nb, panel_items) <= SUB_MAX_TILES) {
         for_worklists(nb, [&](int T) { return 4 * std::max(0, panel_items(T)); },
@@ -981,24 +1037,25 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
           KFAC_LAUNCH_TILE2(potrf_panel_kernel, dim3(grid), stream, table, p, wl);
       });
       if (p + 1 < Pend) {
-        // rows (p, Pend) of the outer panel, all columns to the right
-        auto near_items = [&](int T) { return (std::min(Pend, T) - p - 1) * (T - p - 1); };
-        if (total_items(nb, near_items) <= SUB_MAX_TILES) {
-          for_worklists(nb, [&](int T) { return 4 * std::max(0, near_items(T)); },
+        // panel p's update of block row p+1 (the next diagonal block and row panel need it);
+        // the group's other rows get it beside the next diagonal block
+        auto row_items = [&](int T) { return T > p + 1 ? T - p - 1 : 0; };
+        if (total_items(nb, row_items) <= SUB_MAX_TILES) {
+          for_worklists(nb, [&](int T) { return 4 * std::max(0, row_items(T)); },
                         [&](const WorkList& wl, int grid) {
                           hipLaunchKernelGGL((potrf_sub_kernel<2, 2>), dim3(grid),
                                              dim3(SUB_THREADS), SUB_SMEM_BYTES, stream, table, p,
-                                             1, Pend, wl);
+                                             1, p + 2, wl);
                         });
         } else
-        for_worklists(nb, near_items,
+        for_worklists(nb, row_items,
                       [&](const WorkList& wl, int grid) {
                         if (grid <= FINE_MAX_TILES)
                           hipLaunchKernelGGL(potrf_fine_kernel, dim3(grid), dim3(FINE_THREADS),
-                                             FINE_SMEM_BYTES, stream, table, p, 1, Pend, wl);
+                                             FINE_SMEM_BYTES, stream, table, p, 1, p + 2, wl);
                         else
                           KFAC_LAUNCH_TILE2(potrf_trail_kernel, dim3(grid), stream, table, p, 1,
-                                            p + 1, Pend, wl);
+                                            p + 1, p + 2, wl);
                       });
       }
     }

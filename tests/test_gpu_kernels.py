@@ -353,9 +353,13 @@ def test_large_inverse_at_benchmark_sizes(ops, dev):
     256, rank-deficient before damping).  The error of the float32 result Y is
     measured in float64 on the device through one Newton step,
     Y_true = Y + Y (I - X Y) + O(|I - X Y|^2), and for 4608 also against
-    torch.linalg.inv in float64 (a library routine).  The residual X Y - I of a
-    float32 inverse scales with the condition number (about 7e2 in the second
-    case), so it gets a looser bound."""
+    torch.linalg.inv in float64 (a library routine).  The 9217 matrix has a condition
+    number of about 7e2, where the error of ANY float32 inverse (cond * 2^-24 times a
+    modest factor) sits right at 1e-4: the reference's own float32 result on the same
+    matrix (scipy.linalg.inv, torchsso/utils/inv_cupy.py:32-34, through the oracle) is
+    measured beside it and the bound is 1e-4 or 1.5 x that error, whichever is larger.
+    The residual X Y - I scales with the condition number and gets a looser bound."""
+    from test_gpu_bench_step import inverse_record
     for n, L in [(4608, 1568), (9217, 256)]:
         g = torch.Generator(device='cpu').manual_seed(n)
         x = torch.randn(L, n, generator=g).to(dev)
@@ -364,15 +368,16 @@ def test_large_inverse_at_benchmark_sizes(ops, dev):
         outs, info = ops.damped_inverse_batched([X], [damp])
         assert info.cpu().tolist() == [0]
         Xd = X.double()
+        _, err, err_ref, _ = inverse_record('random rank-%d factor' % L, Xd, damp, outs[0])
         Xd.diagonal().add_(damp)
         Y = outs[0].double()
         R = torch.eye(n, device=dev, dtype=D) - Xd @ Y
-        err = ((Y @ R).norm() / Y.norm()).item()
         res = R.norm().item() / n ** 0.5
-        print('n=%d rel err %.2e residual %.2e' % (n, err, res))
+        print('n=%d rel err %.2e (reference fp32: %.2e) residual %.2e' % (n, err, err_ref, res))
         assert res < 1e-3, (n, res)
-        assert err < TOL, (n, err)
+        assert err <= max(TOL, 1.5 * err_ref), (n, err, err_ref)
         if n == 4608:
+            assert err < TOL
             ref = torch.linalg.inv(Xd)
             assert ((Y - ref).norm() / ref.norm()).item() < TOL
             del ref
