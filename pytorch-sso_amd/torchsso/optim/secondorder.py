@@ -243,15 +243,20 @@ class SecondOrderOptimizer(Optimizer):
     def _accumulate(self, weight):
         """Adds weight * (current gradients, current curvature data) of every group to the
         group's accumulators (reference: secondorder.py:175-182, vi.py:211-220)."""
+        accs, datas = [], []
         for group in self.param_groups:
-            group['acc_grads'].update([p.grad.data for p in group['params']], scale=weight)
+            accs.append(group['acc_grads'])
+            datas.append([p.grad.data for p in group['params']])
             curv = group['curv']
             if curv is not None:
-                group['acc_curv'].update(curv.data, scale=weight)
+                accs.append(group['acc_curv'])
+                datas.append(curv.data)
+        TensorAccumulator.update_many(accs, datas, scale=weight)   # one launch for all layers
 
     def _update_groups(self, groups, target, update_inv, update_std, precondition):
+        self._l2_all(groups, target)        # grad += l2_reg * p, one launch per distinct l2_reg
         for group in groups:
-            self.update_preprocess(group, target=target, grad_type='raw')
+            self.update_preprocess(group, target=target, grad_type='raw', l2_done=True)
 
         curvs = [g['curv'] for g in groups if g['curv'] is not None]
         if curvs:
@@ -330,7 +335,28 @@ class SecondOrderOptimizer(Optimizer):
         if ps:
             _ops.axpby_batched(gs, ps, -group['lr'], 1.)
 
-    def update_preprocess(self, group, target='params', grad_type='raw'):
+    def _l2_all(self, groups, target):
+        """The l2 term of the raw phase for all groups at once (reference:
+        secondorder.py:238-243, per group): grad += l2_reg * p, and the curvature learns
+        the coefficient (it enters the damping through its running average)."""
+        by_coeff = {}
+        for group in groups:
+            if group['l2_reg'] == 0:
+                continue
+            params = [p for p in group[target] if p.grad is not None]
+            for p in params:
+                if p.grad.is_sparse:
+                    raise RuntimeError(
+                        "l2 regularization option is not compatible with sparse gradients")
+            ps, gs = by_coeff.setdefault(group['l2_reg'], ([], []))
+            ps.extend(p.data for p in params)
+            gs.extend(p.grad for p in params)
+            if params and group['curv'] is not None:
+                group['curv'].l2_reg = group['l2_reg']
+        for coeff, (ps, gs) in by_coeff.items():
+            _ops.axpby_batched(ps, gs, coeff, 1.)
+
+    def update_preprocess(self, group, target='params', grad_type='raw', l2_done=False):
         """Gradient transformations before ('raw') and after ('preconditioned')
         preconditioning, in the reference's order (secondorder.py:233-312)."""
         assert grad_type in ['raw', 'preconditioned'], 'Invalid grad type: {}.'.format(grad_type)
@@ -339,7 +365,7 @@ class SecondOrderOptimizer(Optimizer):
             return
         state = self.state
 
-        if grad_type == 'raw' and group['l2_reg'] != 0:
+        if grad_type == 'raw' and group['l2_reg'] != 0 and not l2_done:
             for p in params:
                 if p.grad.is_sparse:
                     raise RuntimeError(

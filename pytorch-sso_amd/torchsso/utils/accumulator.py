@@ -44,6 +44,33 @@ class TensorAccumulator(object):
             return [d * scale for d in data]
         return [a + scale * d for a, d in zip(acc, data)]
 
+    @classmethod
+    def update_many(cls, accumulators, datas, scale=1.):
+        """accumulators[i].update(datas[i], scale) for every i, with ONE batched launch for
+        all HIP tensors of all accumulators (an optimizer step accumulates the gradients
+        and the curvature factors of every layer at once)."""
+        srcs, dsts_new, dsts_old = [], [], []
+        for acc, data in zip(accumulators, datas):
+            acc.check_type(data)
+            as_list = data if isinstance(data, list) else [data]
+            if not as_list[0].is_cuda:
+                acc.update(data, scale)
+                continue
+            src = [d.detach().contiguous() for d in as_list]
+            have = acc._accumulation
+            if have is None:
+                new = [d.new_empty(d.shape) for d in src]
+                acc._accumulation = new if isinstance(data, list) else new[0]
+                srcs.extend(src)
+                dsts_new.extend(new)
+            else:
+                dsts_old.append((src, have if isinstance(have, list) else [have]))
+        if dsts_new:
+            _ops.axpby_batched(srcs, dsts_new, scale, 0.)
+        if dsts_old:
+            _ops.axpby_batched([x for src, _ in dsts_old for x in src],
+                               [y for _, have in dsts_old for y in have], scale, 1.)
+
     def update(self, data, scale=1.):
         self.check_type(data)
         if isinstance(data, list):
