@@ -92,8 +92,11 @@ def test_factors_read_right_after_backward_are_complete():
 
 
 def test_training_steps_match_single_stream_run():
-    """Three optimizer steps of an autograd model, side streams against none.  The
-    network's own kernels are made deterministic, so every bit must agree."""
+    """Three optimizer steps of an autograd model, side streams against none.  The K-FAC
+    kernels give the same bits either way (test above); the network's own backward
+    kernels (MIOpen convolutions) are asked to be deterministic but are not bit-stable
+    across runs on this stack, so the parameters and running averages are compared to
+    1e-6 relative Frobenius, far below anything a misordered stream would leave."""
     dev = torch.device('cuda:0')
     det = torch.backends.cudnn.deterministic
     torch.backends.cudnn.deterministic = True
