@@ -309,8 +309,10 @@ class LayerSet(object):
         self.flat_grad.copy_(self.flat_raw)
 
     def step(self):
-        self.restore_grads()
+        # the factor products go to the side streams first; the copy that stands in for the
+        # backward pass's fresh gradients then runs beside them, as a backward pass would
         self.build_factors()
+        self.restore_grads()
         self.opt.step()
 
     def timed_phases(self, iters):
