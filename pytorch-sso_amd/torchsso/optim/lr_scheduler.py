@@ -51,51 +51,71 @@ class _IterLRScheduler(object):
             group['lr'] = lr
 
 
-class PolynomialDecayIterLR(_IterLRScheduler):
-    """lr = initial_lr * max(1 - (t - start) / (max_count - start), 0) ** rate from
-    iteration `start_iter` on, clipped at `target` when one is given
-    (reference: lr_scheduler.py:51-85)."""
+def polynomial_decay(base_lr, t, rate, max_count, start_iter=0, target=None):
+    """base_lr * max(1 - (t - start) / (max_count - start), 0) ** rate, stopped at `target`
+    when one is given: a decaying schedule (rate > 0) stops at it from above, a growing one
+    (rate <= 0) from below.  Only defined from `start_iter` on."""
+    remaining = max(1 - (t - start_iter) / (max_count - start_iter), 0)
+    lr = base_lr * remaining ** rate
+    if target is None:
+        return lr
+    # (the comparison is made on the quotient, as the reference makes it: a schedule with a
+    # target that decays all the way to 0 raises ZeroDivisionError there too)
+    quotient = target / lr
+    passed = quotient > 1 if rate > 0 else quotient < 1
+    return target if passed else lr
 
-    def __init__(self, optimizer, rate, max_count, target=None, start_iter=0, last_iter=-1):
-        self.rate = rate
-        self.max_count = max_count
-        self.target = target
-        self.start_iter = start_iter
-        super(PolynomialDecayIterLR, self).__init__(optimizer, last_iter)
+
+def linear_warmup(base_lr, t, initial_lr, max_count):
+    """Point t / max_count of the way from `initial_lr` to `base_lr`."""
+    alpha = t / max_count
+    return initial_lr * (1 - alpha) + base_lr * alpha
+
+
+class _FunctionOfIteration(_IterLRScheduler):
+    """A schedule given as a function of (base rate, iteration), active on a range of
+    iterations; outside of it the groups keep the rates they have."""
+
+    def active(self, t):
+        return True
+
+    def rate_at(self, base_lr, t):
+        raise NotImplementedError
 
     def get_lr(self):
         t = self.last_iter
-        if t < self.start_iter:
+        if not self.active(t):
             return self._current()
-        span = self.max_count - self.start_iter
-        decay = max(1 - (t - self.start_iter) / span, 0)
-        lrs = []
-        for base in self.base_lrs:
-            lr = base * decay ** self.rate
-            if self.target is not None:
-                # a decaying schedule (rate > 0) stops at the target from above,
-                # a growing one (rate <= 0) from below
-                ratio = self.target / lr
-                if (self.rate > 0 and ratio > 1) or (self.rate <= 0 and ratio < 1):
-                    lr = self.target
-            lrs.append(lr)
-        return lrs
+        return [self.rate_at(base, t) for base in self.base_lrs]
 
 
-class GradualWarmupIterLR(_IterLRScheduler):
+class PolynomialDecayIterLR(_FunctionOfIteration):
+    """Polynomial decay from iteration `start_iter` on (reference: lr_scheduler.py:51-85)."""
+
+    def __init__(self, optimizer, rate, max_count, target=None, start_iter=0, last_iter=-1):
+        self.rate, self.max_count, self.target, self.start_iter = rate, max_count, target, start_iter
+        super(PolynomialDecayIterLR, self).__init__(optimizer, last_iter)
+
+    def active(self, t):
+        return t >= self.start_iter
+
+    def rate_at(self, base_lr, t):
+        return polynomial_decay(base_lr, t, self.rate, self.max_count, self.start_iter, self.target)
+
+
+class GradualWarmupIterLR(_FunctionOfIteration):
     """Linear ramp from `initial_lr` to the group's own rate over `max_count`
     iterations; unchanged afterwards (reference: lr_scheduler.py:88-108)."""
 
     def __init__(self, optimizer, initial_lr, max_count, last_iter=-1):
-        self.initial_lr = initial_lr
-        self.max_count = max_count
+        self.initial_lr, self.max_count = initial_lr, max_count
         super(GradualWarmupIterLR, self).__init__(optimizer, last_iter)
 
-    def get_lr(self):
-        if self.last_iter > self.max_count:
-            return self._current()
-        alpha = self.last_iter / self.max_count
-        return [self.initial_lr * (1 - alpha) + base * alpha for base in self.base_lrs]
+    def active(self, t):
+        return t <= self.max_count
+
+    def rate_at(self, base_lr, t):
+        return linear_warmup(base_lr, t, self.initial_lr, self.max_count)
 
 
 class MomentumCorrectionLR(object):
