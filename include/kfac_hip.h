@@ -127,6 +127,23 @@ int kfac_pi_damped_inverse_batched(int layers, const int* dA, const int* dG,
                                    float* const* Ainv, float* const* Ginv, int* info,
                                    void* workspace, size_t workspace_bytes, void* stream);
 
+/* kfac_pi_damped_inverse_batched that also delivers, for the layers l with Astd[l] and
+ * Gstd[l] non-NULL (both or neither), the upper Cholesky factors of the two inverses:
+ *   Astd[l]^T Astd[l] = Ainv[l],  Gstd[l]^T Gstd[l] = Ginv[l],  upper triangular, zero below.
+ * Replaces KronCurvature.update_inv followed by update_std, torchsso/curv/curvature.py:302-312
+ * and :317-321 (torchsso.utils.cholesky of each inverse, utils/cholesky_cupy.py:9-14), without
+ * the second factorisation: such a layer's damped factors are factored back to front (rows and
+ * columns reversed, J X J = R^T R), so that X^-1 = J R^-1 R^-T J = W^T W with W = J R^-T J upper
+ * triangular with a positive diagonal -- the Cholesky factor the reference computes from the
+ * inverse -- and W is read off the triangular inverse the inversion forms anyway.  For these
+ * layers a non-zero info[] counts the failing leading minor of the REVERSED matrix. */
+int kfac_pi_damped_inverse_std_batched(int layers, const int* dA, const int* dG,
+                                       const float* const* A, const float* const* G,
+                                       const float* damping,
+                                       float* const* Ainv, float* const* Ginv,
+                                       float* const* Astd, float* const* Gstd, int* info,
+                                       void* workspace, size_t workspace_bytes, void* stream);
+
 /* dst[i] = (src[i] + damp[i]*I)^-1 for `count` symmetric positive definite
  * matrices of sizes dims[i]; damp may be NULL (no shift).  Host arrays as
  * above; info is a DEVICE array of `count` ints.

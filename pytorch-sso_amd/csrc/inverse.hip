@@ -41,10 +41,11 @@ struct MatDesc {
   int is_a;      // pi mode: 1 -> damp*pi, 0 -> damp/pi
   int out;       // position in the caller's info array
   float trace;
-  int pad;
+  int rev;       // 1: the work matrix is src with rows and columns reversed (see run_batched)
+  float* W;      // rev only: receives the upper Cholesky factor of the inverse, else nullptr
 };
 
-constexpr int SETUP_CHUNK = 64;
+constexpr int SETUP_CHUNK = 48;
 struct DescChunk {
   MatDesc d[SETUP_CHUNK];
 };
@@ -98,7 +99,8 @@ __global__ __launch_bounds__(256) void inv_copy_damp_kernel(const MatDesc* table
       const int e = e0 + 256 * k;
       const int row = bi * BM + (e >> 7);
       const int col = bj * BN + (e & 127);
-      v[k] = (row < n && col < n) ? m.src[(size_t)row * n + col] : 0.f;
+      const size_t at = m.rev ? (size_t)(n - 1 - row) * n + (n - 1 - col) : (size_t)row * n + col;
+      v[k] = (row < n && col < n) ? m.src[at] : 0.f;
       if (row == col) v[k] += damp;
     }
 #pragma unroll
@@ -860,6 +862,21 @@ __device__ __forceinline__ void lauum_tile(int T, int local, int& bi, int& bj) {
   bi = bj = 0;       // not reached: the classes hold exactly ntiles tiles
 }
 
+// C[f(row)][f(col)] = v and its mirror image, f(i) = base + sign * i: the identity, or the
+// reversal i -> n - 1 - i that undoes the reversed read of a matrix factored back to front
+struct EpiSymFlip {
+  float* C;
+  int n, base, sign;
+  bool mirror;
+  __device__ __forceinline__ void store(int row, int col, float v) const {
+    if (row < n && col < n) {
+      const int r = base + sign * row, c = base + sign * col;
+      C[(size_t)r * n + c] = v;
+      if (mirror && row != col) C[(size_t)c * n + r] = v;
+    }
+  }
+};
+
 // dst = Y Y^T over the upper tiles (k >= the later block), mirrored
 __global__ __launch_bounds__(NTHREADS) void lauum_kernel(const MatDesc* table, const WorkList wl) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -870,8 +887,39 @@ __global__ __launch_bounds__(NTHREADS) void lauum_kernel(const MatDesc* table, c
   lauum_tile(m.T, local, bi, bj);
   const int n = m.n;
   DenseMK P{m.Y, n, n};
-  EpiStore epi{m.U, n, n, n, 1.f, 0.f, bi != bj};
+  EpiSymFlip epi{m.U, n, m.rev ? n - 1 : 0, m.rev ? -1 : 1, bi != bj};
   gemm_tile(P, P, bi * BM, bj * BN, bj * DB, n, bi == bj, epi, smem);
+}
+
+// W = J Y^T J (J = reversal) for the matrices factored back to front: with S = J X J = R^T R
+// and Y = R^-1, X^-1 = J Y Y^T J = W^T W and W is upper triangular with a positive diagonal,
+// i.e. the upper Cholesky factor of X^-1, read off the triangular inverse instead of being
+// computed by a second factorisation.  W[i][j] = Y[n-1-j][n-1-i] for j >= i, 0 below;
+// 64 x 64 tiles through LDS so that reads and writes are both row-contiguous.
+__global__ __launch_bounds__(256) void std_from_inverse_factor_kernel(const MatDesc* table,
+                                                                      const WorkList wl) {
+  __shared__ float tile[64][65];
+  int mat, local;
+  work_find(wl, mat, local);
+  const MatDesc m = table[mat];
+  if (m.W == nullptr) return;
+  const int n = m.n;
+  const int T64 = (n + 63) / 64;
+  const int ti = local / T64, tj = local - ti * T64;       // tile of W: rows ti, columns tj
+  const int i0 = ti * 64, j0 = tj * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  if (tj >= ti) {
+    // source element for W[i0 + a][j0 + b] is Y[n-1-j0-b][n-1-i0-a]: lanes run along a
+    for (int b = ty; b < 64; b += 4) {
+      const int r = n - 1 - j0 - b, c = n - 1 - i0 - tx;
+      tile[b][tx] = (r >= 0 && c >= 0 && c >= r) ? m.Y[(size_t)r * n + c] : 0.f;
+    }
+  }
+  __syncthreads();
+  for (int a = ty; a < 64; a += 4) {
+    const int i = i0 + a, j = j0 + tx;
+    if (i < n && j < n) m.W[(size_t)i * n + j] = (tj >= ti && j >= i) ? tile[tx][a] : 0.f;
+  }
 }
 
 // zero the strictly lower triangle (Cholesky-factor output)
@@ -903,6 +951,8 @@ struct HostMat {
   int partner;   // index in caller order, or -1
   int is_a;
   int out;
+  float* std = nullptr;   // non-null: factor back to front and also deliver the upper
+                          // Cholesky factor of the inverse (posterior std of Noisy K-FAC)
 };
 
 static size_t inverse_workspace_bytes(const std::vector<int>& dims) {
@@ -960,7 +1010,8 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
       d.is_a = h.is_a;
       d.out = h.out;
       d.trace = 0.f;
-      d.pad = 0;
+      d.rev = h.std != nullptr;
+      d.W = h.std;
       Ts[s0 + k] = d.T;
       Tmax = std::max(Tmax, d.T);
     }
@@ -1092,6 +1143,15 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
   for_worklists(nmat, [](int T) { return T * (T + 1) / 2; }, [&](const WorkList& wl, int grid) {
     KFAC_LAUNCH_TILE2(lauum_kernel, dim3(grid), stream, table, wl);
   });
+  bool any_std = false;
+  for (auto& h : mats) any_std |= h.std != nullptr;
+  if (any_std) {
+    // (items per matrix: its 64 x 64 tiles; Ts holds 128-blocks, so 4 T^2 covers them)
+    for_worklists(nmat, [](int T) { return 4 * T * T; }, [&](const WorkList& wl, int grid) {
+      hipLaunchKernelGGL(std_from_inverse_factor_kernel, dim3(grid), dim3(256), 0, stream, table,
+                         wl);
+    });
+  }
   return launch_status();
 }
 
@@ -1183,6 +1243,30 @@ int kfac_pi_damped_inverse_batched(int layers, const int* dA, const int* dG,
     const float r = sqrtf(damping[l]);
     mats[2 * l] = HostMat{A[l], Ainv[l], dA[l], r, 2 * l + 1, 1, 2 * l};
     mats[2 * l + 1] = HostMat{G[l], Ginv[l], dG[l], r, 2 * l, 0, 2 * l + 1};
+  }
+  return run_batched(mats, MODE_INVERSE, info, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int kfac_pi_damped_inverse_std_batched(int layers, const int* dA, const int* dG,
+                                       const float* const* A, const float* const* G,
+                                       const float* damping, float* const* Ainv,
+                                       float* const* Ginv, float* const* Astd,
+                                       float* const* Gstd, int* info, void* workspace,
+                                       size_t workspace_bytes, void* stream) {
+  if (layers < 0 || (layers > 0 && (!dA || !dG || !A || !G || !damping || !Ainv || !Ginv ||
+                                    !Astd || !Gstd || !info)))
+    return KFAC_ERR_ARG;
+  std::vector<HostMat> mats(2 * layers);
+  for (int l = 0; l < layers; ++l) {
+    if (dA[l] <= 0 || dG[l] <= 0 || dA[l] > 16384 || dG[l] > 16384 || !A[l] || !G[l] ||
+        !Ainv[l] || !Ginv[l] || A[l] == Ainv[l] || G[l] == Ginv[l] || !(damping[l] >= 0.f))
+      return KFAC_ERR_ARG;
+    if ((Astd[l] == nullptr) != (Gstd[l] == nullptr)) return KFAC_ERR_ARG;
+    if (Astd[l] && (Astd[l] == Ainv[l] || Astd[l] == A[l] || Gstd[l] == Ginv[l] || Gstd[l] == G[l]))
+      return KFAC_ERR_ARG;
+    const float r = sqrtf(damping[l]);
+    mats[2 * l] = HostMat{A[l], Ainv[l], dA[l], r, 2 * l + 1, 1, 2 * l, Astd[l]};
+    mats[2 * l + 1] = HostMat{G[l], Ginv[l], dG[l], r, 2 * l, 0, 2 * l + 1, Gstd[l]};
   }
   return run_batched(mats, MODE_INVERSE, info, workspace, workspace_bytes, (hipStream_t)stream);
 }

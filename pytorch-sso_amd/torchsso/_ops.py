@@ -149,6 +149,38 @@ def pi_damped_inverse_batched(As, Gs, dampings, A_invs=None, G_invs=None, info=N
     return A_invs, G_invs, info
 
 
+def pi_damped_inverse_std_batched(As, Gs, dampings, A_invs, G_invs, A_stds, G_stds, info=None):
+    """pi_damped_inverse_batched that also writes, for the layers whose A_stds / G_stds entries
+    are tensors (None: no std for that layer), the upper Cholesky factors of the two inverses
+    (std^T std = inverse), read off the triangular inverse instead of a second factorisation."""
+    lib = _hip.load()
+    layers = len(As)
+    if layers == 0:
+        return None
+    dev = As[0].device
+    dA = _square_dims(As, 'A')
+    dG = _square_dims(Gs, 'G')
+    for l, (a, g, sa, sg) in enumerate(zip(As, Gs, A_stds, G_stds)):
+        if (sa is None) != (sg is None):
+            raise _hip.KfacHipError('layer %d: std buffers must come in pairs' % l)
+        if sa is not None and (sa.shape != a.shape or sg.shape != g.shape):
+            raise _hip.KfacHipError('layer %d: std buffers have the wrong shape' % l)
+    if info is None:
+        info = torch.empty(2 * layers, dtype=torch.int32, device=dev)
+    dims = []
+    for a, g in zip(dA, dG):
+        dims += [a, g]
+    ws, ws_bytes = _hip.workspace(dev, lib.kfac_inverse_workspace_bytes(len(dims), _hip.int_array(dims)))
+    st = lib.kfac_pi_damped_inverse_std_batched(
+        layers, _hip.int_array(dA), _hip.int_array(dG), _hip.ptr_array(As, 'A'),
+        _hip.ptr_array(Gs, 'G'), _hip.f32_array(dampings), _hip.ptr_array(A_invs, 'A_inv'),
+        _hip.ptr_array(G_invs, 'G_inv'), _hip.ptr_array(A_stds, 'A_std', True),
+        _hip.ptr_array(G_stds, 'G_std', True), info.data_ptr(), _ws_ptr(ws), ws_bytes,
+        _hip.stream_ptr(dev))
+    _hip.check(st, 'kfac_pi_damped_inverse_std_batched')
+    return info
+
+
 def damped_inverse_batched(mats, damps=None, outs=None, info=None):
     """outs[i] = (mats[i] + damps[i]*I)^-1."""
     lib = _hip.load()

@@ -427,20 +427,39 @@ def update_ema_all(curvs):
     _ops.max_batched(xs, ys)
 
 
-def update_inv_all(curvs):
+def update_inv_all(curvs, with_std=()):
     """update_inv for every curvature: one batched pi-damped inversion for all
     Kronecker layers (reference: curvature.py:302-312), one element-wise launch
-    for all diagonal layers (curvature.py:193-195,226-232)."""
+    for all diagonal layers (curvature.py:193-195,226-232).
+
+    `with_std`: curvatures whose `std` will be asked for right after (update_std,
+    curvature.py:317-321).  For the Kronecker ones among them the inversion delivers the
+    Cholesky factors of the inverses as well (the engine factors those matrices back to
+    front and reads the factor off the triangular inverse), so that update_std_all has
+    nothing left to compute for them."""
     kron = [c for c in curvs if c.kind == 'kron']
     diag = [c for c in curvs if c.kind == 'diag']
     full = [c for c in curvs if c.kind == 'full']
+    wanted = {id(c) for c in with_std}
     if kron:
         for c in kron:
             if c.inv is None or c.inv[0].shape != c.ema[0].shape or c.inv[1].shape != c.ema[1].shape:
                 c.inv = [torch.empty_like(c.ema[0]), torch.empty_like(c.ema[1])]
-        _, _, info = _ops.pi_damped_inverse_batched(
-            [c.ema[0] for c in kron], [c.ema[1] for c in kron], [c.damping for c in kron],
-            [c.inv[0] for c in kron], [c.inv[1] for c in kron])
+            if id(c) in wanted and (c.std is None
+                                    or any(s.shape != i.shape for s, i in zip(c.std, c.inv))):
+                c.std = [torch.empty_like(i) for i in c.inv]
+        args = ([c.ema[0] for c in kron], [c.ema[1] for c in kron], [c.damping for c in kron],
+                [c.inv[0] for c in kron], [c.inv[1] for c in kron])
+        if any(id(c) in wanted for c in kron):
+            info = _ops.pi_damped_inverse_std_batched(
+                *args, [c.std[0] if id(c) in wanted else None for c in kron],
+                [c.std[1] if id(c) in wanted else None for c in kron])
+            for c in kron:
+                if id(c) in wanted:
+                    c._std_current = True      # update_std_all has nothing to do for it
+                    c.std_info = None          # (a failure shows in `info`)
+        else:
+            _, _, info = _ops.pi_damped_inverse_batched(*args)
         for i, c in enumerate(kron):
             c.info = info[2 * i:2 * i + 2]
     if diag:
@@ -464,7 +483,14 @@ def update_std_all(curvs):
     """update_std: upper Cholesky factors of the inverses for Kronecker layers
     (reference: curvature.py:317-321), sqrt of the inverse for diagonal ones
     (curvature.py:240-241)."""
-    kron = [c for c in curvs if c.kind == 'kron']
+    kron = []
+    for c in curvs:
+        if c.kind != 'kron':
+            continue
+        if getattr(c, '_std_current', False):
+            c._std_current = False             # delivered with the inverses (update_inv_all)
+        else:
+            kron.append(c)
     mats, outs = [], []
     for c in kron:
         if c.std is None or any(s.shape != i.shape for s, i in zip(c.std, c.inv)):
@@ -525,12 +551,12 @@ def step_all(curvs, update_std=False, update_inv=True):
     """Curvature.step for a list (reference: curvature.py:166-172).
     `update_std` may be a bool or a list of bools, one per curvature."""
     update_ema_all(curvs)
-    if update_inv:
-        update_inv_all(curvs)
     if isinstance(update_std, (list, tuple)):
         sel = [c for c, u in zip(curvs, update_std) if u]
     else:
         sel = list(curvs) if update_std else []
+    if update_inv:
+        update_inv_all(curvs, with_std=sel)
     if sel:
         update_std_all(sel)
 

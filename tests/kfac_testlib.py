@@ -211,6 +211,14 @@ class OracleOps(object):
             rg.append(g)
         return (A_invs or ra), (G_invs or rg), torch.zeros(2 * len(As), dtype=torch.int32)
 
+    def pi_damped_inverse_std_batched(self, As, Gs, dampings, A_invs, G_invs, A_stds, G_stds,
+                                      info=None):
+        _, _, info = self.pi_damped_inverse_batched(As, Gs, dampings, A_invs, G_invs)
+        for inv, std in list(zip(A_invs, A_stds)) + list(zip(G_invs, G_stds)):
+            if std is not None:
+                std.copy_(O.cholesky_upper(inv, self.dtype))
+        return info
+
     def damped_inverse_batched(self, mats, damps=None, outs=None, info=None):
         res = [O.damped_inverse(m, 0. if damps is None else damps[i], self.dtype)
                for i, m in enumerate(mats)]

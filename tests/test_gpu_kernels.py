@@ -211,6 +211,53 @@ def test_inverse_and_cholesky_of_random_ragged_batches(ops, dev):
             assert torch.equal(u, torch.triu(u)), (sizes, n)
 
 
+def test_inverse_with_posterior_std_from_the_same_factorisation(ops, dev):
+    """kfac_pi_damped_inverse_std_batched: for the layers that ask for it, the upper Cholesky
+    factor W of each inverse (W^T W = inverse: what torchsso.utils.cholesky of the inverse
+    gives, utils/cholesky_cupy.py:9-14) comes out of the inversion itself, which factors those
+    matrices back to front.  Ragged sizes (1 .. 1500, block-size neighbours), layers with and
+    without std mixed in one call; everything against float64 on the device."""
+    gen = torch.Generator().manual_seed(11)
+    pairs = [(1, 3), (33, 64), (129, 127), (700, 10), (385, 192), (1500, 256), (128, 1025)]
+    As, Gs = [], []
+    for dA, dG in pairs:
+        for n, lst in ((dA, As), (dG, Gs)):
+            a = torch.randn(n, n + 8, generator=gen).to(dev)
+            lst.append((a @ a.t() / (n + 8)).contiguous())
+    damp = [1e-3 * (l + 1) for l in range(len(pairs))]
+    want_std = [l % 3 != 1 for l in range(len(pairs))]
+    Ai = [torch.full_like(a, float('nan')) for a in As]
+    Gi = [torch.full_like(g, float('nan')) for g in Gs]
+    Astd = [torch.full_like(a, float('nan')) if w else None for a, w in zip(As, want_std)]
+    Gstd = [torch.full_like(g, float('nan')) if w else None for g, w in zip(Gs, want_std)]
+    info = ops.pi_damped_inverse_std_batched(As, Gs, damp, Ai, Gi, Astd, Gstd)
+    plainA, plainG, info0 = ops.pi_damped_inverse_batched(As, Gs, damp)
+    assert info.cpu().tolist() == [0] * (2 * len(pairs)) and int(info0.abs().sum()) == 0
+    eye = lambda n: torch.eye(n, dtype=D, device=dev)
+    worst = {'inverse': 0., 'std': 0., 'std^T std vs inverse': 0.}
+    for l, (a, g) in enumerate(zip(As, Gs)):
+        pi = ((a.double().diagonal().sum() / a.shape[0]) / (g.double().diagonal().sum() / g.shape[0])).sqrt()
+        r = damp[l] ** 0.5
+        for X, shift, inv, plain, std in ((a, r * pi, Ai[l], plainA[l], Astd[l]),
+                                          (g, r / pi, Gi[l], plainG[l], Gstd[l])):
+            n = X.shape[0]
+            ref = torch.linalg.inv(X.double() + shift * eye(n))
+            worst['inverse'] = max(worst['inverse'], ((inv.double() - ref).norm() / ref.norm()).item())
+            assert torch.equal(inv, inv.t())
+            if std is None:
+                assert torch.equal(inv, plain)              # untouched by the others' reversal
+                continue
+            W = std.double()
+            assert torch.equal(std, torch.triu(std)) and bool((std.diagonal() > 0).all())
+            refW = torch.linalg.cholesky(ref).mT
+            worst['std'] = max(worst['std'], ((W - refW).norm() / refW.norm()).item())
+            worst['std^T std vs inverse'] = max(worst['std^T std vs inverse'],
+                                                ((W.t() @ W - inv.double()).norm() / inv.double().norm()).item())
+    print('inverse + std in one factorisation, worst rel. Frobenius errors:',
+          {k: '%.2e' % v for k, v in worst.items()})
+    assert worst['inverse'] < TOL and worst['std'] < TOL and worst['std^T std vs inverse'] < 1e-5
+
+
 SHAPES = [(10, 193, True), (64, 76, True), (1000, 785, True), (128, 1601, True),
           (512, 1152, False), (1, 2, True), (3, 1, False), (64, 64, False), (130, 257, True)]
 
