@@ -713,6 +713,12 @@ def main():
     ap.add_argument('--factor-streams', type=int, default=None,
                     help='side streams for the factor products (library default: 3; 0 = none)')
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--factored-min-dim', type=int, default=None,
+                    help='rows from which update_inv keeps an inverse as its triangular factor '
+                         '(library default: KronCurvature.factored_inverse_min_dim)')
+    ap.add_argument('--explicit-inverse', action='store_true',
+                    help='form A^-1 and G^-1 explicitly in update_inv (as the reference does) '
+                         'instead of keeping their triangular factors and applying those')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run a plain 1 GiB device copy (reference for rocprofv3 --pmc '
                          'FETCH_SIZE / WRITE_SIZE readings)')
@@ -730,6 +736,14 @@ def main():
     if args.factor_streams is not None:
         torchsso.set_factor_streams(args.factor_streams)
     factor_streams = torchsso.factor_streams()
+    from torchsso.curv.curvature import KronCurvature
+    if args.explicit_inverse:
+        KronCurvature.factored_inverse_min_dim = None
+    elif args.factored_min_dim is not None:
+        KronCurvature.factored_inverse_min_dim = args.factored_min_dim
+    inverse_form = ('explicit' if KronCurvature.factored_inverse_min_dim is None else
+                    'triangular factor Y (Y Y^T = inverse) for factors of >= %d rows, explicit below'
+                    % KronCurvature.factored_inverse_min_dim)
 
     if args.workload == 'resnet50_train':
         print(json.dumps(run_resnet50_train(args)))
@@ -737,6 +751,7 @@ def main():
     if args.workload == 'noisy_kfac':
         out = run_noisy_kfac(args)
         out['config']['factor_side_streams'] = factor_streams
+        out['config']['inverse_form'] = inverse_form
         if not args.no_cpu_baseline:
             # the same step on the host: 4 x factors + inverse + Cholesky + 4 x sampling products
             specs = convnet_specs()
@@ -779,7 +794,8 @@ def main():
         'config': {'workload': label, 'batch': batch,
                    'kron_layers': sum(1 for s in specs if s['kind'] != 'bn'),
                    'bn_layers': sum(1 for s in specs if s['kind'] == 'bn'),
-                   'damping': 1e-3, 'ema_decay': 0.95, 'invert_every_step': True, 'factor_side_streams': factor_streams,
+                   'damping': 1e-3, 'ema_decay': 0.95, 'invert_every_step': True, 'inverse_form': inverse_form,
+                   'factor_side_streams': factor_streams,
                    'inputs_resident_GB': round(resident / 1e9, 3)},
         'tflops': round(total_flops / (ms * 1e-3) / 1e12, 2),
         'algorithmic_gflop': {k: round(v / 1e9, 1) for k, v in work.items() if not k.endswith('bytes')},

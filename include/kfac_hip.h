@@ -127,8 +127,8 @@ int kfac_pi_damped_inverse_batched(int layers, const int* dA, const int* dG,
                                    float* const* Ainv, float* const* Ginv, int* info,
                                    void* workspace, size_t workspace_bytes, void* stream);
 
-/* kfac_pi_damped_inverse_batched that also delivers, for the layers l with Astd[l] and
- * Gstd[l] non-NULL (both or neither), the upper Cholesky factors of the two inverses:
+/* kfac_pi_damped_inverse_batched that also delivers, for every matrix whose Astd[l] / Gstd[l]
+ * is non-NULL, the upper Cholesky factor of its inverse:
  *   Astd[l]^T Astd[l] = Ainv[l],  Gstd[l]^T Gstd[l] = Ginv[l],  upper triangular, zero below.
  * Replaces KronCurvature.update_inv followed by update_std, torchsso/curv/curvature.py:302-312
  * and :317-321 (torchsso.utils.cholesky of each inverse, utils/cholesky_cupy.py:9-14), without
@@ -136,13 +136,30 @@ int kfac_pi_damped_inverse_batched(int layers, const int* dA, const int* dG,
  * columns reversed, J X J = R^T R), so that X^-1 = J R^-1 R^-T J = W^T W with W = J R^-T J upper
  * triangular with a positive diagonal -- the Cholesky factor the reference computes from the
  * inverse -- and W is read off the triangular inverse the inversion forms anyway.  For these
- * layers a non-zero info[] counts the failing leading minor of the REVERSED matrix. */
+ * matrices a non-zero info[] counts the failing leading minor of the REVERSED matrix. */
 int kfac_pi_damped_inverse_std_batched(int layers, const int* dA, const int* dG,
                                        const float* const* A, const float* const* G,
                                        const float* damping,
                                        float* const* Ainv, float* const* Ginv,
                                        float* const* Astd, float* const* Gstd, int* info,
                                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* kfac_pi_damped_inverse_batched for a caller that applies the inverses rather than reads
+ * them: per matrix EXACTLY ONE of Ainv[l] / Afac[l] (and of Ginv[l] / Gfac[l]) is non-NULL.
+ * Where the `fac` pointer is given the result is the triangular factor of the inverse,
+ *   Afac[l] Afac[l]^T = (A + r*pi*I)^-1 ,  Gfac[l] Gfac[l]^T = (G + (r/pi)*I)^-1 ,
+ * upper triangular with zeros below the diagonal (the inverse of the Cholesky factor), and the
+ * explicit inverse, the last third of that matrix's inversion work, is never formed:
+ * kfac_precondition_factored_batched applies the factor twice at the cost of applying the
+ * inverse once.  Replaces KronCurvature.update_inv, torchsso/curv/curvature.py:302-312 with
+ * utils/inv_cupy.py:27-34; the explicit inverse of a factored matrix is fac * fac^T.
+ * pi, r, info and the workspace as for kfac_pi_damped_inverse_batched. */
+int kfac_pi_damped_inverse_factored_batched(int layers, const int* dA, const int* dG,
+                                            const float* const* A, const float* const* G,
+                                            const float* damping,
+                                            float* const* Ainv, float* const* Ginv,
+                                            float* const* Afac, float* const* Gfac, int* info,
+                                            void* workspace, size_t workspace_bytes, void* stream);
 
 /* dst[i] = (src[i] + damp[i]*I)^-1 for `count` symmetric positive definite
  * matrices of sizes dims[i]; damp may be NULL (no shift).  Host arrays as
@@ -195,6 +212,21 @@ int kfac_precondition_batched(int layers, const int* dG, const int* dA,
                               const float* const* Ginv, const float* const* Ainv,
                               float* const* gradW, float* const* gradb,
                               void* workspace, size_t workspace_bytes, void* stream);
+
+/* kfac_precondition_batched with some or all inverses given by their triangular factors, as
+ * kfac_pi_damped_inverse_factored_batched delivers them: Gop[l] is the upper-triangular Gfac
+ * (Gfac Gfac^T = Ginv, zeros below the diagonal) where g_factored[l] != 0, else Ginv itself;
+ * Aop[l] and a_factored[l] likewise (a NULL flag array means "all factored").
+ *   [gradW | gradb] <- Gfac (Gfac^T [gradW | gradb] Afac) Afac^T , in place;
+ * a factored side takes two products that each skip the zero half of the triangular operand,
+ * which together cost what the one dense product with the explicit inverse costs.  Replaces
+ * the same call sites, torchsso/curv/cov/linear.py:69-84 and cov/conv.py:76-92. */
+size_t kfac_precondition_factored_workspace_bytes(int layers, const int* dG, const int* dA);
+int kfac_precondition_factored_batched(int layers, const int* dG, const int* dA,
+                                       const float* const* Gop, const float* const* Aop,
+                                       const int* g_factored, const int* a_factored,
+                                       float* const* gradW, float* const* gradb,
+                                       void* workspace, size_t workspace_bytes, void* stream);
 
 /* For every layer:  [paramW | paramb] = [meanW | meanb] + std_scale * U_G * E * U_A
  * with U_G, U_A the upper Cholesky factors of the inverses and E = noise[l], a

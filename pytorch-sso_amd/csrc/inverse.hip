@@ -32,8 +32,9 @@ namespace kfac {
 
 struct MatDesc {
   const float* src;
-  float* U;      // = dst
-  float* Y;      // workspace, n*n
+  float* U;      // Cholesky factor, then the inverse: dst (the workspace slot when only Y is wanted)
+  float* Y;      // inverse of the Cholesky factor, n*n: the workspace slot, or the caller's
+                 // buffer when Y itself is the result
   int n;
   int T;         // number of 128-blocks
   float damp;    // given damping, or sqrt(damping) in pi mode
@@ -43,6 +44,8 @@ struct MatDesc {
   float trace;
   int rev;       // 1: the work matrix is src with rows and columns reversed (see run_batched)
   float* W;      // rev only: receives the upper Cholesky factor of the inverse, else nullptr
+  int noinv;     // 1: the explicit inverse is not wanted, Y is the result (Y Y^T = inverse)
+  int pad;
 };
 
 constexpr int SETUP_CHUNK = 48;
@@ -883,6 +886,7 @@ __global__ __launch_bounds__(NTHREADS) void lauum_kernel(const MatDesc* table, c
   int mat, local;
   work_find(wl, mat, local);
   const MatDesc m = table[mat];
+  if (m.noinv) return;
   int bi, bj;
   lauum_tile(m.T, local, bi, bj);
   const int n = m.n;
@@ -922,11 +926,15 @@ __global__ __launch_bounds__(256) void std_from_inverse_factor_kernel(const MatD
   }
 }
 
-// zero the strictly lower triangle (Cholesky-factor output)
-__global__ __launch_bounds__(256) void zero_lower_kernel(const MatDesc* table, const WorkList wl) {
+// zero the strictly lower triangle of a triangular result: of U for every matrix
+// (Cholesky-factor output), or, with `of_y`, of Y for the matrices whose result Y is
+__global__ __launch_bounds__(256) void zero_lower_kernel(const MatDesc* table, int of_y,
+                                                         const WorkList wl) {
   int mat, local;
   work_find(wl, mat, local);
   const MatDesc m = table[mat];
+  if (of_y && !m.noinv) return;
+  float* const X = of_y ? m.Y : m.U;
   const int n = m.n;
   const int T = m.T;
   const int bi = local / T, bj = local - bi * T;
@@ -934,7 +942,7 @@ __global__ __launch_bounds__(256) void zero_lower_kernel(const MatDesc* table, c
   for (int e = threadIdx.x; e < BM * BN; e += 256) {
     const int row = bi * BM + (e >> 7);
     const int col = bj * BN + (e & 127);
-    if (row < n && col < n && col < row) m.U[(size_t)row * n + col] = 0.f;
+    if (row < n && col < n && col < row) X[(size_t)row * n + col] = 0.f;
   }
 }
 
@@ -952,7 +960,10 @@ struct HostMat {
   int is_a;
   int out;
   float* std = nullptr;   // non-null: factor back to front and also deliver the upper
-                          // Cholesky factor of the inverse (posterior std of Noisy K-FAC)
+                          // Cholesky factor W of the inverse (W^T W = inverse; the posterior
+                          // std of Noisy K-FAC)
+  float* fac = nullptr;   // non-null (then dst and std are null): deliver the inverse as its
+                          // triangular factor only, Y upper with Y Y^T = inverse
 };
 
 static size_t inverse_workspace_bytes(const std::vector<int>& dims) {
@@ -1000,8 +1011,12 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
       const HostMat& h = mats[order[s0 + k]];
       MatDesc& d = chunk.d[k];
       d.src = h.src;
-      d.U = h.dst;
-      d.Y = (float*)(ybase + yoff);
+      // the slot of the workspace holds Y, or, when Y goes straight to the caller, the
+      // Cholesky factor that nobody asked for
+      d.noinv = h.fac != nullptr;
+      d.pad = 0;
+      d.U = d.noinv ? (float*)(ybase + yoff) : h.dst;
+      d.Y = d.noinv ? h.fac : (float*)(ybase + yoff);
       yoff += align256((size_t)h.n * h.n * sizeof(float));
       d.n = h.n;
       d.T = cdiv(h.n, DB);
@@ -1121,7 +1136,7 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
   }
   if (mode == MODE_CHOLESKY) {
     for_worklists(nmat, [](int T) { return T * T; }, [&](const WorkList& wl, int grid) {
-      hipLaunchKernelGGL(zero_lower_kernel, dim3(grid), dim3(256), 0, stream, table, wl);
+      hipLaunchKernelGGL(zero_lower_kernel, dim3(grid), dim3(256), 0, stream, table, 0, wl);
     });
     return launch_status();
   }
@@ -1140,11 +1155,20 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
       });
     }
   }
-  for_worklists(nmat, [](int T) { return T * (T + 1) / 2; }, [&](const WorkList& wl, int grid) {
-    KFAC_LAUNCH_TILE2(lauum_kernel, dim3(grid), stream, table, wl);
-  });
-  bool any_std = false;
-  for (auto& h : mats) any_std |= h.std != nullptr;
+  bool any_inv = false, any_std = false, any_fac = false;
+  for (auto& h : mats) {
+    any_inv |= h.dst != nullptr;
+    any_std |= h.std != nullptr;
+    any_fac |= h.fac != nullptr;
+  }
+  if (any_inv)
+    for_worklists(nmat, [](int T) { return T * (T + 1) / 2; }, [&](const WorkList& wl, int grid) {
+      KFAC_LAUNCH_TILE2(lauum_kernel, dim3(grid), stream, table, wl);
+    });
+  if (any_fac)   // the triangular inversion kept intermediate products below the diagonal
+    for_worklists(nmat, [](int T) { return T * T; }, [&](const WorkList& wl, int grid) {
+      hipLaunchKernelGGL(zero_lower_kernel, dim3(grid), dim3(256), 0, stream, table, 1, wl);
+    });
   if (any_std) {
     // (items per matrix: its 64 x 64 tiles; Ts holds 128-blocks, so 4 T^2 covers them)
     for_worklists(nmat, [](int T) { return 4 * T * T; }, [&](const WorkList& wl, int grid) {
@@ -1261,12 +1285,37 @@ int kfac_pi_damped_inverse_std_batched(int layers, const int* dA, const int* dG,
     if (dA[l] <= 0 || dG[l] <= 0 || dA[l] > 16384 || dG[l] > 16384 || !A[l] || !G[l] ||
         !Ainv[l] || !Ginv[l] || A[l] == Ainv[l] || G[l] == Ginv[l] || !(damping[l] >= 0.f))
       return KFAC_ERR_ARG;
-    if ((Astd[l] == nullptr) != (Gstd[l] == nullptr)) return KFAC_ERR_ARG;
-    if (Astd[l] && (Astd[l] == Ainv[l] || Astd[l] == A[l] || Gstd[l] == Ginv[l] || Gstd[l] == G[l]))
-      return KFAC_ERR_ARG;
+    if (Astd[l] && (Astd[l] == Ainv[l] || Astd[l] == A[l])) return KFAC_ERR_ARG;
+    if (Gstd[l] && (Gstd[l] == Ginv[l] || Gstd[l] == G[l])) return KFAC_ERR_ARG;
     const float r = sqrtf(damping[l]);
     mats[2 * l] = HostMat{A[l], Ainv[l], dA[l], r, 2 * l + 1, 1, 2 * l, Astd[l]};
     mats[2 * l + 1] = HostMat{G[l], Ginv[l], dG[l], r, 2 * l, 0, 2 * l + 1, Gstd[l]};
+  }
+  return run_batched(mats, MODE_INVERSE, info, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int kfac_pi_damped_inverse_factored_batched(int layers, const int* dA, const int* dG,
+                                            const float* const* A, const float* const* G,
+                                            const float* damping, float* const* Ainv,
+                                            float* const* Ginv, float* const* Afac,
+                                            float* const* Gfac, int* info, void* workspace,
+                                            size_t workspace_bytes, void* stream) {
+  if (layers < 0 || (layers > 0 && (!dA || !dG || !A || !G || !damping || !Ainv || !Ginv ||
+                                    !Afac || !Gfac || !info)))
+    return KFAC_ERR_ARG;
+  std::vector<HostMat> mats(2 * layers);
+  for (int l = 0; l < layers; ++l) {
+    if (dA[l] <= 0 || dG[l] <= 0 || dA[l] > 16384 || dG[l] > 16384 || !A[l] || !G[l] ||
+        !(damping[l] >= 0.f))
+      return KFAC_ERR_ARG;
+    // per matrix exactly one of the two forms, never on top of its input
+    if ((Ainv[l] == nullptr) == (Afac[l] == nullptr) || (Ginv[l] == nullptr) == (Gfac[l] == nullptr))
+      return KFAC_ERR_ARG;
+    if (Ainv[l] == A[l] || Afac[l] == A[l] || Ginv[l] == G[l] || Gfac[l] == G[l])
+      return KFAC_ERR_ARG;
+    const float r = sqrtf(damping[l]);
+    mats[2 * l] = HostMat{A[l], Ainv[l], dA[l], r, 2 * l + 1, 1, 2 * l, nullptr, Afac[l]};
+    mats[2 * l + 1] = HostMat{G[l], Ginv[l], dG[l], r, 2 * l, 0, 2 * l + 1, nullptr, Gfac[l]};
   }
   return run_batched(mats, MODE_INVERSE, info, workspace, workspace_bytes, (hipStream_t)stream);
 }

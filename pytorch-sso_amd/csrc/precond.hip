@@ -27,7 +27,7 @@ struct LayerDesc {
   float* Tt;             // dA x dG scratch
   int dG, dA, dAw;       // dAw = dA - (has bias)
   float scale;
-  int pad;
+  int flags;         // factored preconditioning: bit 0 L is Wg, bit 1 R is Wa (else the inverses)
 };
 
 constexpr int LAYER_CHUNK = 32;
@@ -77,86 +77,205 @@ struct EpiSplit {
   }
 };
 
+// ---------------------------------------------------------------------------
+// The products.  Explicit inverses:  U = G^-1 V A^-1, two products:
+//   first    T^T[a][i] = sum_k V[k][a] G^-1[k][i]            (T = G^-1 V, kept transposed)
+//   second   U[i][j]   = sum_a T^T[a][i] A^-1[a][j]
+// An inverse may instead be given by its triangular factor Y (upper, Y Y^T = inverse: the
+// inverse of the Cholesky factor, which the batched inversion delivers where the explicit
+// inverse is not asked for; it then skips the n^3/3 product Y Y^T of that matrix).  Bit 0 of
+// a layer's `flags` says that L is Yg, bit 1 that R is Ya.  A factored side takes two
+// products with the triangular operand, each over the non-zero part of its reduction only
+// (half of a dense product), in place of the one dense product:
+//   first    T^T[a][i] = sum_{k <= i} V[k][a] Yg[k][i]       (T = Yg^T V)
+//   second   X[i][j]   = sum_{a <= j} T^T[a][i] Ya[a][j]     (X = T Ya)
+//   third    X'[i][j]  = sum_{a >= j} X[i][a] Ya[j][a]       (X' = X Ya^T)   layers with Ya
+//   fourth   U[i][j]   = sum_{k >= i} Yg[i][k] X'[k][j]      (U = Yg X')     layers with Yg
+// so that the first two read their operand exactly as they read an explicit inverse, only
+// over a shorter range.  The last product a layer takes part in writes the gradients; the
+// results in between live in the two halves of the layer's scratch (T^T in the first; the
+// result of the second and third product in whichever half that product does not read).
+//
+// The reduction of a tile against a triangular operand runs from or to the tile's own
+// position along one tile index (`fast` below), so its length varies from one block to all
+// of them.  Such a layer's tiles are dispatched longest first: all tiles of the longest
+// reduction, then the next shorter, so that the launch ends on its shortest tiles.
+// Workgroups go to the 8 XCDs in turn by dispatch index; consecutive tiles share the
+// triangular operand's panel and an XCD keeps meeting the same few panels of the other
+// operand, so no remapping is needed for the L2s.  Dense layers keep the contiguous-range
+// mapping.  Posterior sampling (U_G E U_A, both upper triangular) uses the first two
+// products with its own operand layouts.
+// ---------------------------------------------------------------------------
+
+// (slow, fast) tile indices of work item `local` of a layer with tslow x tfast tiles.
+// `tri`: the reduction length depends on `fast`; it grows with it if `grows`.
+struct TileItem {
+  int slow, fast;
+};
+__device__ __forceinline__ TileItem tile_item(int local, int tslow, int tfast, bool tri,
+                                              bool grows) {
+  TileItem it;
+  if (tri) {
+    const int rank = local / tslow;
+    it.slow = local - rank * tslow;
+    it.fast = grows ? tfast - 1 - rank : rank;
+  } else {
+    const int item = xcd_remap(local, tslow * tfast);
+    it.slow = item / tfast;
+    it.fast = item - it.slow * tfast;
+  }
+  return it;
+}
+
+// where the products of a layer between the first and the last put their result
+__device__ __forceinline__ float* second_half(const LayerDesc& m) {
+  return m.Tt + (size_t)m.dG * m.dA;
+}
+
 template <bool SAMPLE>
-__global__ __launch_bounds__(NTHREADS) void precond_first_kernel(const LayerDesc* table,
+__global__ __launch_bounds__(NTHREADS, 3) void precond_first_kernel(const LayerDesc* table,
                                                                  const WorkList wl) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   int layer, local;
   work_find(wl, layer, local);
   const LayerDesc m = table[layer];
   const int ta = tiles128(m.dA), tg = tiles128(m.dG);
-  const int item = xcd_remap(local, ta * tg);
-  const int bi = item / tg, bj = item - bi * tg;   // bi over dA, bj over dG
   EpiStore epi{m.Tt, m.dG, m.dA, m.dG, 1.f, 0.f, false};
   if (SAMPLE) {
+    const int item = xcd_remap(local, ta * tg);
+    const int bi = item / tg, bj = item - bi * tg;   // bi over dA, bj over dG
     // noise E is a plain dG x dA matrix; U_G is upper triangular: L(k, i) = U_G[i][k], k >= i
     DenseKM P{m.V, nullptr, m.dA, m.dA, 0};
     DenseMK Q{m.L, m.dG, m.dG};
     gemm_tile(P, Q, bi * BM, bj * BN, bj * BN, m.dG, false, epi, smem);
   } else {
+    const bool tri = m.flags & 1;
+    const TileItem it = tile_item(local, ta, tg, tri, true);
+    const int bi = it.slow, bj = it.fast;            // bi over dA, bj over dG
     DenseKM P{m.V, m.vb, m.dAw, m.dA, m.vb ? 2 : 0};
     DenseKM Q{m.L, nullptr, m.dG, m.dG, 0};
-    gemm_tile(P, Q, bi * BM, bj * BN, 0, m.dG, false, epi, smem);
+    gemm_tile(P, Q, bi * BM, bj * BN, 0, tri ? min(m.dG, (bj + 1) * BN) : m.dG, false, epi, smem);
   }
 }
 
 template <bool SAMPLE>
-__global__ __launch_bounds__(NTHREADS) void precond_second_kernel(const LayerDesc* table,
+__global__ __launch_bounds__(NTHREADS, 3) void precond_second_kernel(const LayerDesc* table,
                                                                  const WorkList wl) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   int layer, local;
   work_find(wl, layer, local);
   const LayerDesc m = table[layer];
   const int ta = tiles128(m.dA), tg = tiles128(m.dG);
-  const int item = xcd_remap(local, ta * tg);
-  const int bi = item / ta, bj = item - bi * ta;   // bi over dG, bj over dA
   DenseKM P{m.Tt, nullptr, m.dG, m.dG, 0};
   DenseKM Q{m.R, nullptr, m.dA, m.dA, 0};
-  EpiSplit epi{m.outW, m.outb, m.meanW, m.meanb, m.dG, m.dA, m.dAw, m.scale};
-  // U_A is upper triangular: rows a > j are zero, so the sum stops at the tile's last column
-  const int kend = SAMPLE ? min(m.dA, (bj + 1) * BN) : m.dA;
-  gemm_tile(P, Q, bi * BM, bj * BN, 0, kend, false, epi, smem);
+  if (SAMPLE) {
+    const int item = xcd_remap(local, ta * tg);
+    const int bi = item / ta, bj = item - bi * ta;   // bi over dG, bj over dA
+    EpiSplit epi{m.outW, m.outb, m.meanW, m.meanb, m.dG, m.dA, m.dAw, m.scale};
+    // U_A is upper triangular: rows a > j are zero, so the sum stops at the tile's last column
+    gemm_tile(P, Q, bi * BM, bj * BN, 0, min(m.dA, (bj + 1) * BN), false, epi, smem);
+  } else {
+    const bool tri = m.flags & 2;
+    const TileItem it = tile_item(local, tg, ta, tri, true);
+    const int bi = it.slow, bj = it.fast;            // bi over dG, bj over dA
+    const EpiSplit epi = m.flags == 0
+        ? EpiSplit{m.outW, m.outb, nullptr, nullptr, m.dG, m.dA, m.dAw, 1.f}
+        : EpiSplit{second_half(m), nullptr, nullptr, nullptr, m.dG, m.dA, m.dA, 1.f};
+    gemm_tile(P, Q, bi * BM, bj * BN, 0, tri ? min(m.dA, (bj + 1) * BN) : m.dA, false, epi, smem);
+  }
+}
+
+// third product, layers whose R is the factor Ya:  X' = X Ya^T, reduction a >= j
+__global__ __launch_bounds__(NTHREADS, 3) void precond_third_kernel(const LayerDesc* table,
+                                                                const WorkList wl) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  int layer, local;
+  work_find(wl, layer, local);
+  const LayerDesc m = table[layer];
+  const int ta = tiles128(m.dA), tg = tiles128(m.dG);
+  const TileItem it = tile_item(local, tg, ta, true, false);
+  const int bi = it.slow, bj = it.fast;              // bi over dG, bj over dA
+  DenseMK P{second_half(m), m.dA, m.dG};
+  DenseMK Q{m.R, m.dA, m.dA};
+  const EpiSplit epi = (m.flags & 1)
+      ? EpiSplit{m.Tt, nullptr, nullptr, nullptr, m.dG, m.dA, m.dA, 1.f}
+      : EpiSplit{m.outW, m.outb, nullptr, nullptr, m.dG, m.dA, m.dAw, 1.f};
+  gemm_tile(P, Q, bi * BM, bj * BN, bj * BN, m.dA, false, epi, smem);
+}
+
+// fourth product, layers whose L is the factor Yg:  U = Yg X', reduction k >= i
+__global__ __launch_bounds__(NTHREADS, 3) void precond_fourth_kernel(const LayerDesc* table,
+                                                                 const WorkList wl) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  int layer, local;
+  work_find(wl, layer, local);
+  const LayerDesc m = table[layer];
+  const int ta = tiles128(m.dA), tg = tiles128(m.dG);
+  const TileItem it = tile_item(local, ta, tg, true, false);
+  const int bi = it.fast, bj = it.slow;              // bi over dG, bj over dA
+  DenseMK P{m.L, m.dG, m.dG};
+  DenseKM Q{(m.flags & 2) ? m.Tt : second_half(m), nullptr, m.dA, m.dA, 0};
+  EpiSplit epi{m.outW, m.outb, nullptr, nullptr, m.dG, m.dA, m.dAw, 1.f};
+  gemm_tile(P, Q, bi * BM, bj * BN, bi * BM, m.dG, false, epi, smem);
 }
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
-static size_t precond_workspace(int layers, const int* dG, const int* dA) {
-  size_t bytes = 2 * align256((size_t)layers * sizeof(LayerDesc));     // one table per product
-  for (int l = 0; l < layers; ++l) bytes += align256((size_t)dG[l] * dA[l] * sizeof(float));
+constexpr int PRODUCTS = 4;
+
+// scratch: one descriptor table per product, then per layer dG*dA floats (twice that when
+// `factored`: a layer with a factored side keeps two results in flight)
+static size_t precond_workspace(int layers, const int* dG, const int* dA, bool factored) {
+  size_t bytes = PRODUCTS * align256((size_t)layers * sizeof(LayerDesc));
+  for (int l = 0; l < layers; ++l)
+    bytes += align256((size_t)(factored ? 2 : 1) * dG[l] * dA[l] * sizeof(float));
   return bytes;
 }
 
+// flags: per layer, bit 0 L is the factor Yg, bit 1 R is the factor Ya (nullptr: none)
 static int run_layers(int layers, const int* dG, const int* dA, const float* const* L,
                       const float* const* R, const float* const* V, const float* const* vb,
                       const float* const* meanW, const float* const* meanb, float* const* outW,
                       float* const* outb, const int* has_bias, float scale, bool sample,
-                      void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                      const int* flags, void* workspace, size_t workspace_bytes,
+                      hipStream_t stream) {
   if (layers == 0) return KFAC_OK;
-  if (!workspace || workspace_bytes < precond_workspace(layers, dG, dA)) return KFAC_ERR_WORKSPACE;
-  // Longest tiles first, so that the tail of a launch is made of short tiles: each of
-  // the two products walks the layers in the order of ITS reduction length (dG for the
-  // first, dA for the second), through a descriptor table of its own.
+  if (!workspace || workspace_bytes < precond_workspace(layers, dG, dA, flags != nullptr))
+    return KFAC_ERR_WORKSPACE;
+  bool any[PRODUCTS] = {true, true, false, false};
+  for (int l = 0; flags && l < layers; ++l) {
+    any[2] |= (flags[l] & 2) != 0;
+    any[3] |= (flags[l] & 1) != 0;
+  }
+  // Longest tiles first, so that the tail of a launch is made of short tiles: each
+  // product walks the layers in the order of ITS reduction length (dG for the first and
+  // fourth, dA for the second and third), through a descriptor table of its own.
   const size_t table_bytes = align256((size_t)layers * sizeof(LayerDesc));
-  LayerDesc* tables[2] = {(LayerDesc*)workspace, (LayerDesc*)((char*)workspace + table_bytes)};
-  char* tbase = (char*)workspace + 2 * table_bytes;
+  char* tbase = (char*)workspace + PRODUCTS * table_bytes;
   std::vector<size_t> toff(layers);
   size_t off = 0;
   for (int l = 0; l < layers; ++l) {
     toff[l] = off;
-    off += align256((size_t)dG[l] * dA[l] * sizeof(float));
+    off += align256((size_t)(flags ? 2 : 1) * dG[l] * dA[l] * sizeof(float));
   }
-  std::vector<int> order[2];
-  for (int pass = 0; pass < 2; ++pass) {
-    const int* key = pass == 0 ? dG : dA;
-    order[pass].resize(layers);
-    for (int l = 0; l < layers; ++l) order[pass][l] = l;
-    std::stable_sort(order[pass].begin(), order[pass].end(),
-                     [&](int a, int b) { return key[a] > key[b]; });
+  // work items of layer l in a product: its tiles, or none where it takes no part
+  auto items = [&](int product, int l) {
+    const int ta = cdiv(dA[l], BN), tg = cdiv(dG[l], BM);
+    const bool gfac = flags && (flags[l] & 1), afac = flags && (flags[l] & 2);
+    return (product < 2 || (product == 2 ? afac : gfac)) ? ta * tg : 0;
+  };
+  std::vector<int> order(layers);
+  for (int product = 0; product < PRODUCTS; ++product) {
+    if (!any[product]) continue;
+    LayerDesc* const table = (LayerDesc*)((char*)workspace + product * table_bytes);
+    const int* key = (product == 0 || product == 3) ? dG : dA;
+    for (int l = 0; l < layers; ++l) order[l] = l;
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return key[a] > key[b]; });
     for (int s0 = 0; s0 < layers; s0 += LAYER_CHUNK) {
       LayerChunk chunk;
       const int cnt = std::min(LAYER_CHUNK, layers - s0);
       for (int k = 0; k < cnt; ++k) {
-        const int l = order[pass][s0 + k];
+        const int l = order[s0 + k];
         LayerDesc& d = chunk.d[k];
         d.L = L[l];
         d.R = R[l];
@@ -171,33 +290,32 @@ static int run_layers(int layers, const int* dG, const int* dA, const float* con
         d.dA = dA[l];
         d.dAw = dA[l] - (has_bias[l] ? 1 : 0);
         d.scale = scale;
-        d.pad = 0;
+        d.flags = flags ? flags[l] : 0;
       }
       hipLaunchKernelGGL(layer_setup_kernel, dim3(1), dim3(LAYER_CHUNK), 0, stream, chunk,
-                         tables[pass], s0, cnt);
+                         table, s0, cnt);
     }
-  }
-  // both products have one tile per 128 x 128 block of the [dG, dA] result; every
-  // first product is enqueued before any second one (stream order is the dependency)
-  for (int pass = 0; pass < 2; ++pass) {
-    LayerDesc* const table = tables[pass];
+    // every launch of a product is enqueued before any of the next one (stream order is
+    // the dependency)
     for (int s0 = 0; s0 < layers; s0 += WL_MAX) {
       WorkList wl;
       wl.first = s0;
       wl.n = std::min(WL_MAX, layers - s0);
       wl.cum[0] = 0;
-      for (int i = 0; i < wl.n; ++i) {
-        const int l = order[pass][s0 + i];
-        wl.cum[i + 1] = wl.cum[i] + cdiv(dG[l], BM) * cdiv(dA[l], BN);
-      }
+      for (int i = 0; i < wl.n; ++i) wl.cum[i + 1] = wl.cum[i] + items(product, order[s0 + i]);
       for (int i = wl.n + 1; i <= WL_MAX; ++i) wl.cum[i] = wl.cum[wl.n];
+      if (wl.cum[wl.n] == 0) continue;
       const dim3 grid(wl.cum[wl.n]);
-      if (pass == 0) {
+      if (product == 0) {
         if (sample) KFAC_LAUNCH_TILE2(precond_first_kernel<true>, grid, stream, table, wl);
         else KFAC_LAUNCH_TILE2(precond_first_kernel<false>, grid, stream, table, wl);
-      } else {
+      } else if (product == 1) {
         if (sample) KFAC_LAUNCH_TILE2(precond_second_kernel<true>, grid, stream, table, wl);
         else KFAC_LAUNCH_TILE2(precond_second_kernel<false>, grid, stream, table, wl);
+      } else if (product == 2) {
+        KFAC_LAUNCH_TILE2(precond_third_kernel, grid, stream, table, wl);
+      } else {
+        KFAC_LAUNCH_TILE2(precond_fourth_kernel, grid, stream, table, wl);
       }
     }
   }
@@ -212,27 +330,57 @@ extern "C" {
 
 size_t kfac_precondition_workspace_bytes(int layers, const int* dG, const int* dA) {
   if (layers <= 0 || !dG || !dA) return 0;
-  return precond_workspace(layers, dG, dA);
+  return precond_workspace(layers, dG, dA, false);
+}
+
+static int check_layers(int layers, const int* dG, const int* dA, const float* const* Gop,
+                        const float* const* Aop, float* const* gradW, float* const* gradb,
+                        std::vector<int>& has_bias) {
+  if (layers < 0 || (layers > 0 && (!dG || !dA || !Gop || !Aop || !gradW || !gradb)))
+    return KFAC_ERR_ARG;
+  has_bias.resize(layers);
+  for (int l = 0; l < layers; ++l) {
+    if (dG[l] <= 0 || dA[l] <= 0 || !Gop[l] || !Aop[l] || !gradW[l]) return KFAC_ERR_ARG;
+    if ((int64_t)dA[l] * dA[l] > (int64_t)1 << 28 || (int64_t)dG[l] * dG[l] > (int64_t)1 << 28 ||
+        (int64_t)dA[l] * dG[l] > (int64_t)1 << 28)
+      return KFAC_ERR_ARG;
+    has_bias[l] = gradb[l] != nullptr;
+    if (has_bias[l] && dA[l] < 2) return KFAC_ERR_ARG;
+  }
+  return KFAC_OK;
 }
 
 int kfac_precondition_batched(int layers, const int* dG, const int* dA,
                               const float* const* Ginv, const float* const* Ainv,
                               float* const* gradW, float* const* gradb, void* workspace,
                               size_t workspace_bytes, void* stream) {
-  if (layers < 0 || (layers > 0 && (!dG || !dA || !Ginv || !Ainv || !gradW || !gradb)))
-    return KFAC_ERR_ARG;
-  std::vector<int> hb(layers);
-  for (int l = 0; l < layers; ++l) {
-    if (dG[l] <= 0 || dA[l] <= 0 || !Ginv[l] || !Ainv[l] || !gradW[l]) return KFAC_ERR_ARG;
-    if ((int64_t)dA[l] * dA[l] > (int64_t)1 << 28 || (int64_t)dG[l] * dG[l] > (int64_t)1 << 28 ||
-        (int64_t)dA[l] * dG[l] > (int64_t)1 << 28)
-      return KFAC_ERR_ARG;
-    hb[l] = gradb[l] != nullptr;
-    if (hb[l] && dA[l] < 2) return KFAC_ERR_ARG;
-  }
+  std::vector<int> hb;
+  const int st = check_layers(layers, dG, dA, Ginv, Ainv, gradW, gradb, hb);
+  if (st != KFAC_OK) return st;
   return run_layers(layers, dG, dA, Ginv, Ainv, (const float* const*)gradW,
                     (const float* const*)gradb, nullptr, nullptr, gradW, gradb, hb.data(), 1.f,
-                    false, workspace, workspace_bytes, (hipStream_t)stream);
+                    false, nullptr, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+size_t kfac_precondition_factored_workspace_bytes(int layers, const int* dG, const int* dA) {
+  if (layers <= 0 || !dG || !dA) return 0;
+  return precond_workspace(layers, dG, dA, true);
+}
+
+int kfac_precondition_factored_batched(int layers, const int* dG, const int* dA,
+                                       const float* const* Gop, const float* const* Aop,
+                                       const int* g_factored, const int* a_factored,
+                                       float* const* gradW, float* const* gradb, void* workspace,
+                                       size_t workspace_bytes, void* stream) {
+  std::vector<int> hb;
+  const int st = check_layers(layers, dG, dA, Gop, Aop, gradW, gradb, hb);
+  if (st != KFAC_OK) return st;
+  std::vector<int> flags(layers);
+  for (int l = 0; l < layers; ++l)
+    flags[l] = ((!g_factored || g_factored[l]) ? 1 : 0) | ((!a_factored || a_factored[l]) ? 2 : 0);
+  return run_layers(layers, dG, dA, Gop, Aop, (const float* const*)gradW,
+                    (const float* const*)gradb, nullptr, nullptr, gradW, gradb, hb.data(), 1.f,
+                    false, flags.data(), workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 int kfac_sample_batched(int layers, const int* dG, const int* dA, const float* const* U_G,
@@ -254,7 +402,8 @@ int kfac_sample_batched(int layers, const int* dG, const int* dA, const float* c
     if (hb[l] && (!meanb[l] || dA[l] < 2)) return KFAC_ERR_ARG;
   }
   return run_layers(layers, dG, dA, U_G, U_A, noise, nullptr, meanW, meanb, paramW, paramb,
-                    hb.data(), std_scale, true, workspace, workspace_bytes, (hipStream_t)stream);
+                    hb.data(), std_scale, true, nullptr, workspace, workspace_bytes,
+                    (hipStream_t)stream);
 }
 
 }  // extern "C"

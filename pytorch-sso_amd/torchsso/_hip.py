@@ -51,6 +51,12 @@ _SIGNATURES = {
                                                c_ptr, c_ptr, c_ptr, c_size, c_ptr]),
     'kfac_pi_damped_inverse_std_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
                                                    c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_size, c_ptr]),
+    'kfac_pi_damped_inverse_factored_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
+                                                        c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
+                                                        c_size, c_ptr]),
+    'kfac_precondition_factored_workspace_bytes': (c_size, [c_int, c_ptr, c_ptr]),
+    'kfac_precondition_factored_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
+                                                   c_ptr, c_ptr, c_ptr, c_size, c_ptr]),
     'kfac_damped_inverse_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
                                             c_ptr, c_size, c_ptr]),
     'kfac_static_workspace_bytes': (c_size, []),

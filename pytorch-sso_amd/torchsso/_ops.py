@@ -149,10 +149,9 @@ def pi_damped_inverse_batched(As, Gs, dampings, A_invs=None, G_invs=None, info=N
     return A_invs, G_invs, info
 
 
-def pi_damped_inverse_std_batched(As, Gs, dampings, A_invs, G_invs, A_stds, G_stds, info=None):
-    """pi_damped_inverse_batched that also writes, for the layers whose A_stds / G_stds entries
-    are tensors (None: no std for that layer), the upper Cholesky factors of the two inverses
-    (std^T std = inverse), read off the triangular inverse instead of a second factorisation."""
+def _pi_inverse_two_outputs(entry, As, Gs, dampings, A_invs, G_invs, A_others, G_others, info,
+                            check):
+    """Common part of the pi-damped inversions that write up to two results per matrix."""
     lib = _hip.load()
     layers = len(As)
     if layers == 0:
@@ -160,25 +159,71 @@ def pi_damped_inverse_std_batched(As, Gs, dampings, A_invs, G_invs, A_stds, G_st
     dev = As[0].device
     dA = _square_dims(As, 'A')
     dG = _square_dims(Gs, 'G')
-    for l, (a, g, sa, sg) in enumerate(zip(As, Gs, A_stds, G_stds)):
-        if (sa is None) != (sg is None):
-            raise _hip.KfacHipError('layer %d: std buffers must come in pairs' % l)
-        if sa is not None and (sa.shape != a.shape or sg.shape != g.shape):
-            raise _hip.KfacHipError('layer %d: std buffers have the wrong shape' % l)
+    for what, srcs, invs, others in (('A', As, A_invs, A_others), ('G', Gs, G_invs, G_others)):
+        for l, (x, i, o) in enumerate(zip(srcs, invs, others)):
+            check(l, what, i, o)
+            if any(t is not None and t.shape != x.shape for t in (i, o)):
+                raise _hip.KfacHipError('layer %d: output buffers of %s have the wrong shape' % (l, what))
     if info is None:
         info = torch.empty(2 * layers, dtype=torch.int32, device=dev)
     dims = []
     for a, g in zip(dA, dG):
         dims += [a, g]
     ws, ws_bytes = _hip.workspace(dev, lib.kfac_inverse_workspace_bytes(len(dims), _hip.int_array(dims)))
-    st = lib.kfac_pi_damped_inverse_std_batched(
+    st = getattr(lib, entry)(
         layers, _hip.int_array(dA), _hip.int_array(dG), _hip.ptr_array(As, 'A'),
-        _hip.ptr_array(Gs, 'G'), _hip.f32_array(dampings), _hip.ptr_array(A_invs, 'A_inv'),
-        _hip.ptr_array(G_invs, 'G_inv'), _hip.ptr_array(A_stds, 'A_std', True),
-        _hip.ptr_array(G_stds, 'G_std', True), info.data_ptr(), _ws_ptr(ws), ws_bytes,
+        _hip.ptr_array(Gs, 'G'), _hip.f32_array(dampings), _hip.ptr_array(A_invs, 'A_inv', True),
+        _hip.ptr_array(G_invs, 'G_inv', True), _hip.ptr_array(A_others, 'A output', True),
+        _hip.ptr_array(G_others, 'G output', True), info.data_ptr(), _ws_ptr(ws), ws_bytes,
         _hip.stream_ptr(dev))
-    _hip.check(st, 'kfac_pi_damped_inverse_std_batched')
+    _hip.check(st, entry)
     return info
+
+
+def pi_damped_inverse_std_batched(As, Gs, dampings, A_invs, G_invs, A_stds, G_stds, info=None):
+    """pi_damped_inverse_batched that also writes, for the matrices whose A_stds / G_stds entry
+    is a tensor (None: no std for it), the upper Cholesky factor of the inverse
+    (std^T std = inverse), read off the triangular inverse instead of a second factorisation."""
+    def check(l, what, inv, std):
+        if inv is None:
+            raise _hip.KfacHipError('layer %d: no buffer for the inverse of %s' % (l, what))
+    return _pi_inverse_two_outputs('kfac_pi_damped_inverse_std_batched', As, Gs, dampings,
+                                   A_invs, G_invs, A_stds, G_stds, info, check)
+
+
+def pi_damped_inverse_factored_batched(As, Gs, dampings, A_invs, G_invs, A_facs, G_facs, info=None):
+    """The pi-damped inverses, each in exactly one of two forms: the matrix itself (a tensor in
+    A_invs / G_invs, None in A_facs / G_facs) or only its upper-triangular factor Y with
+    Y Y^T = inverse (the other way round), for which the explicit inverse is never formed."""
+    def check(l, what, inv, fac):
+        if (inv is None) == (fac is None):
+            raise _hip.KfacHipError('layer %d: exactly one of inverse and factor must be asked for %s'
+                                    % (l, what))
+    return _pi_inverse_two_outputs('kfac_pi_damped_inverse_factored_batched', As, Gs, dampings,
+                                   A_invs, G_invs, A_facs, G_facs, info, check)
+
+
+def precondition_factored_batched(G_ops, A_ops, grad_ws, grad_bs, g_factored=None, a_factored=None):
+    """[gW | gb] <- G^-1 [gW | gb] A^-1 in place for every layer (gb may be None), with the
+    inverses given by their upper-triangular factors (Y Y^T = inverse) where the flag of that
+    side is true (no flag list: all of them), and as the explicit matrices elsewhere."""
+    lib = _hip.load()
+    layers = len(G_ops)
+    if layers == 0:
+        return
+    dev = G_ops[0].device
+    _square_dims(G_ops, 'G operand')
+    _square_dims(A_ops, 'A operand')
+    dG, dA = _kron_dims(G_ops, A_ops, grad_ws, grad_bs, 'precondition')
+    dGa, dAa = _hip.int_array(dG), _hip.int_array(dA)
+    flags = [None if f is None else _hip.int_array([int(bool(v)) for v in f])
+             for f in (g_factored, a_factored)]
+    ws, ws_bytes = _hip.workspace(dev, lib.kfac_precondition_factored_workspace_bytes(layers, dGa, dAa))
+    st = lib.kfac_precondition_factored_batched(
+        layers, dGa, dAa, _hip.ptr_array(G_ops, 'G operand'), _hip.ptr_array(A_ops, 'A operand'),
+        flags[0], flags[1], _hip.ptr_array(grad_ws, 'weight grad'),
+        _hip.ptr_array(grad_bs, 'bias grad', True), _ws_ptr(ws), ws_bytes, _hip.stream_ptr(dev))
+    _hip.check(st, 'kfac_precondition_factored_batched')
 
 
 def damped_inverse_batched(mats, damps=None, outs=None, info=None):

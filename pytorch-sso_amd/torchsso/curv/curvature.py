@@ -247,7 +247,17 @@ class KronCurvature(Curvature):
     kind = 'kron'
     _lanes_dealt = 0
 
+    # update_inv keeps the inverse of a factor with at least this many rows as its
+    # upper-triangular factor Y (Y Y^T = inverse) and preconditioning applies Y twice
+    # instead of the inverse once: the same work there, and the inversion is spared the
+    # product that forms the explicit inverse, a third of its work.  Below this size that
+    # product is negligible and a triangular operand only wastes tile space.  `inv` forms
+    # a missing inverse on first access.  None: update_inv forms every inverse explicitly.
+    factored_inverse_min_dim = 256
+
     def __init__(self, *args, **kwargs):
+        self._inv = None
+        self._inv_factors = [None, None]
         super(KronCurvature, self).__init__(*args, **kwargs)
         self._A = None
         self._G = None
@@ -257,6 +267,48 @@ class KronCurvature(Curvature):
         self._next = [None, None]        # receives the next running average
         self._fresh = [False, False]     # _next[i] holds the next average (hook ran since the last step)
         self._prev_ok = [False, False]   # _next[i] holds the average before the current one
+
+    # ---- inverses ---------------------------------------------------------------
+
+    @property
+    def inv(self):
+        """[A_inv, G_inv] (reference: curvature.py:302-312).  An inverse that update_inv kept
+        in factored form is formed here, on first access, as Y Y^T."""
+        if self._inv is not None:
+            for k, y in enumerate(self._inv_factors):
+                if self._inv[k] is None and y is not None:
+                    self._inv[k] = _ops.factor_linear(y.t().contiguous(), False, 1.)
+        return self._inv
+
+    @inv.setter
+    def inv(self, value):
+        self._inv = None if value is None else list(value)
+        self._inv_factors = [None, None]      # inverses given from outside have no factors
+
+    def _inverse_outputs(self, with_std):
+        """Output buffers for one update_inv of this layer, None where that output is not
+        wanted: ([A_inv, G_inv], [A_fac, G_fac], [A_std, G_std]).  A side is kept either as
+        the inverse or as its factor; with a posterior std to deliver (std^T std = inverse,
+        another factor than Y) every inverse is explicit."""
+        min_dim = None if with_std else self.factored_inverse_min_dim
+        old_inv = self._inv or [None, None]
+        old_std = self.std or [None, None]
+        invs, facs, stds = [None, None], [None, None], [None, None]
+
+        def reuse(t, like):
+            return t if t is not None and t.shape == like.shape else torch.empty_like(like)
+        for k, e in enumerate(self.ema):
+            if min_dim is not None and e.shape[0] >= min_dim:
+                facs[k] = reuse(self._inv_factors[k], e)
+            else:
+                invs[k] = reuse(old_inv[k], e)
+                if with_std:
+                    stds[k] = reuse(old_std[k], e)
+        self._inv = list(invs)
+        self._inv_factors = list(facs)
+        if with_std:
+            self.std = list(stds)
+        return invs, facs, stds
 
     # ---- raw factors ------------------------------------------------------------
 
@@ -442,24 +494,26 @@ def update_inv_all(curvs, with_std=()):
     full = [c for c in curvs if c.kind == 'full']
     wanted = {id(c) for c in with_std}
     if kron:
-        for c in kron:
-            if c.inv is None or c.inv[0].shape != c.ema[0].shape or c.inv[1].shape != c.ema[1].shape:
-                c.inv = [torch.empty_like(c.ema[0]), torch.empty_like(c.ema[1])]
-            if id(c) in wanted and (c.std is None
-                                    or any(s.shape != i.shape for s, i in zip(c.std, c.inv))):
-                c.std = [torch.empty_like(i) for i in c.inv]
-        args = ([c.ema[0] for c in kron], [c.ema[1] for c in kron], [c.damping for c in kron],
-                [c.inv[0] for c in kron], [c.inv[1] for c in kron])
-        if any(id(c) in wanted for c in kron):
-            info = _ops.pi_damped_inverse_std_batched(
-                *args, [c.std[0] if id(c) in wanted else None for c in kron],
-                [c.std[1] if id(c) in wanted else None for c in kron])
+        outs = [c._inverse_outputs(id(c) in wanted) for c in kron]
+        column = lambda which, k: [o[which][k] for o in outs]
+        args = ([c.ema[0] for c in kron], [c.ema[1] for c in kron], [c.damping for c in kron])
+        if any(f is not None for _, facs, _ in outs for f in facs):
+            # (a layer with a std to deliver has no factored side, but others may: its std
+            # then takes a launch of its own below)
+            info = _ops.pi_damped_inverse_factored_batched(*args, column(0, 0), column(0, 1),
+                                                           column(1, 0), column(1, 1))
+            for c in kron:
+                if id(c) in wanted:
+                    c._std_current = False
+        elif wanted:
+            info = _ops.pi_damped_inverse_std_batched(*args, column(0, 0), column(0, 1),
+                                                      column(2, 0), column(2, 1))
             for c in kron:
                 if id(c) in wanted:
                     c._std_current = True      # update_std_all has nothing to do for it
                     c.std_info = None          # (a failure shows in `info`)
         else:
-            _, _, info = _ops.pi_damped_inverse_batched(*args)
+            _, _, info = _ops.pi_damped_inverse_batched(*args, column(0, 0), column(0, 1))
         for i, c in enumerate(kron):
             c.info = info[2 * i:2 * i + 2]
     if diag:
@@ -493,9 +547,10 @@ def update_std_all(curvs):
             kron.append(c)
     mats, outs = [], []
     for c in kron:
-        if c.std is None or any(s.shape != i.shape for s, i in zip(c.std, c.inv)):
-            c.std = [torch.empty_like(i) for i in c.inv]
-        mats.extend(c.inv)
+        inv = c.inv                            # (forms an inverse kept in factored form)
+        if c.std is None or any(s is None or s.shape != i.shape for s, i in zip(c.std, inv)):
+            c.std = [torch.empty_like(i) for i in inv]
+        mats.extend(inv)
         outs.extend(c.std)
     if mats:
         _, info = _ops.cholesky_upper_batched(mats, outs)
@@ -565,24 +620,24 @@ def precondition_all(pairs):
     """precondition_grad for a list of (curvature, params): grads are replaced
     in place by G^-1 [dW|db] A^-1 (reference: cov/linear.py:69-84,
     cov/conv.py:76-92) or inv * grad (curvature.py:234-238)."""
-    Gi, Ai, gw, gb = [], [], [], []
+    kron = ([], [], [], [], [], [])     # G operand, A operand, gW, gb, G is a factor, A is a factor
     dinv, dgrad = [], []
     for c, params in pairs:
         if c.kind == 'kron':
-            A_inv, G_inv = c.inv
             w = params[0]
             if not w.grad.is_contiguous():
                 w.grad = w.grad.contiguous()
-            Gi.append(G_inv)
-            Ai.append(A_inv)
-            gw.append(w.grad)
+            gb = None
             if c.bias:
                 b = params[1]
                 if not b.grad.is_contiguous():
                     b.grad = b.grad.contiguous()
-                gb.append(b.grad)
-            else:
-                gb.append(None)
+                gb = b.grad
+            fa, fg = c._inv_factors
+            for lst, v in zip(kron, (fg if fg is not None else c._inv[1],
+                                     fa if fa is not None else c._inv[0],
+                                     w.grad, gb, fg is not None, fa is not None)):
+                lst.append(v)
         elif c.kind == 'diag':
             for p, inv in zip(params, c.inv):
                 if not p.grad.is_contiguous():
@@ -590,8 +645,11 @@ def precondition_all(pairs):
                 dinv.append(inv)
                 dgrad.append(p.grad)
         # 'full' curvatures do not precondition (reference: cov/linear.py:24-25)
-    if Gi:
-        _ops.precondition_batched(Gi, Ai, gw, gb)
+    if any(kron[4]) or any(kron[5]):
+        # one call for all layers, explicit ones included: every product is then one launch
+        _ops.precondition_factored_batched(*kron)
+    elif kron[0]:
+        _ops.precondition_batched(*kron[:4])
     if dinv:
         _ops.diag_precondition_batched(dinv, dgrad)
 

@@ -219,6 +219,28 @@ class OracleOps(object):
                 std.copy_(O.cholesky_upper(inv, self.dtype))
         return info
 
+    def pi_damped_inverse_factored_batched(self, As, Gs, dampings, A_invs, G_invs, A_facs, G_facs,
+                                           info=None):
+        ra, rg, info = self.pi_damped_inverse_batched(As, Gs, dampings)
+        for res, invs, facs in ((ra, A_invs, A_facs), (rg, G_invs, G_facs)):
+            for r, inv, fac in zip(res, invs, facs):
+                assert (inv is None) != (fac is None)
+                if inv is not None:
+                    inv.copy_(r)
+                else:
+                    # the upper Y with Y Y^T = r: the lower Cholesky factor of r with rows
+                    # and columns reversed, reversed back
+                    low = torch.linalg.cholesky(r.double().flip(0, 1))
+                    fac.copy_(low.flip(0, 1).to(r.dtype))
+        return info
+
+    def precondition_factored_batched(self, G_ops, A_ops, grad_ws, grad_bs, g_factored=None,
+                                      a_factored=None):
+        def explicit(ops, flags):
+            return [op @ op.t() if flags is None or flags[l] else op for l, op in enumerate(ops)]
+        self.precondition_batched(explicit(G_ops, g_factored), explicit(A_ops, a_factored),
+                                  grad_ws, grad_bs)
+
     def damped_inverse_batched(self, mats, damps=None, outs=None, info=None):
         res = [O.damped_inverse(m, 0. if damps is None else damps[i], self.dtype)
                for i, m in enumerate(mats)]

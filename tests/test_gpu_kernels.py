@@ -258,6 +258,91 @@ def test_inverse_with_posterior_std_from_the_same_factorisation(ops, dev):
     assert worst['inverse'] < TOL and worst['std'] < TOL and worst['std^T std vs inverse'] < 1e-5
 
 
+def test_inverse_in_factored_form(ops, dev):
+    """kfac_pi_damped_inverse_factored_batched: per matrix either the inverse or only its
+    upper-triangular factor Y (Y Y^T = inverse, zeros below the diagonal), for which no
+    explicit inverse is formed.  Every combination per layer in one call; Y against the
+    inverse of the float64 Cholesky factor, Y Y^T and the explicit inverses against the
+    float64 inverse; ragged sizes around the 128-blocks."""
+    gen = torch.Generator().manual_seed(12)
+    pairs = [(1, 2), (64, 33), (127, 129), (10, 700), (192, 385), (1025, 128), (257, 1500), (300, 513)]
+    As, Gs = [], []
+    for dA, dG in pairs:
+        for n, lst in ((dA, As), (dG, Gs)):
+            a = torch.randn(n, n + 8, generator=gen).to(dev)
+            lst.append((a @ a.t() / (n + 8)).contiguous())
+    damp = [1e-3 * (l + 1) for l in range(len(pairs))]
+    nan = lambda x: torch.full_like(x, float('nan'))
+    # per layer: the form asked for A and for G ('f' factor, 'i' inverse)
+    plan = ['ff', 'fi', 'if', 'ff', 'fi', 'ff', 'ii', 'if']
+    Ai = [nan(a) if p[0] == 'i' else None for a, p in zip(As, plan)]
+    Gi = [nan(g) if p[1] == 'i' else None for g, p in zip(Gs, plan)]
+    Af = [nan(a) if p[0] == 'f' else None for a, p in zip(As, plan)]
+    Gf = [nan(g) if p[1] == 'f' else None for g, p in zip(Gs, plan)]
+    info = ops.pi_damped_inverse_factored_batched(As, Gs, damp, Ai, Gi, Af, Gf)
+    assert info.cpu().tolist() == [0] * (2 * len(pairs))
+    eye = lambda n: torch.eye(n, dtype=D, device=dev)
+    worst = {'factor': 0., 'Y Y^T vs inverse': 0., 'inverse': 0.}
+    for l, (a, g) in enumerate(zip(As, Gs)):
+        pi = ((a.double().diagonal().sum() / a.shape[0]) / (g.double().diagonal().sum() / g.shape[0])).sqrt()
+        r = damp[l] ** 0.5
+        for X, shift, inv, y in ((a, r * pi, Ai[l], Af[l]), (g, r / pi, Gi[l], Gf[l])):
+            Xd = X.double() + shift * eye(X.shape[0])
+            ref = torch.linalg.inv(Xd)
+            if inv is not None:
+                assert torch.equal(inv, inv.t())
+                worst['inverse'] = max(worst['inverse'], ((inv.double() - ref).norm() / ref.norm()).item())
+            else:
+                assert torch.equal(y, torch.triu(y)) and bool((y.diagonal() > 0).all())
+                refY = torch.linalg.inv(torch.linalg.cholesky(Xd).mT)     # X = R^T R, Y = R^-1
+                Y = y.double()
+                worst['factor'] = max(worst['factor'], ((Y - refY).norm() / refY.norm()).item())
+                worst['Y Y^T vs inverse'] = max(worst['Y Y^T vs inverse'],
+                                                ((Y @ Y.t() - ref).norm() / ref.norm()).item())
+    print('factored inverse, worst rel. Frobenius errors:', {k: '%.2e' % v for k, v in worst.items()})
+    assert max(worst.values()) < TOL
+    with pytest.raises(Exception, match='exactly one of inverse and factor'):
+        ops.pi_damped_inverse_factored_batched(As[:1], Gs[:1], damp[:1], [None], [nan(Gs[0])],
+                                               [None], [None])
+
+
+def test_precondition_with_factored_inverses(ops, dev):
+    """kfac_precondition_factored_batched: G^-1 [gW | gb] A^-1 with each side given either by
+    its upper-triangular factor Y (Y Y^T = inverse, applied twice) or by the explicit inverse,
+    all four combinations, against the float64 product with the explicit inverses; with and
+    without bias column, sizes on both sides of the 128-tiles, more layers than one table
+    chunk holds.  The strict lower triangles of the factor buffers hold zeros, as the
+    inversion leaves them."""
+    torch.manual_seed(21)
+    shapes = SHAPES + [(257, 640, True), (385, 129, False), (1100, 300, True), (640, 900, True)] \
+        + [(1 + (13 * i) % 140, 2 + (29 * i) % 260, i % 2 == 0) for i in range(135)]
+    Gy = [torch.triu(torch.randn(g, g) / g ** 0.5 + torch.eye(g)) for g, a, b in shapes]
+    Ay = [torch.triu(torch.randn(a, a) / a ** 0.5 + torch.eye(a)) for g, a, b in shapes]
+    gfac = [i % 4 in (0, 1) for i in range(len(shapes))]
+    afac = [i % 4 in (0, 2) for i in range(len(shapes))]
+    Ginv = [y.double() @ y.double().t() for y in Gy]
+    Ainv = [y.double() @ y.double().t() for y in Ay]
+    Gop = [(y if f else i.float()).to(dev) for y, i, f in zip(Gy, Ginv, gfac)]
+    Aop = [(y if f else i.float()).to(dev) for y, i, f in zip(Ay, Ainv, afac)]
+    gws = [torch.randn(g, a - (1 if b else 0)) for g, a, b in shapes]
+    gbs = [torch.randn(g) if b else None for g, a, b in shapes]
+    for flags in ((gfac, afac), (None, None)):
+        dgw = [x.to(dev).clone() for x in gws]
+        dgb = [None if x is None else x.to(dev).clone() for x in gbs]
+        if flags[0] is None:        # no flag arrays: every operand is a factor
+            ops.precondition_factored_batched([y.to(dev) for y in Gy], [y.to(dev) for y in Ay], dgw, dgb)
+        else:
+            ops.precondition_factored_batched(Gop, Aop, dgw, dgb, gfac, afac)
+        worst = 0.
+        for i in range(len(shapes)):
+            rw, rb = O.precondition(Ginv[i], Ainv[i], gws[i], gbs[i], D)
+            errs = [O.rel_fro(dgw[i], rw)] + ([] if rb is None else [O.rel_fro(dgb[i], rb)])
+            worst = max([worst] + errs)
+            assert max(errs) < TOL, (shapes[i], gfac[i], afac[i])
+        print('factored preconditioning over %d layers (%s): worst rel. Frobenius error %.2e'
+              % (len(shapes), 'mixed' if flags[0] else 'all factored', worst))
+
+
 SHAPES = [(10, 193, True), (64, 76, True), (1000, 785, True), (128, 1601, True),
           (512, 1152, False), (1, 2, True), (3, 1, False), (64, 64, False), (130, 257, True)]
 

@@ -16,8 +16,14 @@ import kfac_testlib as T
 from oracle import kfac_oracle as O
 
 
-@pytest.fixture
-def oracle_ops(monkeypatch):
+# rows from which update_inv keeps an inverse as its triangular factor: the library's
+# default (beyond every test network: all inverses explicit), every factor, and a value
+# that splits the test networks' layers into sides of both kinds
+@pytest.fixture(params=[None, 1, 20], ids=['explicit', 'factored', 'mixed'])
+def oracle_ops(monkeypatch, request):
+    from torchsso.curv.curvature import KronCurvature
+    if request.param is not None:
+        monkeypatch.setattr(KronCurvature, 'factored_inverse_min_dim', request.param)
     fake = T.OracleOps()
     for name in dir(fake):
         if not name.startswith('_') and callable(getattr(fake, name)) and hasattr(_ops, name):
@@ -248,13 +254,19 @@ def test_check_spd_raises_and_names_the_layer(oracle_ops, monkeypatch):
     opt = torchsso.optim.SecondOrderOptimizer(model, 'Cov', {'Linear': 'Kron'}, {'damping': 1e-3},
                                               check_spd=True)
     opt.step(closure=_closure(model, x, y))        # healthy factors: no complaint
-    real = oracle_ops.pi_damped_inverse_batched
+    real, real_fac = oracle_ops.pi_damped_inverse_batched, oracle_ops.pi_damped_inverse_factored_batched
 
     def failing(As, Gs, dampings, A_invs=None, G_invs=None, info=None):
         a, g, info = real(As, Gs, dampings, A_invs, G_invs, info)
         info[3] = 2                                 # layer 1, factor G, leading minor 2
         return a, g, info
+
+    def failing_factored(*args, **kwargs):
+        info = real_fac(*args, **kwargs)
+        info[3] = 2
+        return info
     monkeypatch.setattr(_ops, 'pi_damped_inverse_batched', failing)
+    monkeypatch.setattr(_ops, 'pi_damped_inverse_factored_batched', failing_factored)
     with pytest.raises(NotPositiveDefiniteError, match=r'layer 1 \(Linear\): inverse of factor G.*order 2'):
         opt.step(closure=_closure(model, x, y))
     opt.check_spd = False                           # the default: nothing is read
