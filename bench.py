@@ -350,9 +350,9 @@ class LayerSet(object):
 
 def time_steps(step, steps, warmup):
     """(ms per step by the slower of HIP events and the host clock, ms by events, host
-    enqueue ms per step).  The third figure is the host's own time to enqueue a step with no
-    synchronisation in between (Python + ctypes + launch calls), taken over a second run of
-    the same steps; where it approaches the first, the step is bound by the host."""
+    enqueue ms per step).  The third figure is the host's own time to enqueue one step
+    (Python + ctypes + launch calls; the median over steps that each start on an idle
+    device); where it approaches the first, the step is bound by the host."""
     import torch
     for _ in range(warmup):
         step()
@@ -366,11 +366,17 @@ def time_steps(step, steps, warmup):
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     ev_ms = start.elapsed_time(end) / steps
-    t0 = time.perf_counter()
-    for _ in range(steps):
+    # host enqueue time: each step starts on an idle device (with a backlog of several steps
+    # the runtime makes the host wait for queue space, and the figure would drift towards the
+    # device time)
+    host = []
+    for _ in range(min(steps, 10)):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
         step()
-    host_ms = (time.perf_counter() - t0) * 1e3 / steps
+        host.append(time.perf_counter() - t0)
     torch.cuda.synchronize()
+    host_ms = sorted(host)[len(host) // 2] * 1e3
     return max(wall_ms, ev_ms), ev_ms, host_ms
 
 
@@ -712,6 +718,10 @@ def main():
     ap.add_argument('--workload', default='resnet50', choices=sorted(WORKLOADS) + ['noisy_kfac', 'resnet50_train'])
     ap.add_argument('--factor-streams', type=int, default=None,
                     help='side streams for the factor products (library default: 3; 0 = none)')
+    ap.add_argument('--factor-mode', default=None, choices=['grouped', 'eager'],
+                    help='grouped (library default): the hooks queue their factor products and one '
+                         'engine call runs them all; eager: a launch sequence per product, on the '
+                         'side streams')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--factored-min-dim', type=int, default=None,
                     help='rows from which update_inv keeps an inverse as its triangular factor '
@@ -735,7 +745,9 @@ def main():
     import torchsso
     if args.factor_streams is not None:
         torchsso.set_factor_streams(args.factor_streams)
-    factor_streams = torchsso.factor_streams()
+    if args.factor_mode is not None:
+        torchsso.set_factor_mode(args.factor_mode)
+    factor_streams = torchsso.factor_streams() if torchsso.factor_mode() == 'eager' else 0
     from torchsso.curv.curvature import KronCurvature
     if args.explicit_inverse:
         KronCurvature.factored_inverse_min_dim = None
@@ -795,7 +807,7 @@ def main():
                    'kron_layers': sum(1 for s in specs if s['kind'] != 'bn'),
                    'bn_layers': sum(1 for s in specs if s['kind'] == 'bn'),
                    'damping': 1e-3, 'ema_decay': 0.95, 'invert_every_step': True, 'inverse_form': inverse_form,
-                   'factor_side_streams': factor_streams,
+                   'factor_mode': torchsso.factor_mode(), 'factor_side_streams': factor_streams,
                    'inputs_resident_GB': round(resident / 1e9, 3)},
         'tflops': round(total_flops / (ms * 1e-3) / 1e12, 2),
         'algorithmic_gflop': {k: round(v / 1e9, 1) for k, v in work.items() if not k.endswith('bytes')},

@@ -99,6 +99,49 @@ int kfac_factor_conv_g(const float* g, int n, int c, int h, int w,
                        float alpha, float beta, const float* C_prev, float* C,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- Grouped factor build (the products of many layers in one call) ------ */
+
+#define KFAC_FACTOR_LINEAR 0   /* kfac_factor_linear: x is [rows, c], ldx = c */
+#define KFAC_FACTOR_CONV_A 1   /* kfac_factor_conv_a: x is [rows, c, H, W] */
+#define KFAC_FACTOR_CONV_G 2   /* kfac_factor_conv_g: x is [rows, c, H, W] (H, W of the output) */
+
+/* One product of a grouped call: the arguments of the single-product entry point of
+ * its `kind` (fields that kind does not use are ignored). */
+typedef struct kfac_factor_job {
+  int kind;
+  int add_bias;
+  const float* x;            /* device */
+  int64_t rows;              /* linear: rows of x; conv: batch size n */
+  int c, H, W;
+  int kh, kw, sh, sw, ph, pw, dh, dw;     /* KFAC_FACTOR_CONV_A only */
+  float alpha, beta;
+  const float* C_prev;       /* device, may be NULL (see kfac_factor_linear) */
+  float* C;                  /* device */
+} kfac_factor_job;
+
+/* Scratch for kfac_factor_grouped on this list (`jobs` is a HOST array): the device
+ * tables of its launches, the k-split partials of all products at once, and the scratch
+ * of the products that go through their single-product routine. */
+size_t kfac_factor_grouped_workspace_bytes(int count, const kfac_factor_job* jobs);
+
+/* Every product of the list, C_i = alpha_i * P_i^T P_i + beta_i * C_prev_i, with the same
+ * results as `count` calls of kfac_factor_linear / kfac_factor_conv_a / kfac_factor_conv_g
+ * up to the summation order of the k-splits, in a handful of launches: one per operand
+ * kind and tile size holds the (tile, k-split) work items of all its products, longest
+ * first, and two more reduce the partial sums of all of them.  For a host that collects
+ * the factor products of a whole forward / backward pass (hooks of
+ * torchsso/curv/curvature.py:118-155 calling cov/linear.py:50-67 and cov/conv.py:47-74
+ * layer by layer) and hands them over before the first reader of a factor: a launch per
+ * layer drains and refills the chip a hundred times per step.  The outputs C_i must be
+ * distinct buffers, and no C_i may be an input or C_prev of another product of the call.
+ * Stride-1 k x k convolution inputs (the correlation kernels) and inputs above 1 GiB run
+ * through their single-product routines on the same stream. */
+int kfac_factor_grouped(int count, const kfac_factor_job* jobs, void* workspace,
+                        size_t workspace_bytes, void* stream);
+
+/* Plan query: the fp32 MFMA flops kfac_factor_grouped executes for this list. */
+double kfac_factor_grouped_executed_flops(int count, const kfac_factor_job* jobs);
+
 /* ---- Damped factor inversion ------------------------------------------- */
 
 /* Scratch for the three batched routines below: a descriptor table plus one

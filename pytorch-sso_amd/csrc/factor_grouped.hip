@@ -1,0 +1,608 @@
+// Grouped Kronecker factor build: the symmetric products of MANY layers in a handful of
+// launches.
+//
+// A factor product depends only on the tensor its hook was handed and nothing reads it
+// before the optimizer step, so the host may collect the products of a whole
+// forward / backward pass and hand them over together.  One launch per operand kind
+// and tile configuration then holds the (tile, k-split) work items of all its products,
+// longest first: a launch of thousands of items keeps every CU busy until its end,
+// where a launch per product (a few hundred items, often fewer) drains and refills the
+// chip a hundred times per step; the k-split partials of all products are reduced by
+// two more launches at the end instead of one or two per product.
+//
+//   work item -> product: binary search in the table of first items (uniform per
+//   workgroup, scalar loads); inside a product the items are renumbered so that each
+//   XCD (own L2) walks a contiguous run of (split, tile) pairs, tile fastest, as in
+//   the single-product kernel.
+//
+// Products whose input exceeds the 1 GiB addressing window of an operand, and the
+// stride-1 k x k layers served by the correlation kernels, are handed to their
+// single-product routines on the same stream.
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+#include <vector>
+
+#include "common.h"
+#include "operands.h"
+#include "syrk_reduce.h"
+
+namespace kfac {
+
+// ---- device tables -----------------------------------------------------------
+
+template <class OP>
+struct SyJob {
+  OP op;
+  float* C;
+  const float* Cin;
+  float* ws;            // partials of this product (splits > 1)
+  int d, K, T, ntiles, splits, cps;
+  float alpha, beta;
+};
+
+struct RdJob {
+  const float* ws;
+  float* C;
+  const float* Cin;
+  int d, T, ntiles, splits;
+  float alpha, beta;
+};
+
+// tables reach the device as kernel arguments, a chunk per launch
+constexpr int BLOB_WORDS = 960;     // 3840 bytes
+struct Blob {
+  unsigned w[BLOB_WORDS];
+};
+__global__ __launch_bounds__(256) void upload_kernel(Blob blob, unsigned* dst, int words) {
+  for (int i = threadIdx.x; i < words; i += 256) dst[i] = blob.w[i];
+}
+
+// first table entry whose range holds `item` (cum[j] <= item < cum[j + 1])
+__device__ __forceinline__ int find_job(const int* __restrict__ cum, int njobs, int item) {
+  int lo = 0, hi = njobs;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cum[mid] <= item) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// Workgroups go to the 8 XCDs round-robin by dispatch index g.  The n items of one
+// product occupy the dispatch indices [c0, c0 + n); this permutation of [0, n) gives
+// every XCD a contiguous run of them.
+__device__ __forceinline__ int xcd_remap_range(int g, int c0, int n) {
+  const int s = c0 & 7;
+  const int v = g - c0 + s;        // index in a virtual range that starts at a multiple of 8
+  const int x = v & 7;
+  const int tv = n + s;
+  int base = 0;
+#pragma unroll
+  for (int y = 0; y < 8; ++y) {
+    const int cnt = ((tv - y + 7) >> 3) - (y < s ? 1 : 0);
+    base += y < x ? cnt : 0;
+  }
+  return base + (v >> 3) - (x < s ? 1 : 0);
+}
+
+template <class OP, int W>
+__global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void syrk_grouped_kernel(
+    const SyJob<OP>* __restrict__ jobs, const int* __restrict__ cum, int njobs) {
+  constexpr int TS = 64 * W;
+  constexpr int KC = Cfg<W, W>::KC;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  const int g = blockIdx.x;
+  const int j = find_job(cum, njobs, g);
+  const SyJob<OP>& jb = jobs[j];
+  const int c0 = cum[j];
+  const int ntiles = jb.ntiles, splits = jb.splits;
+  const int item = xcd_remap_range(g, c0, ntiles * splits);
+  const int tile = item % ntiles;
+  const int split = item / ntiles;
+  int bi, bj;
+  upper_tile(tile, jb.T, bi, bj);
+  const int K = jb.K, d = jb.d;
+  const int kbeg = split * jb.cps * KC;
+  int kend = kbeg + jb.cps * KC;
+  if (kend > K) kend = K;
+  const OP op = jb.op;
+  if (splits == 1) {
+    EpiStore epi{jb.C, d, d, d, jb.alpha, jb.beta, bi != bj, jb.Cin};
+    gemm_tile_cfg<W, W>(op, op, bi * TS, bj * TS, kbeg, kend, bi == bj, epi, smem);
+  } else {
+    EpiPartial epi{jb.ws + ((size_t)split * ntiles + tile) * (TS * TS), bi * TS, bj * TS, d, d, TS};
+    gemm_tile_cfg<W, W>(op, op, bi * TS, bj * TS, kbeg, kend, bi == bj, epi, smem);
+  }
+}
+
+// many splits: item = (tile, row of the tile, 64-wide segment)
+template <int TS>
+__global__ __launch_bounds__(256) void reduce_many_grouped_kernel(const RdJob* __restrict__ jobs,
+                                                                  const int* __restrict__ cum,
+                                                                  int njobs) {
+  const int j = find_job(cum, njobs, blockIdx.x);
+  const RdJob jb = jobs[j];
+  const int local = blockIdx.x - cum[j];
+  constexpr int PER_TILE = TS * (TS / 64);
+  const int tile = local / PER_TILE;
+  syrk_reduce_many<TS>(jb.ws, jb.d, jb.T, jb.ntiles, jb.splits, jb.C, jb.Cin, jb.alpha, jb.beta,
+                       tile, local - tile * PER_TILE);
+}
+
+// few splits: item = (tile, 32-row block, 64-column block)
+template <int TS>
+__global__ __launch_bounds__(256) void reduce_tile_grouped_kernel(const RdJob* __restrict__ jobs,
+                                                                  const int* __restrict__ cum,
+                                                                  int njobs) {
+  const int j = find_job(cum, njobs, blockIdx.x);
+  const RdJob jb = jobs[j];
+  const int local = blockIdx.x - cum[j];
+  constexpr int CB = TS / 64, PER_TILE = (TS / 32) * CB;
+  const int tile = local / PER_TILE;
+  const int rem = local - tile * PER_TILE;
+  syrk_reduce_tile<TS>(jb.ws, jb.d, jb.T, jb.ntiles, jb.splits, jb.C, jb.Cin, jb.alpha, jb.beta,
+                       tile, rem / CB, rem % CB);
+}
+
+// ---- host side -----------------------------------------------------------------
+
+// Items of a grouped launch are dispatched longest first and the launch holds many of
+// them, so an item may be long: about this many 16-deep chunks, which keeps the
+// partial tiles that a split writes and the reduction reads small beside the input.
+constexpr int GROUP_TARGET_CPS_W2 = 96;
+constexpr int GROUP_TARGET_CPS_W1 = 192;
+constexpr int MANY_SPLITS = 16;          // above: the reduction with 16 split lanes
+
+struct GroupPlan {
+  int w, ts, T, ntiles, splits, cps;
+  size_t partial_floats() const {
+    return splits > 1 ? (size_t)splits * ntiles * ts * ts : 0;
+  }
+};
+
+static int env_int(const char* name, int dflt) {
+  const char* s = getenv(name);
+  return s && *s ? atoi(s) : dflt;
+}
+
+static GroupPlan plan_group(int d, long K, long target) {
+  GroupPlan p;
+  p.w = d <= 256 ? 1 : 2;
+  p.ts = 64 * p.w;
+  p.T = cdiv(d, p.ts);
+  p.ntiles = p.T * (p.T + 1) / 2;
+  const long nchunks = (K + 15) / 16;
+  long splits = (nchunks + target / 2) / target;
+  if (splits < 1) splits = 1;
+  long cps = (nchunks + splits - 1) / splits;
+  splits = (nchunks + cps - 1) / cps;
+  p.splits = (int)splits;
+  p.cps = (int)cps;
+  return p;
+}
+
+// Chunks per item for one launch: the default when the launch holds plenty of items at that
+// length, shorter items when it would not fill the chip twice (resident workgroups: 3 per CU
+// of four waves, 8 per CU of one wave).
+static long launch_target(int w, double total_units) {
+  static const int t2 = env_int("KFAC_GROUP_CPS2", GROUP_TARGET_CPS_W2);
+  static const int t1 = env_int("KFAC_GROUP_CPS1", GROUP_TARGET_CPS_W1);
+  const long dflt = w == 1 ? t1 : t2;
+  const double slots = w == 1 ? 2048. : 768.;
+  long t = (long)(total_units / (2. * slots));
+  if (t > dflt) t = dflt;
+  if (t < 8) t = 8;
+  return t;
+}
+
+enum Path { P_DENSE, P_CONVG, P_CONVA, P_TAPS, P_SINGLE, P_BAD };
+
+struct Classified {
+  Path path;
+  int d;
+  long K;
+  int OH, OW;
+};
+
+static Classified classify(const kfac_factor_job& j) {
+  Classified c{P_BAD, 0, 0, 0, 0};
+  if (j.rows <= 0 || j.c <= 0) return c;
+  const int bias = j.add_bias ? 1 : 0;
+  if (j.kind == KFAC_FACTOR_LINEAR) {
+    c.d = j.c + bias;
+    c.K = j.rows;
+    if ((int64_t)c.d * c.d * 4 > MAX_OPERAND_BYTES) return c;
+    c.path = (int64_t)j.rows * j.c * 4 <= MAX_OPERAND_BYTES ? P_DENSE : P_SINGLE;
+    return c;
+  }
+  if (j.rows > INT32_MAX || j.H <= 0 || j.W <= 0) return c;
+  const int64_t tensor_bytes = (int64_t)j.rows * j.c * j.H * j.W * 4;
+  if (j.kind == KFAC_FACTOR_CONV_G) {
+    c.d = j.c;
+    c.K = (long)j.rows * j.H * j.W;
+    if ((int64_t)c.d * c.d * 4 > MAX_OPERAND_BYTES) return c;
+    c.path = tensor_bytes <= MAX_OPERAND_BYTES && c.K <= INT32_MAX ? P_CONVG : P_SINGLE;
+    return c;
+  }
+  if (j.kind != KFAC_FACTOR_CONV_A) return c;
+  if (j.kh <= 0 || j.kw <= 0 || j.sh <= 0 || j.sw <= 0 || j.ph < 0 || j.pw < 0 || j.dh <= 0 ||
+      j.dw <= 0)
+    return c;
+  if (j.H >= 16384 || j.W >= 16384 || j.kh * j.dh >= 16384 || j.kw * j.dw >= 16384) return c;
+  c.OH = (j.H + 2 * j.ph - j.dh * (j.kh - 1) - 1) / j.sh + 1;
+  c.OW = (j.W + 2 * j.pw - j.dw * (j.kw - 1) - 1) / j.sw + 1;
+  if (c.OH <= 0 || c.OW <= 0) return c;
+  const int64_t dd = (int64_t)j.c * j.kh * j.kw + bias;
+  if (dd * dd * 4 > MAX_OPERAND_BYTES) return c;
+  c.d = (int)dd;
+  c.K = (long)j.rows * c.OH * c.OW;
+  if (tensor_bytes > MAX_OPERAND_BYTES || c.K > INT32_MAX) {
+    c.path = P_SINGLE;
+  } else if (j.kh == 1 && j.kw == 1 && j.sh == 1 && j.sw == 1 && j.ph == 0 && j.pw == 0 && !bias) {
+    c.path = P_CONVG;          // a pointwise convolution: M is the input viewed as [c, n*H*W]
+  } else if (conv_a_taps_applicable(j.c, j.kh, j.kw, j.sh, j.sw, bias) &&
+             conv_a_taps_workspace((int)j.rows, j.c, j.H, j.W, j.kh, j.kw, j.ph, j.pw, j.dh,
+                                   j.dw) > 0) {
+    c.path = P_TAPS;
+  } else {
+    c.path = P_CONVA;
+  }
+  return c;
+}
+
+static size_t single_workspace(const kfac_factor_job& j, const Classified& c) {
+  if (j.kind == KFAC_FACTOR_CONV_A)
+    return kfac_factor_conv_a_workspace_bytes((int)j.rows, j.c, j.H, j.W, j.kh, j.kw, j.sh, j.sw,
+                                              j.ph, j.pw, j.dh, j.dw, j.add_bias ? 1 : 0);
+  // (linear / conv G in slices: the largest slice is the whole reduction at most)
+  return kfac_factor_workspace_bytes(c.d, c.K);
+}
+
+static int run_single(const kfac_factor_job& j, void* ws, size_t ws_bytes, void* stream) {
+  switch (j.kind) {
+    case KFAC_FACTOR_LINEAR:
+      return kfac_factor_linear(j.x, j.rows, j.c, j.c, j.add_bias, j.alpha, j.beta, j.C_prev, j.C,
+                                ws, ws_bytes, stream);
+    case KFAC_FACTOR_CONV_G:
+      return kfac_factor_conv_g(j.x, (int)j.rows, j.c, j.H, j.W, j.alpha, j.beta, j.C_prev, j.C, ws,
+                                ws_bytes, stream);
+    default:
+      return kfac_factor_conv_a(j.x, (int)j.rows, j.c, j.H, j.W, j.kh, j.kw, j.sh, j.sw, j.ph,
+                                j.pw, j.dh, j.dw, j.add_bias, j.alpha, j.beta, j.C_prev, j.C, ws,
+                                ws_bytes, stream);
+  }
+}
+
+static size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// The whole plan of a grouped call: which path every product takes, where its partials
+// live, and the device tables of the launches.
+struct GroupedPlan {
+  bool ok = true;
+  std::vector<Classified> cls;
+  std::vector<GroupPlan> plans;         // syrk paths only
+  std::vector<size_t> partial_off;      // floats, from the partial area
+  size_t table_bytes = 0, partial_floats = 0, single_bytes = 0;
+  double executed_flops = 0.;
+  // members of each launch, longest items first
+  std::vector<int> members[3][2];       // [P_DENSE | P_CONVG | P_CONVA][w - 1]
+  std::vector<int> reduce_many[2], reduce_tile[2];   // [w - 1]
+  std::vector<int> singles;             // P_TAPS and P_SINGLE, in call order
+};
+
+template <class T>
+static size_t table_size(size_t n) {
+  return n ? align_up(n * sizeof(T), 16) + align_up((n + 1) * sizeof(int), 16) : 0;
+}
+
+static GroupedPlan make_plan(int count, const kfac_factor_job* jobs) {
+  GroupedPlan gp;
+  gp.cls.resize(count);
+  gp.plans.resize(count);
+  gp.partial_off.assign(count, 0);
+  for (int i = 0; i < count; ++i) {
+    const Classified c = classify(jobs[i]);
+    gp.cls[i] = c;
+    if (c.path == P_BAD) {
+      gp.ok = false;
+      return gp;
+    }
+    if (c.path == P_TAPS || c.path == P_SINGLE) {
+      gp.singles.push_back(i);
+      gp.single_bytes = std::max(gp.single_bytes, single_workspace(jobs[i], c));
+      const kfac_factor_job& j = jobs[i];
+      gp.executed_flops +=
+          j.kind == KFAC_FACTOR_CONV_A
+              ? kfac_factor_conv_a_executed_flops((int)j.rows, j.c, j.H, j.W, j.kh, j.kw, j.sh,
+                                                  j.sw, j.ph, j.pw, j.dh, j.dw, j.add_bias ? 1 : 0)
+              : kfac_factor_executed_flops(c.d, c.K);
+      continue;
+    }
+    const int w = c.d <= 256 ? 1 : 2;
+    gp.members[c.path][w - 1].push_back(i);
+  }
+  for (int path = 0; path < 3; ++path)
+    for (int w = 0; w < 2; ++w) {
+      double units = 0.;
+      for (int i : gp.members[path][w]) {
+        const int T = cdiv(gp.cls[i].d, 64 * (w + 1));
+        units += (double)(T * (T + 1) / 2) * (double)((gp.cls[i].K + 15) / 16);
+      }
+      const long target = launch_target(w + 1, units);
+      for (int i : gp.members[path][w]) {
+        const Classified& c = gp.cls[i];
+        const GroupPlan p = plan_group(c.d, c.K, target);
+        gp.plans[i] = p;
+        gp.partial_off[i] = gp.partial_floats;
+        gp.partial_floats += p.partial_floats();
+        if (p.splits > MANY_SPLITS)
+          gp.reduce_many[w].push_back(i);
+        else if (p.splits > 1)
+          gp.reduce_tile[w].push_back(i);
+        gp.executed_flops += (double)p.ntiles * (double)((c.K + 15) / 16) * 16 * 2.0 * p.ts * p.ts;
+      }
+    }
+  for (int path = 0; path < 3; ++path)
+    for (int w = 0; w < 2; ++w) {
+      auto& m = gp.members[path][w];
+      std::stable_sort(m.begin(), m.end(),
+                       [&](int a, int b) { return gp.plans[a].cps > gp.plans[b].cps; });
+    }
+  for (int w = 0; w < 2; ++w) {
+    gp.table_bytes += table_size<SyJob<DenseKM>>(gp.members[P_DENSE][w].size());
+    gp.table_bytes += table_size<SyJob<ConvG>>(gp.members[P_CONVG][w].size());
+    gp.table_bytes += table_size<SyJob<ConvA>>(gp.members[P_CONVA][w].size());
+    gp.table_bytes += table_size<RdJob>(gp.reduce_many[w].size());
+    gp.table_bytes += table_size<RdJob>(gp.reduce_tile[w].size());
+  }
+  gp.table_bytes = align_up(gp.table_bytes, 256);
+  return gp;
+}
+
+// The plan depends on the shapes only, and a training loop hands over the same few lists
+// step after step: the last plans of every host thread are kept (never freed: objects of
+// this library have no destructors that could run at process exit).
+struct JobShape {
+  int kind, add_bias, c, H, W, kh, kw, sh, sw, ph, pw, dh, dw;
+  int64_t rows;
+  bool operator==(const JobShape& o) const { return memcmp(this, &o, sizeof(JobShape)) == 0; }
+};
+
+static JobShape shape_of(const kfac_factor_job& j) {
+  JobShape s;
+  memset(&s, 0, sizeof(s));
+  s.kind = j.kind;
+  s.add_bias = j.add_bias ? 1 : 0;
+  s.c = j.c;
+  s.H = j.kind == KFAC_FACTOR_LINEAR ? 0 : j.H;
+  s.W = j.kind == KFAC_FACTOR_LINEAR ? 0 : j.W;
+  if (j.kind == KFAC_FACTOR_CONV_A) {
+    s.kh = j.kh; s.kw = j.kw; s.sh = j.sh; s.sw = j.sw;
+    s.ph = j.ph; s.pw = j.pw; s.dh = j.dh; s.dw = j.dw;
+  }
+  s.rows = j.rows;
+  return s;
+}
+
+struct CachedPlan {
+  std::vector<JobShape> shapes;
+  GroupedPlan plan;
+};
+
+static const GroupedPlan& cached_plan(int count, const kfac_factor_job* jobs) {
+  constexpr int SLOTS = 16;
+  static thread_local CachedPlan** slots = nullptr;
+  static thread_local int next_slot = 0;
+  if (!slots) slots = new CachedPlan*[SLOTS]();
+  std::vector<JobShape> shapes((size_t)count);
+  for (int i = 0; i < count; ++i) shapes[i] = shape_of(jobs[i]);
+  for (int k = 0; k < SLOTS; ++k)
+    if (slots[k] && slots[k]->shapes == shapes) return slots[k]->plan;
+  CachedPlan* fresh = new CachedPlan{std::move(shapes), make_plan(count, jobs)};
+  CachedPlan*& slot = slots[next_slot];
+  next_slot = (next_slot + 1) % SLOTS;
+  delete slot;
+  slot = fresh;
+  return slot->plan;
+}
+
+static size_t plan_workspace(const GroupedPlan& gp) {
+  return gp.table_bytes + align_up(gp.partial_floats * sizeof(float), 256) + gp.single_bytes;
+}
+
+// host image of the device tables, filled section by section
+struct TableWriter {
+  std::vector<unsigned> words;
+  template <class T>
+  size_t put(const std::vector<T>& v, size_t align = 16) {       // returns the byte offset
+    const size_t off = words.size() * 4;
+    const size_t bytes = align_up(v.size() * sizeof(T), align);
+    words.resize(words.size() + bytes / 4, 0u);
+    memcpy((char*)words.data() + off, v.data(), v.size() * sizeof(T));
+    return off;
+  }
+};
+
+template <class OP>
+static OP make_op(const kfac_factor_job& j, const Classified& c);
+
+template <>
+DenseKM make_op<DenseKM>(const kfac_factor_job& j, const Classified& c) {
+  return DenseKM{j.x, nullptr, j.c, c.d, j.add_bias ? 1 : 0};
+}
+template <>
+ConvG make_op<ConvG>(const kfac_factor_job& j, const Classified&) {
+  return ConvG(j.x, j.c, j.H * j.W);
+}
+template <>
+ConvA make_op<ConvA>(const kfac_factor_job& j, const Classified& c) {
+  return ConvA(j.x, j.c, j.H, j.W, j.kh, j.kw, j.sh, j.sw, j.ph, j.pw, j.dh, j.dw, c.OH, c.OW, c.d,
+               j.add_bias ? 1 : 0);
+}
+
+struct Launch {
+  size_t jobs_off, cum_off;
+  int njobs, items;
+};
+
+template <class OP>
+static Launch fill_syrk(TableWriter& tw, const GroupedPlan& gp, const std::vector<int>& members,
+                        const kfac_factor_job* jobs, float* partials) {
+  if (members.empty()) return Launch{0, 0, 0, 0};
+  std::vector<SyJob<OP>> tab;
+  std::vector<int> cum;
+  int items = 0;
+  for (int i : members) {
+    const GroupPlan& p = gp.plans[i];
+    const kfac_factor_job& j = jobs[i];
+    SyJob<OP> s;
+    s.op = make_op<OP>(j, gp.cls[i]);
+    s.C = j.C;
+    s.Cin = j.C_prev;
+    s.ws = partials + gp.partial_off[i];
+    s.d = gp.cls[i].d;
+    s.K = (int)gp.cls[i].K;
+    s.T = p.T;
+    s.ntiles = p.ntiles;
+    s.splits = p.splits;
+    s.cps = p.cps;
+    s.alpha = j.alpha;
+    s.beta = j.beta;
+    tab.push_back(s);
+    cum.push_back(items);
+    items += p.ntiles * p.splits;
+  }
+  cum.push_back(items);
+  Launch l;
+  l.jobs_off = tw.put(tab);
+  l.cum_off = tw.put(cum);
+  l.njobs = (int)members.size();
+  l.items = items;
+  return l;
+}
+
+static Launch fill_reduce(TableWriter& tw, const GroupedPlan& gp, const std::vector<int>& members,
+                          const kfac_factor_job* jobs, float* partials, bool many) {
+  if (members.empty()) return Launch{0, 0, 0, 0};
+  std::vector<RdJob> tab;
+  std::vector<int> cum;
+  int items = 0;
+  for (int i : members) {
+    const GroupPlan& p = gp.plans[i];
+    const kfac_factor_job& j = jobs[i];
+    tab.push_back(RdJob{partials + gp.partial_off[i], j.C, j.C_prev, gp.cls[i].d, p.T, p.ntiles,
+                        p.splits, j.alpha, j.beta});
+    cum.push_back(items);
+    items += p.ntiles * (many ? p.ts * (p.ts / 64) : (p.ts / 32) * (p.ts / 64));
+  }
+  cum.push_back(items);
+  Launch l;
+  l.jobs_off = tw.put(tab);
+  l.cum_off = tw.put(cum);
+  l.njobs = (int)members.size();
+  l.items = items;
+  return l;
+}
+
+template <class OP, int W>
+static bool launch_syrk_group(const Launch& l, char* table, hipStream_t stream) {
+  if (l.njobs == 0) return true;
+  constexpr int lds_bytes = Cfg<W, W>::SMEM_FLOATS * (int)sizeof(float);
+  if (!enable_large_lds((const void*)syrk_grouped_kernel<OP, W>, lds_bytes)) return false;
+  hipLaunchKernelGGL((syrk_grouped_kernel<OP, W>), dim3(l.items), dim3(64 * W * W), lds_bytes,
+                     stream, (const SyJob<OP>*)(table + l.jobs_off),
+                     (const int*)(table + l.cum_off), l.njobs);
+  return true;
+}
+
+}  // namespace kfac
+
+using namespace kfac;
+
+extern "C" {
+
+size_t kfac_factor_grouped_workspace_bytes(int count, const kfac_factor_job* jobs) {
+  if (count <= 0 || !jobs) return 0;
+  const GroupedPlan& gp = cached_plan(count, jobs);
+  return gp.ok ? plan_workspace(gp) : 0;
+}
+
+double kfac_factor_grouped_executed_flops(int count, const kfac_factor_job* jobs) {
+  if (count <= 0 || !jobs) return 0.;
+  const GroupedPlan& gp = cached_plan(count, jobs);
+  return gp.ok ? gp.executed_flops : 0.;
+}
+
+int kfac_factor_grouped(int count, const kfac_factor_job* jobs, void* workspace,
+                        size_t workspace_bytes, void* stream_) {
+  if (count < 0 || (count > 0 && !jobs)) return KFAC_ERR_ARG;
+  if (count == 0) return KFAC_OK;
+  const GroupedPlan& gp = cached_plan(count, jobs);
+  if (!gp.ok) return KFAC_ERR_ARG;
+  for (int i = 0; i < count; ++i)
+    if (!jobs[i].x || !jobs[i].C) return KFAC_ERR_ARG;
+  // two products of one call must not write the same factor
+  {
+    std::vector<const float*> outs;
+    for (int i = 0; i < count; ++i) outs.push_back(jobs[i].C);
+    std::sort(outs.begin(), outs.end());
+    if (std::adjacent_find(outs.begin(), outs.end()) != outs.end()) return KFAC_ERR_ARG;
+  }
+  const size_t need = plan_workspace(gp);
+  if (need > 0 && (!workspace || workspace_bytes < need)) return KFAC_ERR_WORKSPACE;
+  hipStream_t stream = (hipStream_t)stream_;
+  char* table = (char*)workspace;
+  float* partials = (float*)(table + gp.table_bytes);
+  char* single_ws = (char*)partials + align_up(gp.partial_floats * sizeof(float), 256);
+
+  TableWriter tw;
+  Launch sy[3][2], rm[2], rt[2];
+  for (int w = 0; w < 2; ++w) {
+    sy[P_DENSE][w] = fill_syrk<DenseKM>(tw, gp, gp.members[P_DENSE][w], jobs, partials);
+    sy[P_CONVG][w] = fill_syrk<ConvG>(tw, gp, gp.members[P_CONVG][w], jobs, partials);
+    sy[P_CONVA][w] = fill_syrk<ConvA>(tw, gp, gp.members[P_CONVA][w], jobs, partials);
+    rm[w] = fill_reduce(tw, gp, gp.reduce_many[w], jobs, partials, true);
+    rt[w] = fill_reduce(tw, gp, gp.reduce_tile[w], jobs, partials, false);
+  }
+  if (tw.words.size() * 4 > gp.table_bytes) return KFAC_ERR_LAUNCH;     // (cannot happen)
+  for (size_t w0 = 0; w0 < tw.words.size(); w0 += BLOB_WORDS) {
+    Blob b;
+    const int n = (int)std::min<size_t>(BLOB_WORDS, tw.words.size() - w0);
+    memcpy(b.w, tw.words.data() + w0, (size_t)n * 4);
+    hipLaunchKernelGGL(upload_kernel, dim3(1), dim3(256), 0, stream, b, (unsigned*)table + w0, n);
+  }
+  // the correlation layers first: each of their launches fills the chip by itself
+  for (int i : gp.singles) {
+    const int st = run_single(jobs[i], gp.single_bytes ? single_ws : nullptr, gp.single_bytes,
+                              stream_);
+    if (st != KFAC_OK) return st;
+  }
+  bool ok = true;
+  ok = ok && launch_syrk_group<ConvA, 2>(sy[P_CONVA][1], table, stream);
+  ok = ok && launch_syrk_group<ConvG, 2>(sy[P_CONVG][1], table, stream);
+  ok = ok && launch_syrk_group<DenseKM, 2>(sy[P_DENSE][1], table, stream);
+  ok = ok && launch_syrk_group<ConvA, 1>(sy[P_CONVA][0], table, stream);
+  ok = ok && launch_syrk_group<ConvG, 1>(sy[P_CONVG][0], table, stream);
+  ok = ok && launch_syrk_group<DenseKM, 1>(sy[P_DENSE][0], table, stream);
+  if (!ok) return KFAC_ERR_LAUNCH;
+  if (rm[1].njobs)
+    hipLaunchKernelGGL(reduce_many_grouped_kernel<128>, dim3(rm[1].items), dim3(256), 0, stream,
+                       (const RdJob*)(table + rm[1].jobs_off), (const int*)(table + rm[1].cum_off),
+                       rm[1].njobs);
+  if (rt[1].njobs)
+    hipLaunchKernelGGL(reduce_tile_grouped_kernel<128>, dim3(rt[1].items), dim3(256), 0, stream,
+                       (const RdJob*)(table + rt[1].jobs_off), (const int*)(table + rt[1].cum_off),
+                       rt[1].njobs);
+  if (rm[0].njobs)
+    hipLaunchKernelGGL(reduce_many_grouped_kernel<64>, dim3(rm[0].items), dim3(256), 0, stream,
+                       (const RdJob*)(table + rm[0].jobs_off), (const int*)(table + rm[0].cum_off),
+                       rm[0].njobs);
+  if (rt[0].njobs)
+    hipLaunchKernelGGL(reduce_tile_grouped_kernel<64>, dim3(rt[0].items), dim3(256), 0, stream,
+                       (const RdJob*)(table + rt[0].jobs_off), (const int*)(table + rt[0].cum_off),
+                       rt[0].njobs);
+  return launch_status();
+}
+
+}  // extern "C"

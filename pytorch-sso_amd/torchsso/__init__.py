@@ -23,5 +23,10 @@ from torchsso import optim  # NOQA
 set_factor_streams = _lanes.set_count
 factor_streams = _lanes.count
 join_factor_streams = _lanes.join
+# 'grouped' (default): hooks collect their factor products, the first reader of factor data
+# runs them in one engine call; 'eager': every product runs in its hook, on the side streams
+set_factor_mode = _lanes.set_mode
+factor_mode = _lanes.mode
+set_factor_flush_work = _lanes.set_flush_work
 
 __version__ = '0.1.0'

@@ -22,6 +22,19 @@ c_f32 = ctypes.c_float
 c_ptr = ctypes.c_void_p
 c_size = ctypes.c_size_t
 
+
+
+class FactorJob(ctypes.Structure):
+    """kfac_factor_job of include/kfac_hip.h: one product of kfac_factor_grouped."""
+    _fields_ = [('kind', c_int), ('add_bias', c_int), ('x', c_ptr), ('rows', c_i64),
+                ('c', c_int), ('H', c_int), ('W', c_int),
+                ('kh', c_int), ('kw', c_int), ('sh', c_int), ('sw', c_int),
+                ('ph', c_int), ('pw', c_int), ('dh', c_int), ('dw', c_int),
+                ('alpha', c_f32), ('beta', c_f32), ('C_prev', c_ptr), ('C', c_ptr)]
+
+
+FACTOR_LINEAR, FACTOR_CONV_A, FACTOR_CONV_G = 0, 1, 2
+
 ERRORS = {1: 'invalid argument', 2: 'workspace too small', 3: 'HIP launch failed',
           4: 'problem too large for the built-in scratch'}
 
@@ -46,6 +59,9 @@ _SIGNATURES = {
                                                            c_ptr, c_size, c_ptr]),
     'kfac_factor_conv_g': (c_int, [c_ptr, c_int, c_int, c_int, c_int, c_f32, c_f32, c_ptr, c_ptr,
                                    c_ptr, c_size, c_ptr]),
+    'kfac_factor_grouped_workspace_bytes': (c_size, [c_int, c_ptr]),
+    'kfac_factor_grouped_executed_flops': (ctypes.c_double, [c_int, c_ptr]),
+    'kfac_factor_grouped': (c_int, [c_int, c_ptr, c_ptr, c_size, c_ptr]),
     'kfac_inverse_workspace_bytes': (c_size, [c_int, c_ptr]),
     'kfac_pi_damped_inverse_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
                                                c_ptr, c_ptr, c_ptr, c_size, c_ptr]),

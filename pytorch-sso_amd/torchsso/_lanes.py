@@ -22,6 +22,13 @@ Ordering rules, all enforced here:
 All default-priority streams.  `set_count(0)` puts every product back on the
 caller's stream.  The results do not depend on the setting: the kernels are
 deterministic and each stream has its own scratch.
+
+Grouped mode (`set_mode('grouped')`, the default) goes one step further: a hook only
+describes its product (`defer`) and keeps the tensor it reads alive; the first reader of
+factor data (`join()`, as before) hands all products collected so far to ONE engine call,
+which runs them as a handful of launches holding the work items of all layers.  The
+side streams are not used then.  `set_mode('eager')` runs every product in its hook, on
+the side streams, as described above.
 """
 import atexit
 import threading
@@ -29,7 +36,24 @@ import threading
 import torch
 
 _count = 3
+_mode = 'grouped'
 _lock = threading.Lock()
+_flush_work = 2.5e11
+
+
+class _Queue(object):
+    """Factor products of one device waiting for their engine call."""
+    __slots__ = ('keys', 'items', 'work')
+
+    def __init__(self):
+        self.keys = set()
+        self.items = []      # (job, tensors kept alive, stream of the hook)
+        self.work = 0.
+
+
+_deferred = {}     # device index -> _Queue
+_calls = {}        # device index -> engine calls made so far (deals them to the side streams)
+_inflight = {}     # device index -> list of (event, items) of calls the side streams may still run
 _streams = {}      # device index -> list of (torch.cuda.Stream, torch.cuda.Event for the fork)
 _pending = {}      # device index -> set of lane indices with work since the last join
 
@@ -46,6 +70,128 @@ def set_count(n):
 
 def count():
     return _count
+
+
+def set_mode(mode):
+    """'grouped': hooks collect their factor products and the first reader of factor data
+    runs them all in one engine call; 'eager': every product runs in its hook."""
+    global _mode
+    if mode not in ('grouped', 'eager'):
+        raise ValueError("factor mode: expected 'grouped' or 'eager', got %r" % (mode,))
+    join()
+    _mode = mode
+
+
+def mode():
+    return _mode
+
+
+def set_flush_work(work):
+    """Grouped mode: the queue of a device also runs as soon as the products collected
+    amount to `work` multiply-adds (d^2 * K summed over them), so that the engine starts on
+    the first layers of a pass while the hooks of the later ones are still being called; a
+    pass then takes a few engine calls instead of one.  None: only readers run the queue."""
+    global _flush_work
+    if work is not None and work <= 0:
+        raise ValueError('flush work must be positive or None')
+    _flush_work = work
+
+
+def flush_work():
+    return _flush_work
+
+
+def defer(device, key, job, keep, work=0.):
+    """Queues one factor product (a `_hip.FactorJob` whose pointers refer to the tensors in
+    `keep`, which stay referenced until the product has been enqueued).  `key` names the
+    factor: a second product for a key that is still queued runs the queue first, so at
+    most one pass of products is ever pending.  `work`: its multiply-adds."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    stream = torch.cuda.current_stream(device)
+    with _lock:
+        q = _deferred.get(idx)
+        if q is None:
+            q = _deferred[idx] = _Queue()
+        dup = key in q.keys
+    if dup:
+        _run_deferred(idx)
+    with _lock:
+        q = _deferred[idx]
+        q.keys.add(key)
+        q.items.append((job, keep, stream))
+        q.work += work
+        full = _flush_work is not None and q.work >= _flush_work
+    if full:
+        _run_deferred(idx)
+
+
+def flush_if_queued(device, key):
+    """Runs the queue of `device` if it holds a product for `key` (the caller is about to
+    reuse that product's job object or output buffer)."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    with _lock:
+        q = _deferred.get(idx)
+        dup = q is not None and key in q.keys
+    if dup:
+        _run_deferred(idx)
+
+
+def deferred_count():
+    """Products queued and not yet handed to the engine (all devices)."""
+    with _lock:
+        return sum(len(q.items) for q in _deferred.values())
+
+
+def _run_deferred(only=None):
+    from torchsso import _ops
+    with _lock:
+        todo = []
+        for i, q in _deferred.items():
+            if q.items and (only is None or only == i):
+                todo.append((i, q.items))
+                _deferred[i] = _Queue()
+    for i, items in todo:
+        device = torch.device('cuda', i)
+        cur = torch.cuda.current_stream(i)
+        side = None
+        if _count > 0:
+            # the engine call goes to a side stream (the calls of a pass take turns), so
+            # that it runs beside whatever the caller's stream does next
+            _, lst = _lane_streams(device)
+            with _lock:
+                lane = _calls.get(i, 0) % _count
+                _calls[i] = _calls.get(i, 0) + 1
+            side, fork = lst[lane]
+            if side == cur:
+                side = None
+        target = cur if side is None else side
+        # a product queued under another stream: its input is complete once that stream
+        # has run what it held at the time of the hook (all of it, to keep this simple)
+        others = []
+        for _, keep, st in items:
+            if st != cur:
+                if st not in others and st != target:
+                    others.append(st)
+                for t in keep:
+                    if t is not None:
+                        t.record_stream(target)
+        if side is not None:
+            with _lock:
+                fork.record(cur)
+                side.wait_event(fork)
+        for st in others:
+            target.wait_stream(st)
+        _ops.factor_grouped([job for job, _, _ in items], device, stream=side)
+        if side is not None:
+            # the tensors stay referenced until the caller's stream has been made to wait
+            # for the side stream (join), or until the side stream is seen to have passed
+            done = torch.cuda.Event()
+            done.record(side)
+            with _lock:
+                held = [h for h in _inflight.get(i, []) if not h[0].query()]
+                held.append((done, items))
+                _inflight[i] = held
+                _pending.setdefault(i, set()).add(lane)
 
 
 def _lane_streams(device):
@@ -91,6 +237,8 @@ def run(device, key, reads, launch):
 def join(device=None):
     """The current stream of `device` (all devices if None) waits for the factor
     products enqueued so far."""
+    if _deferred:
+        _run_deferred(None if device is None or device.index is None else device.index)
     if not _pending:
         return
     with _lock:
@@ -102,6 +250,8 @@ def join(device=None):
         cur = torch.cuda.current_stream(i)
         for lane in lanes:
             cur.wait_stream(_streams[i][lane][0])
+        with _lock:
+            _inflight.pop(i, None)      # (what these calls read may be freed from here on)
 
 
 def _at_exit():
@@ -115,6 +265,8 @@ def _at_exit():
         pass
     _pending.clear()
     _streams.clear()
+    _deferred.clear()
+    _inflight.clear()
 
 
 atexit.register(_at_exit)

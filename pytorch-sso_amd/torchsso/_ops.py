@@ -105,6 +105,91 @@ def factor_conv_g(g, alpha, out=None, beta=0., prev=None, stream=None):
     return out
 
 
+def factor_job(kind, x, alpha, out, beta=0., prev=None, add_bias=False, kernel_size=1,
+               stride=1, padding=0, dilation=1):
+    """A `_hip.FactorJob` describing  out = alpha * P^T P + beta * (prev if given else out)
+    for kfac_factor_grouped: kind 'linear' (x [rows, f]), 'conv_a' (x [n, c, H, W] and the
+    geometry of the convolution) or 'conv_g' (x = grad_output [n, c, h, w]).  The tensors
+    must stay alive until factor_grouped has run."""
+    job = _hip.FactorJob()
+    if kind == 'linear':
+        if x.dim() != 2:
+            raise _hip.KfacHipError('linear factor input must be [rows, f], got %s' % (tuple(x.shape),))
+        rows, c = x.shape
+        d = c + (1 if add_bias else 0)
+        job.kind, job.H, job.W = _hip.FACTOR_LINEAR, 1, 1
+    else:
+        if x.dim() != 4:
+            raise _hip.KfacHipError('conv factor input must be [n, c, H, W], got %s' % (tuple(x.shape),))
+        rows, c, H, W = x.shape
+        job.H, job.W = H, W
+        if kind == 'conv_a':
+            job.kind = _hip.FACTOR_CONV_A
+            job.kh, job.kw = _pair(kernel_size)
+            job.sh, job.sw = _pair(stride)
+            job.ph, job.pw = _pair(padding)
+            job.dh, job.dw = _pair(dilation)
+            d = c * job.kh * job.kw + (1 if add_bias else 0)
+        elif kind == 'conv_g':
+            job.kind = _hip.FACTOR_CONV_G
+            d = c
+        else:
+            raise _hip.KfacHipError('unknown factor kind %r' % (kind,))
+    if tuple(out.shape) != (d, d) or (prev is not None and tuple(prev.shape) != (d, d)):
+        raise _hip.KfacHipError('factor buffers must be (%d, %d)' % (d, d))
+    if beta != 0 and prev is None:
+        prev = out
+    job.add_bias = int(bool(add_bias))
+    job.x = _hip.dev_ptr(x, 'input')
+    job.rows, job.c = rows, c
+    job.alpha, job.beta = float(alpha), float(beta)
+    job.C_prev = _prev_ptr(prev)
+    job.C = _hip.dev_ptr(out, 'factor')
+    return job
+
+
+def factor_job_update(job, x, alpha, out, beta=0., prev=None):
+    """Points an existing job (same kind, shapes and geometry) at new tensors."""
+    if beta != 0 and prev is None:
+        prev = out
+    job.x = _hip.dev_ptr(x, 'input')
+    job.alpha, job.beta = float(alpha), float(beta)
+    job.C_prev = _prev_ptr(prev)
+    job.C = _hip.dev_ptr(out, 'factor')
+
+
+def conv_output_positions(x, kernel_size=1, stride=1, padding=0, dilation=1):
+    """Output positions per image of a convolution over x [n, c, H, W]."""
+    kh, kw = _pair(kernel_size)
+    sh, sw = _pair(stride)
+    ph, pw = _pair(padding)
+    dh, dw = _pair(dilation)
+    oh = (x.shape[2] + 2 * ph - dh * (kh - 1) - 1) // sh + 1
+    ow = (x.shape[3] + 2 * pw - dw * (kw - 1) - 1) // sw + 1
+    return max(oh, 0) * max(ow, 0)
+
+
+def factor_grouped(jobs, device, stream=None):
+    """Runs a list of `factor_job`s in one engine call (a handful of launches for all of them)."""
+    lib = _hip.load()
+    if len(jobs) == 0:
+        return
+    arr = (_hip.FactorJob * len(jobs))(*jobs)
+    ws, ws_bytes = _hip.workspace(device, lib.kfac_factor_grouped_workspace_bytes(len(jobs), arr),
+                                  stream)
+    st = lib.kfac_factor_grouped(len(jobs), arr, _ws_ptr(ws), ws_bytes,
+                                 _hip.stream_ptr(device, stream))
+    _hip.check(st, 'kfac_factor_grouped')
+
+
+def factor_grouped_executed_flops(jobs):
+    lib = _hip.load()
+    if len(jobs) == 0:
+        return 0.
+    arr = (_hip.FactorJob * len(jobs))(*jobs)
+    return lib.kfac_factor_grouped_executed_flops(len(jobs), arr)
+
+
 def _ws_ptr(ws):
     return None if ws is None else ws.data_ptr()
 

@@ -48,17 +48,16 @@ class KronCovConv2d(KronCurvature):
         conv2d = self._module
         n = data_input.shape[0]
         data_input = data_input.contiguous()
-        self._build_factor(0, data_input, lambda scale, out, beta, prev, stream: _ops.factor_conv_a(
-            data_input, conv2d.kernel_size, conv2d.stride, conv2d.padding, conv2d.dilation,
-            self.bias, scale / n, out=out, beta=beta, prev=prev, stream=stream))
+        self._build_factor(0, data_input, 'conv_a', 1. / n, add_bias=self.bias,
+                           kernel_size=conv2d.kernel_size, stride=conv2d.stride,
+                           padding=conv2d.padding, dilation=conv2d.dilation)
 
     def update_in_backward(self, grad_output):
         # G = m m^T / (n h w), then * n^2                (reference: conv.py:69-74,
         #                                                 curvature.py:154-155,299-300)
         n, c, h, w = grad_output.shape
         grad_output = grad_output.contiguous()
-        self._build_factor(1, grad_output, lambda scale, out, beta, prev, stream: _ops.factor_conv_g(
-            grad_output, scale * n / (h * w), out=out, beta=beta, prev=prev, stream=stream))
+        self._build_factor(1, grad_output, 'conv_g', n / (h * w))
 
     def _get_shape(self):
         c_out, c_in, k_h, k_w = self._module.weight.shape

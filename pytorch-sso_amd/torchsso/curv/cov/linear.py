@@ -45,8 +45,7 @@ class KronCovLinear(KronCurvature):
         a = input_data.reshape(-1, input_data.shape[-1]) if input_data.dim() != 2 else input_data
         a = a.contiguous()
         n = input_data.shape[0]
-        self._build_factor(0, a, lambda scale, out, beta, prev, stream: _ops.factor_linear(
-            a, self.bias, scale / n, out=out, beta=beta, prev=prev, stream=stream))
+        self._build_factor(0, a, 'linear', 1. / n, add_bias=self.bias)
 
     def update_in_backward(self, grad_output):
         # G = g^T g / n, then * n^2                   (reference: linear.py:61-67,
@@ -54,8 +53,7 @@ class KronCovLinear(KronCurvature):
         g = grad_output.reshape(-1, grad_output.shape[-1]) if grad_output.dim() != 2 else grad_output
         g = g.contiguous()
         n = grad_output.shape[0]
-        self._build_factor(1, g, lambda scale, out, beta, prev, stream: _ops.factor_linear(
-            g, False, scale * n, out=out, beta=beta, prev=prev, stream=stream))
+        self._build_factor(1, g, 'linear', float(n))
 
     def _get_shape(self):
         f_out, f_in = self._module.weight.shape

@@ -265,6 +265,7 @@ class KronCurvature(Curvature):
         self._lane = KronCurvature._lanes_dealt   # the side stream its factor products use
         KronCurvature._lanes_dealt += 1
         self._next = [None, None]        # receives the next running average
+        self._jobs = [None, None]        # grouped mode: (signature, engine job, d, work) per factor
         self._fresh = [False, False]     # _next[i] holds the next average (hook ran since the last step)
         self._prev_ok = [False, False]   # _next[i] holds the average before the current one
 
@@ -312,31 +313,78 @@ class KronCurvature(Curvature):
 
     # ---- raw factors ------------------------------------------------------------
 
-    def _build_factor(self, idx, source, build):
-        """Runs `build(scale, out, beta, prev, stream)` (a factor kernel computing
-        out = scale * factor + beta * prev on `stream`, reading the contiguous tensor
-        `source`) either for the raw factor or, in fused mode, for the next running
-        average; on this layer's side stream."""
+    def _build_factor(self, idx, source, kind, scale, add_bias=False, **geometry):
+        """Builds factor `idx` (0: A, 1: G) as  scale * P^T P  from the contiguous tensor
+        `source` (`kind`: 'linear', 'conv_a' with the convolution's geometry, 'conv_g'):
+        the raw factor or, in fused mode, the next running average.  In grouped mode the
+        product is only queued here and runs with all others when factor data is first read
+        (torchsso._lanes); in eager mode it runs now, on this layer's side stream."""
         beta = self.ema_decay
         device = source.device
-        lane = 2 * self._lane + idx    # A and G of a layer on different lanes, each always on its own
-        if self.fuse_ema and self.ema is not None and beta != 1:
-            ema = self.ema[idx]
-            nxt = self._next[idx]
-            if nxt is None or nxt.shape != ema.shape:
-                nxt = torch.empty_like(ema)
-            self._next[idx] = _lanes.run(device, lane, (source, ema),
-                                         lambda st: build(beta, nxt, 1. - beta, ema, st))
+        fused = self.fuse_ema and self.ema is not None and beta != 1
+        if fused:
+            prev = self.ema[idx]
+            out = self._next[idx]
+            if out is None or out.shape != prev.shape:
+                out = torch.empty_like(prev)
+            alpha, b = beta * scale, 1. - beta
+        else:
+            prev, out = None, None
+            alpha, b = scale, 0.
+        if _lanes.mode() == 'grouped' and device.type == 'cuda':
+            # (the job object of this factor is reused from pass to pass: the engine copies
+            # it when the queue runs, and a second product of a queued factor runs the queue)
+            _lanes.flush_if_queued(device, (id(self), idx))
+            sig = (kind, tuple(source.shape), add_bias, tuple(sorted(geometry.items())))
+            cached = self._jobs[idx]
+            if cached is None or cached[0] != sig:
+                d = self._factor_dim(idx, source, kind, add_bias, geometry)
+                if out is None:
+                    out = torch.empty((d, d), dtype=torch.float32, device=device)
+                job = _ops.factor_job(kind, source, alpha, out, beta=b, prev=prev,
+                                      add_bias=add_bias, **geometry)     # (checks the shapes)
+                if kind == 'conv_a':
+                    terms = source.shape[0] * _ops.conv_output_positions(source, **geometry)
+                else:
+                    terms = source.numel() // source.shape[1]
+                cached = self._jobs[idx] = (sig, job, d, float(d) * d * terms)
+            _, job, d, work = cached
+            if out is None:
+                out = torch.empty((d, d), dtype=torch.float32, device=device)
+            _ops.factor_job_update(job, source, alpha, out, b, prev)
+            _lanes.defer(device, (id(self), idx), job, (source, prev, out), work)
+        else:
+            lane = 2 * self._lane + idx    # A and G of a layer on different lanes, each always on its own
+            if kind == 'linear':
+                build = lambda st: _ops.factor_linear(source, add_bias, alpha, out=out, beta=b,
+                                                      prev=prev, stream=st)
+            elif kind == 'conv_a':
+                build = lambda st: _ops.factor_conv_a(
+                    source, geometry['kernel_size'], geometry['stride'], geometry['padding'],
+                    geometry['dilation'], add_bias, alpha, out=out, beta=b, prev=prev, stream=st)
+            else:
+                build = lambda st: _ops.factor_conv_g(source, alpha, out=out, beta=b, prev=prev,
+                                                      stream=st)
+            out = _lanes.run(device, lane, (source, prev), build)
+        if fused:
+            self._next[idx] = out
             self._fresh[idx] = True
             self._prev_ok[idx] = False
             raw = None
         else:
-            raw = _lanes.run(device, lane, (source,), lambda st: build(1., None, 0., None, st))
+            raw = out
             self._fresh[idx] = False
         if idx == 0:
             self._A = raw
         else:
             self._G = raw
+
+    @staticmethod
+    def _factor_dim(idx, source, kind, add_bias, geometry):
+        if kind == 'conv_a':
+            kh, kw = _ops._pair(geometry['kernel_size'])
+            return source.shape[1] * kh * kw + (1 if add_bias else 0)
+        return source.shape[1] + (1 if add_bias else 0)
 
     def _raw(self, idx):
         _lanes.join()
