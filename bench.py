@@ -205,8 +205,36 @@ def factor_executed_flops(specs, batch):
     correlation plan the launches use (the library's plan queries): upper-triangular tiles x
     whole reduction chunks x 2 * tile^2 * chunk depth; 13 shared correlations instead of 45
     tap-pair products for a stride-1 3x3 layer."""
+    import torchsso
     from torchsso import _hip
     lib = _hip.load()
+    if torchsso.factor_mode() == 'grouped':
+        # the plan of ONE engine call over all products (the figure does not depend on how the
+        # hooks cut a pass into calls: it counts tiles x reduction chunks, not k-splits)
+        jobs = []
+        for s in specs:
+            if s['kind'] == 'bn':
+                continue
+            for kind in ('a', 'g'):
+                j = _hip.FactorJob()
+                j.x, j.C, j.rows, j.alpha = 256, 256 * (len(jobs) + 2), batch, 1.   # (never dereferenced)
+                if s['kind'] == 'conv' and kind == 'a':
+                    j.kind, j.add_bias = _hip.FACTOR_CONV_A, int(s['bias'])
+                    j.c, j.H, j.W = s['cin'], s['hin'], s['hin']
+                    j.kh = j.kw = s['k']
+                    j.sh = j.sw = s['stride']
+                    j.ph = j.pw = s['pad']
+                    j.dh = j.dw = 1
+                elif s['kind'] == 'conv':
+                    j.kind = _hip.FACTOR_CONV_G
+                    j.c, j.H, j.W = s['cout'], s['hout'], s['hout']
+                else:
+                    j.kind = _hip.FACTOR_LINEAR
+                    j.add_bias = int(s['bias']) if kind == 'a' else 0
+                    j.c = s['fin'] if kind == 'a' else s['fout']
+                jobs.append(j)
+        arr = (_hip.FactorJob * len(jobs))(*jobs)
+        return lib.kfac_factor_grouped_executed_flops(len(jobs), arr)
     total = 0.
     for s in specs:
         if s['kind'] == 'bn':
@@ -294,16 +322,18 @@ class LayerSet(object):
 
     # -- the three phases of a step -----------------------------------------
     def build_factors(self, kinds=('conv', 'linear', 'bn')):
-        for s, m, c, xin, g in zip(self.specs, self.model, self.curvs, self.inputs, self.gouts):
-            if s['kind'] not in kinds:
-                continue
+        """The hooks of one training pass: the forward hooks in layer order, then the backward
+        hooks in reverse order."""
+        layers = [(s, m, c, xin, g) for s, m, c, xin, g in
+                  zip(self.specs, self.model, self.curvs, self.inputs, self.gouts)
+                  if s['kind'] in kinds]
+        for s, m, c, xin, g in layers:
             if s['kind'] == 'bn':
-                # forward hook: sum_hw xhat^2 from the layer output; backward hook: the rest
-                c.forward_postprocess(m, (xin,), xin)
-                c.update_in_backward(g)
+                c.forward_postprocess(m, (xin,), xin)    # sum_hw xhat^2 from the layer output
             else:
                 c.update_in_forward(xin)
-                c.update_in_backward(g)
+        for s, m, c, xin, g in reversed(layers):
+            c.update_in_backward(g)
 
     def restore_grads(self):
         self.flat_grad.copy_(self.flat_raw)
@@ -330,7 +360,9 @@ class LayerSet(object):
             e = [ev() for _ in range(7)]
             e[0].record()
             self.build_factors(('conv', 'linear'))
-            torchsso.join_factor_streams()   # the products run on the library's side streams
+            # (the products run on the library's side streams: eager mode from their hooks, grouped
+            # mode in a few engine calls that the hooks and this join trigger)
+            torchsso.join_factor_streams()
             e[1].record()
             self.build_factors(('bn',))
             e[2].record()
@@ -722,6 +754,9 @@ def main():
                     help='grouped (library default): the hooks queue their factor products and one '
                          'engine call runs them all; eager: a launch sequence per product, on the '
                          'side streams')
+    ap.add_argument('--factor-flush-work', default=None,
+                    help='grouped mode: multiply-adds of queued products from which the queue runs '
+                         'without waiting for a reader (library default: 1e11); "none": never')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--factored-min-dim', type=int, default=None,
                     help='rows from which update_inv keeps an inverse as its triangular factor '
@@ -747,7 +782,10 @@ def main():
         torchsso.set_factor_streams(args.factor_streams)
     if args.factor_mode is not None:
         torchsso.set_factor_mode(args.factor_mode)
-    factor_streams = torchsso.factor_streams() if torchsso.factor_mode() == 'eager' else 0
+    if args.factor_flush_work is not None:
+        torchsso.set_factor_flush_work(None if args.factor_flush_work == 'none'
+                                       else float(args.factor_flush_work))
+    factor_streams = torchsso.factor_streams()
     from torchsso.curv.curvature import KronCurvature
     if args.explicit_inverse:
         KronCurvature.factored_inverse_min_dim = None
@@ -821,7 +859,8 @@ def main():
         'host_enqueue_ms': round(host_ms, 4),
         'not_spd_factors': not_spd,
         'roofline': {'bound': 'mfma',
-                     'kernel': 'Kronecker factor build, all layers (syrk_kernel, corr_kernel)',
+                     'kernel': 'Kronecker factor build, all layers (syrk_grouped_kernel, corr_grouped_kernel; '
+                               'syrk_kernel, corr_kernel in eager mode)',
                      'achieved': round(work['factor'] / f_ms / 1e9, 2),
                      'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
                      'frac': round(work['factor'] / f_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4),

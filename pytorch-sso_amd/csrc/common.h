@@ -34,6 +34,26 @@ int conv_a_taps(const float* x, int n, int c, int H, int W, int kh, int kw, int 
                 int dw, float alpha, float beta, const float* A_prev, float* A, void* workspace,
                 size_t workspace_bytes, hipStream_t stream);
 
+// Copies a small host table to device memory at `dev` (4-byte aligned, `bytes` rounded up to
+// a multiple of 4 are written) as kernel arguments of a few tiny launches on `stream`: no
+// hipMemcpy, so the caller stays capturable and never waits for the device.  The host
+// memory may be reused as soon as this returns.
+void upload_table(const void* host, size_t bytes, void* dev, hipStream_t stream);
+
+// The stride-1 k x k input factors of several layers at once (factor_conv_taps.hip): every
+// geometry must be one that conv_a_taps covers (conv_a_taps_workspace(...) > 0).
+struct TapsJob {
+  const float* x;
+  int n, c, H, W, kh, kw, ph, pw, dh, dw;
+  float alpha, beta;
+  const float* A_prev;
+  float* A;
+};
+size_t conv_a_taps_grouped_workspace(int count, const TapsJob* jobs);
+double conv_a_taps_grouped_executed_flops(int count, const TapsJob* jobs);
+int conv_a_taps_grouped(int count, const TapsJob* jobs, void* workspace, size_t workspace_bytes,
+                        hipStream_t stream);
+
 inline int launch_status() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? KFAC_OK : KFAC_ERR_LAUNCH;

@@ -4,6 +4,8 @@
 #include "operands.h"
 #include "syrk_reduce.h"
 
+#include <string.h>
+
 #include <atomic>
 
 namespace kfac {
@@ -39,6 +41,27 @@ bool enable_large_lds(const void* kernel, int bytes) {
   // table full or device index out of its range: set the attribute on every call
   return hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) ==
          hipSuccess;
+}
+
+constexpr int UPLOAD_WORDS = 960;     // 3840 bytes of the 4 KiB a launch may carry as arguments
+struct UploadChunk {
+  unsigned w[UPLOAD_WORDS];
+};
+__global__ __launch_bounds__(256) void upload_kernel(UploadChunk chunk, unsigned* dst, int words) {
+  for (int i = threadIdx.x; i < words; i += 256) dst[i] = chunk.w[i];
+}
+
+void upload_table(const void* host, size_t bytes, void* dev, hipStream_t stream) {
+  const size_t words = (bytes + 3) / 4;
+  for (size_t w0 = 0; w0 < words; w0 += UPLOAD_WORDS) {
+    UploadChunk c;
+    const size_t n = words - w0 < (size_t)UPLOAD_WORDS ? words - w0 : (size_t)UPLOAD_WORDS;
+    const size_t nb = (w0 + n) * 4 <= bytes ? n * 4 : bytes - w0 * 4;
+    c.w[n - 1] = 0;
+    memcpy(c.w, (const char*)host + w0 * 4, nb);
+    hipLaunchKernelGGL(upload_kernel, dim3(1), dim3(256), 0, stream, c, (unsigned*)dev + w0,
+                       (int)n);
+  }
 }
 
 // Tile configuration and k-split of a symmetric d x d product reduced over K:

@@ -86,15 +86,13 @@ struct TapPlanDev {
   short pair_jobs[MAX_PAIR_JOBS];
 };
 static_assert(sizeof(TapPlanDev) <= 3800, "plan must fit the kernel argument buffer");
+// work item `item` of one layer's plan -> (job, split, tile), and that tile's product
 template <int W>
-__global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void corr_kernel(
-    const float* x, int nimg, int C, int H, int Wd, const TapPlanDev plan, int tiles_side,
-    float* ws) {
+__device__ __forceinline__ void corr_item(const float* x, int nimg, int C, int H, int Wd,
+                                          const TapPlanDev& plan, int tiles_side, float* ws,
+                                          int item, float* smem) {
   constexpr int TS = 64 * W;
   constexpr int KC = Cfg<W, W>::KC;
-  extern __shared__ __attribute__((aligned(16))) float smem[];
-  // work item -> (job, split, tile)
-  const int item = blockIdx.x;
   int j = -1;
 #pragma unroll
   for (int q = 0; q < MAX_JOBS; ++q) j += plan.item0[q] <= item ? 1 : 0;
@@ -119,17 +117,56 @@ __global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void corr_kernel(
   gemm_tile_cfg<W, W>(P, Q, bi * TS, bj * TS, kbeg, kend, false, epi, smem);
 }
 
+template <int W>
+__global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void corr_kernel(
+    const float* x, int nimg, int C, int H, int Wd, const TapPlanDev plan, int tiles_side,
+    float* ws) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  corr_item<W>(x, nimg, C, H, Wd, plan, tiles_side, ws, blockIdx.x, smem);
+}
+
+// One layer of a grouped call: its tensors, and where its plan's partials and block sums live.
+struct TapLayer {
+  const float* x;
+  float* ws;
+  float* B;
+  const float* Ain;
+  float* A;
+  int n, C, H, W, T, tiles_side;
+  float alpha, beta;
+};
+
+__device__ __forceinline__ int find_layer(const int* __restrict__ cum, int n, int item) {
+  int lo = 0, hi = n;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cum[mid] <= item) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// the correlation items of all layers of one tile size in one launch
+template <int W>
+__global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void corr_grouped_kernel(
+    const TapLayer* __restrict__ layers, const TapPlanDev* __restrict__ plans,
+    const int* __restrict__ index, const int* __restrict__ cum, int nlayers) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  const int k = find_layer(cum, nlayers, blockIdx.x);
+  const int l = index[k];
+  const TapLayer& L = layers[l];
+  corr_item<W>(L.x, L.n, L.C, L.H, L.W, plans[l], L.tiles_side, L.ws, blockIdx.x - cum[k], smem);
+}
+
 // B[pair][c][c'] = sum over the pair's jobs and their k-splits, in a fixed order.
 // One workgroup owns 64 float4 groups of the block; its 4 waves take the partials
 // (all splits of all jobs, as one list) round-robin, two loads in flight each, and
 // the 4 wave sums are added in wave order.
-__global__ __launch_bounds__(256) void block_sum_kernel(const TapPlanDev plan, const float* ws,
-                                                        int CC, float* B) {
+__device__ __forceinline__ void block_sum_item(const TapPlanDev& plan, const float* ws, int CC,
+                                               float* B, int eblock, int pair) {
   __shared__ float4 red[4][64];
-  const int pair = blockIdx.y;
   const int jb = plan.pair_first[pair], je = plan.pair_first[pair + 1];
   const int lane = threadIdx.x & 63, sl = threadIdx.x >> 6;
-  const int e = (blockIdx.x * 64 + lane) * 4;   // CC is a multiple of 4 (channel counts are even, >= 16)
+  const int e = (eblock * 64 + lane) * 4;   // CC is a multiple of 4 (channel counts are even, >= 16)
   const bool live = e < CC;
   float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
   int turn = 0;                                 // position in the pair's list of partials, mod 4
@@ -164,17 +201,34 @@ __global__ __launch_bounds__(256) void block_sum_kernel(const TapPlanDev plan, c
   }
 }
 
+__global__ __launch_bounds__(256) void block_sum_kernel(const TapPlanDev plan, const float* ws,
+                                                        int CC, float* B) {
+  block_sum_item(plan, ws, CC, B, blockIdx.x, blockIdx.y);
+}
+
+// ... of all layers: item = (layer, pair, block of 256 elements)
+__global__ __launch_bounds__(256) void block_sum_grouped_kernel(
+    const TapLayer* __restrict__ layers, const TapPlanDev* __restrict__ plans,
+    const int* __restrict__ cum, int nlayers) {
+  const int l = find_layer(cum, nlayers, blockIdx.x);
+  const TapLayer& L = layers[l];
+  const int CC = L.C * L.C;
+  const int eblocks = (CC / 4 + 63) / 64;
+  const int local = blockIdx.x - cum[l];
+  const int pair = local / eblocks;
+  block_sum_item(plans[l], L.ws, CC, L.B, local - pair * eblocks, pair);
+}
+
 // One workgroup writes, for one tap t, the rows (c, t) of 16 channels c against the
 // columns (c', t') of 32 channels c' and all taps t': 16 runs of 32*T consecutive
 // elements of A.  The T blocks B[(t,t')] that feed them are read along their rows
 // (blocks below the diagonal: the transposed block, along its rows as well) and
 // go through LDS into the interleaved order.
-__global__ __launch_bounds__(256) void interleave_kernel(const TapPlanDev plan, const float* B,
-                                                         int C, int T, float alpha, float beta,
-                                                         const float* Ain, float* A) {
+__device__ __forceinline__ void interleave_item(const TapPlanDev& plan, const float* B, int C,
+                                                int T, float alpha, float beta, const float* Ain,
+                                                float* A, int qblock, int cblock, int t) {
   __shared__ float out[IL_ROWS][IL_COLS * MAX_TAPS + 1];
-  const int t = blockIdx.z;
-  const int c0 = blockIdx.y * IL_ROWS, q0 = blockIdx.x * IL_COLS;
+  const int c0 = cblock * IL_ROWS, q0 = qblock * IL_COLS;
   const int d = C * T;
   const size_t CC = (size_t)C * C;
   const int tid = threadIdx.x;
@@ -224,6 +278,27 @@ __global__ __launch_bounds__(256) void interleave_kernel(const TapPlanDev plan, 
     for (int k = 0; k < BATCH; ++k)
       if (e0 + 256 * k < total) A[idx[k]] = alpha * val[k] + beta * old[k];
   }
+}
+
+__global__ __launch_bounds__(256) void interleave_kernel(const TapPlanDev plan, const float* B,
+                                                         int C, int T, float alpha, float beta,
+                                                         const float* Ain, float* A) {
+  interleave_item(plan, B, C, T, alpha, beta, Ain, A, blockIdx.x, blockIdx.y, blockIdx.z);
+}
+
+// ... of all layers: item = (layer, tap, block of 16 channels, block of 32 channels)
+__global__ __launch_bounds__(256) void interleave_grouped_kernel(
+    const TapLayer* __restrict__ layers, const TapPlanDev* __restrict__ plans,
+    const int* __restrict__ cum, int nlayers) {
+  const int l = find_layer(cum, nlayers, blockIdx.x);
+  const TapLayer& L = layers[l];
+  const int qb = (L.C + IL_COLS - 1) / IL_COLS, cb = (L.C + IL_ROWS - 1) / IL_ROWS;
+  int local = blockIdx.x - cum[l];
+  const int t = local / (qb * cb);
+  local -= t * qb * cb;
+  const int cblock = local / qb;
+  interleave_item(plans[l], L.B, L.C, L.T, L.alpha, L.beta, L.Ain, L.A, local - cblock * qb,
+                  cblock, t);
 }
 
 // ---------------------------------------------------------------------------
@@ -283,8 +358,11 @@ struct TapPlanHost {
   bool ok;
 };
 
+// `group_cps` > 0: the plan is for a launch shared with other layers, which fills the chip
+// whatever this layer contributes: every job is then cut into items of about that many
+// chunks (fewer, longer items: fewer partial blocks to write and to add up).
 static TapPlanHost plan_taps(int n, int c, int H, int Wd, int kh, int kw, int ph, int pw, int dh,
-                             int dw) {
+                             int dw, int group_cps = 0) {
   TapPlanHost hp;
   hp.ok = false;
   const int T = kh * kw;
@@ -347,7 +425,9 @@ static TapPlanHost plan_taps(int n, int c, int H, int Wd, int kh, int kw, int ph
   for (int j = 0; j < pd.njobs; ++j) {
     JobDesc& jd = pd.jobs[j];
     const long nchunks = (job_k(jd) + kc - 1) / kc;
-    long splits = (long)(target_items * ((double)job_k(jd) / total) / ntiles + 0.5);
+    long splits = group_cps > 0
+                      ? (nchunks + group_cps / 2) / group_cps
+                      : (long)(target_items * ((double)job_k(jd) / total) / ntiles + 0.5);
     const long max_splits = std::max<long>(1, nchunks / (128 / kc));
     splits = std::max<long>(1, std::min(std::min(splits, max_splits), 4096L));
     long cps = (nchunks + splits - 1) / splits;
@@ -380,10 +460,7 @@ size_t conv_a_taps_workspace(int n, int c, int H, int W, int kh, int kw, int ph,
 
 // MFMA flops corr_kernel executes for this geometry: whole chunks on full tiles, for every
 // (job, split, tile) work item.
-double conv_a_taps_executed_flops(int n, int c, int H, int W, int kh, int kw, int ph, int pw,
-                                  int dh, int dw) {
-  const TapPlanHost hp = plan_taps(n, c, H, W, kh, kw, ph, pw, dh, dw);
-  if (!hp.ok) return 0.;
+static double plan_executed_flops(const TapPlanHost& hp, int n) {
   const int ts = 64 * hp.w;
   const int kc = hp.w == 1 ? Cfg<1, 1>::KC : Cfg<2, 2>::KC;
   const double ntiles = (double)hp.tiles_side * hp.tiles_side;
@@ -394,6 +471,12 @@ double conv_a_taps_executed_flops(int n, int c, int H, int W, int kh, int kw, in
     total += ntiles * (double)((K + kc - 1) / kc) * kc * 2.0 * ts * ts;
   }
   return total;
+}
+
+double conv_a_taps_executed_flops(int n, int c, int H, int W, int kh, int kw, int ph, int pw,
+                                  int dh, int dw) {
+  const TapPlanHost hp = plan_taps(n, c, H, W, kh, kw, ph, pw, dh, dw);
+  return hp.ok ? plan_executed_flops(hp, n) : 0.;
 }
 
 // returns KFAC_OK, an error, or -1 when the geometry is not covered (the caller
@@ -423,6 +506,185 @@ int conv_a_taps(const float* x, int n, int c, int H, int W, int kh, int kw, int 
   hipLaunchKernelGGL(interleave_kernel, dim3(cdiv(c, IL_COLS), cdiv(c, IL_ROWS), T), dim3(256), 0,
                      stream, hp.dev, B, c,
                      T, alpha, beta, A_prev, A);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// several layers at once
+// ---------------------------------------------------------------------------
+struct TapsShape {
+  int n, c, H, W, kh, kw, ph, pw, dh, dw;
+  bool operator==(const TapsShape& o) const { return memcmp(this, &o, sizeof(TapsShape)) == 0; }
+};
+
+// Everything of a grouped call that depends on the shapes only.
+struct TapsGroupPlan {
+  std::vector<TapsShape> shapes;
+  std::vector<TapPlanHost> plans;
+  std::vector<size_t> ws_off;          // floats, per layer, from the partial area
+  std::vector<int> members[2];         // layers by tile size (w - 1), longest items first
+  std::vector<int> cum_corr[2], cum_sum, cum_il;
+  size_t layers_off, plans_off, index_off[2], cum_corr_off[2], cum_sum_off, cum_il_off;
+  size_t table_bytes, partial_floats;
+  double executed_flops;
+  bool ok;
+};
+
+static size_t pad16(size_t v) { return (v + 15) / 16 * 16; }
+
+// chunks per item of a grouped launch (one-wave 64-wide tiles / four-wave 128-wide tiles);
+// measured flat between 48 and 192
+constexpr int TAPS_GROUP_CPS1 = 192, TAPS_GROUP_CPS2 = 96;
+
+static TapsGroupPlan* make_taps_group_plan(int count, const TapsJob* jobs) {
+  TapsGroupPlan* gp = new TapsGroupPlan();
+  gp->ok = true;
+  gp->partial_floats = 0;
+  gp->executed_flops = 0.;
+  for (int i = 0; i < count; ++i) {
+    const TapsJob& j = jobs[i];
+    gp->shapes.push_back(TapsShape{j.n, j.c, j.H, j.W, j.kh, j.kw, j.ph, j.pw, j.dh, j.dw});
+    gp->plans.push_back(plan_taps(j.n, j.c, j.H, j.W, j.kh, j.kw, j.ph, j.pw, j.dh, j.dw,
+                                  j.c <= 64 ? TAPS_GROUP_CPS1 : TAPS_GROUP_CPS2));
+    const TapPlanHost& hp = gp->plans.back();
+    if (!hp.ok) {
+      gp->ok = false;
+      return gp;
+    }
+    gp->ws_off.push_back(gp->partial_floats);
+    gp->partial_floats += (hp.partial_floats + 63) / 64 * 64;
+    gp->members[hp.w - 1].push_back(i);
+    gp->executed_flops += plan_executed_flops(hp, j.n);
+  }
+  for (int w = 0; w < 2; ++w) {
+    auto& m = gp->members[w];
+    auto longest = [&](int i) {
+      int c = 0;
+      for (int q = 0; q < gp->plans[i].dev.njobs; ++q) c = std::max(c, gp->plans[i].dev.jobs[q].cps);
+      return c;
+    };
+    std::stable_sort(m.begin(), m.end(), [&](int a, int b) { return longest(a) > longest(b); });
+    int items = 0;
+    for (int i : m) {
+      gp->cum_corr[w].push_back(items);
+      items += gp->plans[i].items;
+    }
+    gp->cum_corr[w].push_back(items);
+  }
+  int s_items = 0, il_items = 0;
+  for (int i = 0; i < count; ++i) {
+    const TapsJob& j = jobs[i];
+    const int T = j.kh * j.kw;
+    gp->cum_sum.push_back(s_items);
+    gp->cum_il.push_back(il_items);
+    s_items += cdiv(j.c * j.c / 4, 64) * gp->plans[i].dev.npairs;
+    il_items += cdiv(j.c, IL_COLS) * cdiv(j.c, IL_ROWS) * T;
+  }
+  gp->cum_sum.push_back(s_items);
+  gp->cum_il.push_back(il_items);
+  size_t off = 0;
+  gp->layers_off = off;
+  off += pad16((size_t)count * sizeof(TapLayer));
+  gp->plans_off = off;
+  off += pad16((size_t)count * sizeof(TapPlanDev));
+  for (int w = 0; w < 2; ++w) {
+    gp->index_off[w] = off;
+    off += pad16(gp->members[w].size() * sizeof(int));
+    gp->cum_corr_off[w] = off;
+    off += pad16(gp->cum_corr[w].size() * sizeof(int));
+  }
+  gp->cum_sum_off = off;
+  off += pad16(gp->cum_sum.size() * sizeof(int));
+  gp->cum_il_off = off;
+  off += pad16(gp->cum_il.size() * sizeof(int));
+  gp->table_bytes = (off + 255) / 256 * 256;
+  return gp;
+}
+
+// the last plans of every host thread are kept (and never freed: nothing of this library
+// has a destructor that could run at process exit)
+static const TapsGroupPlan& taps_group_plan(int count, const TapsJob* jobs) {
+  constexpr int SLOTS = 16;
+  static thread_local TapsGroupPlan** slots = nullptr;
+  static thread_local int next_slot = 0;
+  if (!slots) slots = new TapsGroupPlan*[SLOTS]();
+  for (int k = 0; k < SLOTS; ++k) {
+    const TapsGroupPlan* p = slots[k];
+    if (!p || (int)p->shapes.size() != count) continue;
+    bool same = true;
+    for (int i = 0; i < count && same; ++i) {
+      const TapsJob& j = jobs[i];
+      same = p->shapes[i] == TapsShape{j.n, j.c, j.H, j.W, j.kh, j.kw, j.ph, j.pw, j.dh, j.dw};
+    }
+    if (same) return *p;
+  }
+  TapsGroupPlan*& slot = slots[next_slot];
+  next_slot = (next_slot + 1) % SLOTS;
+  delete slot;
+  slot = make_taps_group_plan(count, jobs);
+  return *slot;
+}
+
+size_t conv_a_taps_grouped_workspace(int count, const TapsJob* jobs) {
+  if (count <= 0) return 0;
+  const TapsGroupPlan& gp = taps_group_plan(count, jobs);
+  return gp.ok ? gp.table_bytes + gp.partial_floats * sizeof(float) : 0;
+}
+
+double conv_a_taps_grouped_executed_flops(int count, const TapsJob* jobs) {
+  if (count <= 0) return 0.;
+  const TapsGroupPlan& gp = taps_group_plan(count, jobs);
+  return gp.ok ? gp.executed_flops : 0.;
+}
+
+int conv_a_taps_grouped(int count, const TapsJob* jobs, void* workspace, size_t workspace_bytes,
+                        hipStream_t stream) {
+  if (count <= 0) return KFAC_OK;
+  const TapsGroupPlan& gp = taps_group_plan(count, jobs);
+  if (!gp.ok) return KFAC_ERR_ARG;
+  if (!workspace || workspace_bytes < gp.table_bytes + gp.partial_floats * sizeof(float))
+    return KFAC_ERR_WORKSPACE;
+  char* table = (char*)workspace;
+  float* partials = (float*)(table + gp.table_bytes);
+  std::vector<char> img(gp.table_bytes, 0);
+  TapLayer* layers = (TapLayer*)(img.data() + gp.layers_off);
+  TapPlanDev* plans = (TapPlanDev*)(img.data() + gp.plans_off);
+  for (int i = 0; i < count; ++i) {
+    const TapsJob& j = jobs[i];
+    const TapPlanHost& hp = gp.plans[i];
+    float* ws = partials + gp.ws_off[i];
+    layers[i] = TapLayer{j.x, ws, ws + hp.sum_offset, j.A_prev, j.A, j.n, j.c, j.H, j.W,
+                         j.kh * j.kw, hp.tiles_side, j.alpha, j.beta};
+    plans[i] = hp.dev;
+  }
+  for (int w = 0; w < 2; ++w) {
+    if (!gp.members[w].empty())
+      memcpy(img.data() + gp.index_off[w], gp.members[w].data(), gp.members[w].size() * sizeof(int));
+    memcpy(img.data() + gp.cum_corr_off[w], gp.cum_corr[w].data(), gp.cum_corr[w].size() * sizeof(int));
+  }
+  memcpy(img.data() + gp.cum_sum_off, gp.cum_sum.data(), gp.cum_sum.size() * sizeof(int));
+  memcpy(img.data() + gp.cum_il_off, gp.cum_il.data(), gp.cum_il.size() * sizeof(int));
+  upload_table(img.data(), img.size(), table, stream);
+  const TapLayer* dl = (const TapLayer*)(table + gp.layers_off);
+  const TapPlanDev* dp = (const TapPlanDev*)(table + gp.plans_off);
+  if (!gp.members[1].empty()) {
+    constexpr int lds = Cfg<2, 2>::SMEM_FLOATS * (int)sizeof(float);
+    if (!enable_large_lds((const void*)corr_grouped_kernel<2>, lds)) return KFAC_ERR_LAUNCH;
+    hipLaunchKernelGGL(corr_grouped_kernel<2>, dim3(gp.cum_corr[1].back()), dim3(256), lds, stream,
+                       dl, dp, (const int*)(table + gp.index_off[1]),
+                       (const int*)(table + gp.cum_corr_off[1]), (int)gp.members[1].size());
+  }
+  if (!gp.members[0].empty()) {
+    constexpr int lds = Cfg<1, 1>::SMEM_FLOATS * (int)sizeof(float);
+    if (!enable_large_lds((const void*)corr_grouped_kernel<1>, lds)) return KFAC_ERR_LAUNCH;
+    hipLaunchKernelGGL(corr_grouped_kernel<1>, dim3(gp.cum_corr[0].back()), dim3(64), lds, stream,
+                       dl, dp, (const int*)(table + gp.index_off[0]),
+                       (const int*)(table + gp.cum_corr_off[0]), (int)gp.members[0].size());
+  }
+  hipLaunchKernelGGL(block_sum_grouped_kernel, dim3(gp.cum_sum.back()), dim3(256), 0, stream, dl, dp,
+                     (const int*)(table + gp.cum_sum_off), count);
+  hipLaunchKernelGGL(interleave_grouped_kernel, dim3(gp.cum_il.back()), dim3(256), 0, stream, dl, dp,
+                     (const int*)(table + gp.cum_il_off), count);
   return launch_status();
 }
 

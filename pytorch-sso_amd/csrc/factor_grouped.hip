@@ -18,7 +18,6 @@
 // Products whose input exceeds the 1 GiB addressing window of an operand, and the
 // stride-1 k x k layers served by the correlation kernels, are handed to their
 // single-product routines on the same stream.
-#include <stdlib.h>
 #include <string.h>
 
 #include <algorithm>
@@ -49,15 +48,6 @@ struct RdJob {
   int d, T, ntiles, splits;
   float alpha, beta;
 };
-
-// tables reach the device as kernel arguments, a chunk per launch
-constexpr int BLOB_WORDS = 960;     // 3840 bytes
-struct Blob {
-  unsigned w[BLOB_WORDS];
-};
-__global__ __launch_bounds__(256) void upload_kernel(Blob blob, unsigned* dst, int words) {
-  for (int i = threadIdx.x; i < words; i += 256) dst[i] = blob.w[i];
-}
 
 // first table entry whose range holds `item` (cum[j] <= item < cum[j + 1])
 __device__ __forceinline__ int find_job(const int* __restrict__ cum, int njobs, int item) {
@@ -161,11 +151,6 @@ struct GroupPlan {
   }
 };
 
-static int env_int(const char* name, int dflt) {
-  const char* s = getenv(name);
-  return s && *s ? atoi(s) : dflt;
-}
-
 static GroupPlan plan_group(int d, long K, long target) {
   GroupPlan p;
   p.w = d <= 256 ? 1 : 2;
@@ -186,9 +171,7 @@ static GroupPlan plan_group(int d, long K, long target) {
 // length, shorter items when it would not fill the chip twice (resident workgroups: 3 per CU
 // of four waves, 8 per CU of one wave).
 static long launch_target(int w, double total_units) {
-  static const int t2 = env_int("KFAC_GROUP_CPS2", GROUP_TARGET_CPS_W2);
-  static const int t1 = env_int("KFAC_GROUP_CPS1", GROUP_TARGET_CPS_W1);
-  const long dflt = w == 1 ? t1 : t2;
+  const long dflt = w == 1 ? GROUP_TARGET_CPS_W1 : GROUP_TARGET_CPS_W2;
   const double slots = w == 1 ? 2048. : 768.;
   long t = (long)(total_units / (2. * slots));
   if (t > dflt) t = dflt;
@@ -288,12 +271,24 @@ struct GroupedPlan {
   // members of each launch, longest items first
   std::vector<int> members[3][2];       // [P_DENSE | P_CONVG | P_CONVA][w - 1]
   std::vector<int> reduce_many[2], reduce_tile[2];   // [w - 1]
-  std::vector<int> singles;             // P_TAPS and P_SINGLE, in call order
+  std::vector<int> singles;             // P_SINGLE, in call order
+  std::vector<int> taps;                // P_TAPS, in call order
+  size_t taps_bytes = 0;
 };
 
 template <class T>
 static size_t table_size(size_t n) {
   return n ? align_up(n * sizeof(T), 16) + align_up((n + 1) * sizeof(int), 16) : 0;
+}
+
+static std::vector<TapsJob> taps_jobs(const GroupedPlan& gp, const kfac_factor_job* jobs) {
+  std::vector<TapsJob> tj;
+  for (int i : gp.taps) {
+    const kfac_factor_job& j = jobs[i];
+    tj.push_back(TapsJob{j.x, (int)j.rows, j.c, j.H, j.W, j.kh, j.kw, j.ph, j.pw, j.dh, j.dw,
+                         j.alpha, j.beta, j.C_prev, j.C});
+  }
+  return tj;
 }
 
 static GroupedPlan make_plan(int count, const kfac_factor_job* jobs) {
@@ -308,7 +303,11 @@ static GroupedPlan make_plan(int count, const kfac_factor_job* jobs) {
       gp.ok = false;
       return gp;
     }
-    if (c.path == P_TAPS || c.path == P_SINGLE) {
+    if (c.path == P_TAPS) {
+      gp.taps.push_back(i);
+      continue;
+    }
+    if (c.path == P_SINGLE) {
       gp.singles.push_back(i);
       gp.single_bytes = std::max(gp.single_bytes, single_workspace(jobs[i], c));
       const kfac_factor_job& j = jobs[i];
@@ -357,6 +356,11 @@ static GroupedPlan make_plan(int count, const kfac_factor_job* jobs) {
     gp.table_bytes += table_size<RdJob>(gp.reduce_tile[w].size());
   }
   gp.table_bytes = align_up(gp.table_bytes, 256);
+  if (!gp.taps.empty()) {
+    const std::vector<TapsJob> tj = taps_jobs(gp, jobs);
+    gp.taps_bytes = align_up(conv_a_taps_grouped_workspace((int)tj.size(), tj.data()), 256);
+    gp.executed_flops += conv_a_taps_grouped_executed_flops((int)tj.size(), tj.data());
+  }
   return gp;
 }
 
@@ -408,7 +412,8 @@ static const GroupedPlan& cached_plan(int count, const kfac_factor_job* jobs) {
 }
 
 static size_t plan_workspace(const GroupedPlan& gp) {
-  return gp.table_bytes + align_up(gp.partial_floats * sizeof(float), 256) + gp.single_bytes;
+  return gp.table_bytes + align_up(gp.partial_floats * sizeof(float), 256) + gp.taps_bytes +
+         gp.single_bytes;
 }
 
 // host image of the device tables, filled section by section
@@ -554,7 +559,8 @@ int kfac_factor_grouped(int count, const kfac_factor_job* jobs, void* workspace,
   hipStream_t stream = (hipStream_t)stream_;
   char* table = (char*)workspace;
   float* partials = (float*)(table + gp.table_bytes);
-  char* single_ws = (char*)partials + align_up(gp.partial_floats * sizeof(float), 256);
+  char* taps_ws = (char*)partials + align_up(gp.partial_floats * sizeof(float), 256);
+  char* single_ws = taps_ws + gp.taps_bytes;
 
   TableWriter tw;
   Launch sy[3][2], rm[2], rt[2];
@@ -566,16 +572,15 @@ int kfac_factor_grouped(int count, const kfac_factor_job* jobs, void* workspace,
     rt[w] = fill_reduce(tw, gp, gp.reduce_tile[w], jobs, partials, false);
   }
   if (tw.words.size() * 4 > gp.table_bytes) return KFAC_ERR_LAUNCH;     // (cannot happen)
-  for (size_t w0 = 0; w0 < tw.words.size(); w0 += BLOB_WORDS) {
-    Blob b;
-    const int n = (int)std::min<size_t>(BLOB_WORDS, tw.words.size() - w0);
-    memcpy(b.w, tw.words.data() + w0, (size_t)n * 4);
-    hipLaunchKernelGGL(upload_kernel, dim3(1), dim3(256), 0, stream, b, (unsigned*)table + w0, n);
-  }
-  // the correlation layers first: each of their launches fills the chip by itself
+  upload_table(tw.words.data(), tw.words.size() * 4, table, stream);
   for (int i : gp.singles) {
     const int st = run_single(jobs[i], gp.single_bytes ? single_ws : nullptr, gp.single_bytes,
                               stream_);
+    if (st != KFAC_OK) return st;
+  }
+  if (!gp.taps.empty()) {
+    const std::vector<TapsJob> tj = taps_jobs(gp, jobs);
+    const int st = conv_a_taps_grouped((int)tj.size(), tj.data(), taps_ws, gp.taps_bytes, stream);
     if (st != KFAC_OK) return st;
   }
   bool ok = true;

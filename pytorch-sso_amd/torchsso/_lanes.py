@@ -38,17 +38,18 @@ import torch
 _count = 3
 _mode = 'grouped'
 _lock = threading.Lock()
-_flush_work = 2.5e11
+_flush_work = 1e11
 
 
 class _Queue(object):
     """Factor products of one device waiting for their engine call."""
-    __slots__ = ('keys', 'items', 'work')
+    __slots__ = ('keys', 'items', 'work', 'forward')
 
     def __init__(self):
         self.keys = set()
         self.items = []      # (job, tensors kept alive, stream of the hook)
         self.work = 0.
+        self.forward = False    # holds products queued by forward hooks
 
 
 _deferred = {}     # device index -> _Queue
@@ -101,23 +102,26 @@ def flush_work():
     return _flush_work
 
 
-def defer(device, key, job, keep, work=0.):
+def defer(device, key, job, keep, work=0., backward=False):
     """Queues one factor product (a `_hip.FactorJob` whose pointers refer to the tensors in
     `keep`, which stay referenced until the product has been enqueued).  `key` names the
     factor: a second product for a key that is still queued runs the queue first, so at
-    most one pass of products is ever pending.  `work`: its multiply-adds."""
+    most one pass of products is ever pending.  `work`: its multiply-adds.  `backward`: the
+    product belongs to a backward hook; the first of those runs what the forward hooks have
+    queued, so that the input factors are computed beside the backward pass."""
     idx = device.index if device.index is not None else torch.cuda.current_device()
     stream = torch.cuda.current_stream(device)
     with _lock:
         q = _deferred.get(idx)
         if q is None:
             q = _deferred[idx] = _Queue()
-        dup = key in q.keys
-    if dup:
+        run_first = key in q.keys or (backward and q.forward)
+    if run_first:
         _run_deferred(idx)
     with _lock:
         q = _deferred[idx]
         q.keys.add(key)
+        q.forward = q.forward or not backward
         q.items.append((job, keep, stream))
         q.work += work
         full = _flush_work is not None and q.work >= _flush_work

@@ -352,7 +352,7 @@ class KronCurvature(Curvature):
             if out is None:
                 out = torch.empty((d, d), dtype=torch.float32, device=device)
             _ops.factor_job_update(job, source, alpha, out, b, prev)
-            _lanes.defer(device, (id(self), idx), job, (source, prev, out), work)
+            _lanes.defer(device, (id(self), idx), job, (source, prev, out), work, backward=idx == 1)
         else:
             lane = 2 * self._lane + idx    # A and G of a layer on different lanes, each always on its own
             if kind == 'linear':

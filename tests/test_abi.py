@@ -78,3 +78,38 @@ def test_argument_errors_are_codes_not_crashes():
     assert lib.kfac_damped_inverse_batched_static(1, big, one, None, one, one, None) == 1
     with pytest.raises(_hip.KfacHipError):
         _hip.check(2, 'x')
+
+
+def _job(kind, c, rows, H=1, W=1, k=1, stride=1, pad=0, x=256, C=512):
+    j = _hip.FactorJob()
+    j.kind, j.c, j.rows, j.H, j.W = kind, c, rows, H, W
+    j.kh = j.kw = k
+    j.sh = j.sw = stride
+    j.ph = j.pw = pad
+    j.dh = j.dw = 1
+    j.alpha, j.x, j.C = 1., x, C
+    return j
+
+
+def test_grouped_factor_plan_needs_no_device():
+    """The plan of a grouped call (scratch, executed flops) is host arithmetic; bad lists are
+    refused before anything is launched."""
+    lib = _hip.load()
+    jobs = [_job(_hip.FACTOR_LINEAR, 784, 128, C=1 << 20),
+            _job(_hip.FACTOR_CONV_G, 64, 32, 56, 56, C=2 << 20),          # long reduction: k-splits
+            _job(_hip.FACTOR_CONV_A, 64, 32, 56, 56, k=3, pad=1, C=3 << 20),   # correlation kernels
+            _job(_hip.FACTOR_CONV_A, 128, 32, 28, 28, k=3, stride=2, pad=1, C=4 << 20)]
+    arr = (_hip.FactorJob * len(jobs))(*jobs)
+    assert lib.kfac_factor_grouped_workspace_bytes(len(jobs), arr) > 64 * 64 * 4
+    # executed flops: the same tiles and reduction chunks as the single-product plans
+    single = (lib.kfac_factor_executed_flops(784, 128) + lib.kfac_factor_executed_flops(64, 32 * 56 * 56)
+              + lib.kfac_factor_conv_a_executed_flops(32, 64, 56, 56, 3, 3, 1, 1, 1, 1, 1, 1, 0)
+              + lib.kfac_factor_conv_a_executed_flops(32, 128, 28, 28, 3, 3, 2, 2, 1, 1, 1, 1, 0))
+    assert abs(lib.kfac_factor_grouped_executed_flops(len(jobs), arr) - single) <= 1e-9 * single
+    assert lib.kfac_factor_grouped(0, None, None, 0, None) == 0
+    assert lib.kfac_factor_grouped(1, None, None, 0, None) == 1
+    assert lib.kfac_factor_grouped(len(jobs), arr, None, 0, None) == 2            # no scratch
+    bad = (_hip.FactorJob * 1)(_job(7, 4, 4))
+    assert lib.kfac_factor_grouped(1, bad, None, 0, None) == 1                    # unknown kind
+    twice = (_hip.FactorJob * 2)(_job(_hip.FACTOR_LINEAR, 4, 4), _job(_hip.FACTOR_LINEAR, 4, 4))
+    assert lib.kfac_factor_grouped(2, twice, None, 0, None) == 1                  # one output twice

@@ -613,6 +613,37 @@ def test_factor_side_streams_host_logic():
     assert torchsso.factor_streams() == 3     # the default
 
 
+def test_factor_mode_host_logic():
+    """Grouped / eager mode and the flush threshold are validated on the host; a tensor that
+    is not on a HIP device is never queued (its product runs, and raises, where it is)."""
+    from torchsso import _lanes
+    assert torchsso.factor_mode() == 'grouped'       # the default
+    before_work = _lanes.flush_work()
+    try:
+        with pytest.raises(ValueError):
+            torchsso.set_factor_mode('deferred')
+        torchsso.set_factor_mode('eager')
+        assert torchsso.factor_mode() == 'eager'
+        torchsso.set_factor_mode('grouped')
+        for bad in (0, -1.):
+            with pytest.raises(ValueError):
+                torchsso.set_factor_flush_work(bad)
+        torchsso.set_factor_flush_work(None)
+        assert _lanes.flush_work() is None
+        torchsso.set_factor_flush_work(5e9)
+        assert _lanes.flush_work() == 5e9
+        assert _lanes.deferred_count() == 0
+        lin = torch.nn.Linear(3, 2)
+        curv = torchsso.KronCovLinear(lin)
+        with pytest.raises(torchsso._hip.KfacHipError):
+            lin(torch.randn(4, 3))                   # CPU input: no queue, no CPU path
+        assert _lanes.deferred_count() == 0
+        del curv
+    finally:
+        torchsso.set_factor_mode('grouped')
+        torchsso.set_factor_flush_work(before_work)
+
+
 def test_fisher_closure_exact_and_mc(oracle_ops):
     """Exact Fisher: the G factor of the logits layer equals mean_n(diag(p) - p p^T);
     every layer (also the first) gets a G factor; gradients are those of the true
