@@ -206,17 +206,46 @@ __global__ __launch_bounds__(256) void block_sum_kernel(const TapPlanDev plan, c
   block_sum_item(plan, ws, CC, B, blockIdx.x, blockIdx.y);
 }
 
-// ... of all layers: item = (layer, pair, block of 256 elements)
+// ... of all layers: item = (layer, pair, block of 1024 elements).  A grouped plan cuts the
+// jobs into few, long splits, so a pair's list of partials is short: every thread owns one
+// float4 of the block and walks the whole list itself (fixed order, four loads in flight)
+// instead of four waves sharing the list of a quarter as many elements.
+constexpr int SUM_BLOCK = 1024;
 __global__ __launch_bounds__(256) void block_sum_grouped_kernel(
     const TapLayer* __restrict__ layers, const TapPlanDev* __restrict__ plans,
     const int* __restrict__ cum, int nlayers) {
   const int l = find_layer(cum, nlayers, blockIdx.x);
   const TapLayer& L = layers[l];
+  const TapPlanDev& plan = plans[l];
   const int CC = L.C * L.C;
-  const int eblocks = (CC / 4 + 63) / 64;
+  const int eblocks = (CC + SUM_BLOCK - 1) / SUM_BLOCK;
   const int local = blockIdx.x - cum[l];
   const int pair = local / eblocks;
-  block_sum_item(plans[l], L.ws, CC, L.B, local - pair * eblocks, pair);
+  const int e = ((local - pair * eblocks) * 256 + threadIdx.x) * 4;
+  if (e >= CC) return;
+  const int jb = plan.pair_first[pair], je = plan.pair_first[pair + 1];
+  float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int q = jb; q < je; ++q) {
+    const JobDesc& jd = plan.jobs[plan.pair_jobs[q]];
+    const float* part = L.ws + (size_t)jd.part0 * CC + e;
+    const int splits = jd.splits;
+    int sp = 0;
+    for (; sp + 4 <= splits; sp += 4) {
+      const float4 v0 = *reinterpret_cast<const float4*>(part + (size_t)sp * CC);
+      const float4 v1 = *reinterpret_cast<const float4*>(part + (size_t)(sp + 1) * CC);
+      const float4 v2 = *reinterpret_cast<const float4*>(part + (size_t)(sp + 2) * CC);
+      const float4 v3 = *reinterpret_cast<const float4*>(part + (size_t)(sp + 3) * CC);
+      s.x += v0.x; s.y += v0.y; s.z += v0.z; s.w += v0.w;
+      s.x += v1.x; s.y += v1.y; s.z += v1.z; s.w += v1.w;
+      s.x += v2.x; s.y += v2.y; s.z += v2.z; s.w += v2.w;
+      s.x += v3.x; s.y += v3.y; s.z += v3.z; s.w += v3.w;
+    }
+    for (; sp < splits; ++sp) {
+      const float4 v = *reinterpret_cast<const float4*>(part + (size_t)sp * CC);
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+  }
+  *reinterpret_cast<float4*>(L.B + (size_t)pair * CC + e) = s;
 }
 
 // One workgroup writes, for one tap t, the rows (c, t) of 16 channels c against the
@@ -541,11 +570,29 @@ static TapsGroupPlan* make_taps_group_plan(int count, const TapsJob* jobs) {
   gp->ok = true;
   gp->partial_floats = 0;
   gp->executed_flops = 0.;
+  // chunks per item: the default where a tile size has plenty of work, shorter items where
+  // its launch would not fill the chip twice (3 layers of 64 channels, say)
+  double units[2] = {0., 0.};
+  for (int i = 0; i < count; ++i) {
+    const TapsJob& j = jobs[i];
+    const int w = j.c <= 64 ? 1 : 2;
+    const double tiles = (double)cdiv(j.c, 64 * w) * cdiv(j.c, 64 * w);
+    // 13 of the 45 tap pairs of a 3x3 kernel are computed; in general about T(T+1)/2 / 3.4
+    const int T = j.kh * j.kw;
+    units[w - 1] += tiles * (T * (T + 1) / 2 / 3.4) * ((double)j.n * j.H * j.W / 16.);
+  }
+  int group_cps[2];
+  for (int w = 0; w < 2; ++w) {
+    const double slots = w == 0 ? 2048. : 768.;
+    const int dflt = w == 0 ? TAPS_GROUP_CPS1 : TAPS_GROUP_CPS2;
+    long t = (long)(units[w] / (2. * slots));
+    group_cps[w] = (int)std::max(8L, std::min((long)dflt, t));
+  }
   for (int i = 0; i < count; ++i) {
     const TapsJob& j = jobs[i];
     gp->shapes.push_back(TapsShape{j.n, j.c, j.H, j.W, j.kh, j.kw, j.ph, j.pw, j.dh, j.dw});
     gp->plans.push_back(plan_taps(j.n, j.c, j.H, j.W, j.kh, j.kw, j.ph, j.pw, j.dh, j.dw,
-                                  j.c <= 64 ? TAPS_GROUP_CPS1 : TAPS_GROUP_CPS2));
+                                  group_cps[j.c <= 64 ? 0 : 1]));
     const TapPlanHost& hp = gp->plans.back();
     if (!hp.ok) {
       gp->ok = false;
@@ -577,7 +624,7 @@ static TapsGroupPlan* make_taps_group_plan(int count, const TapsJob* jobs) {
     const int T = j.kh * j.kw;
     gp->cum_sum.push_back(s_items);
     gp->cum_il.push_back(il_items);
-    s_items += cdiv(j.c * j.c / 4, 64) * gp->plans[i].dev.npairs;
+    s_items += cdiv(j.c * j.c, SUM_BLOCK) * gp->plans[i].dev.npairs;
     il_items += cdiv(j.c, IL_COLS) * cdiv(j.c, IL_ROWS) * T;
   }
   gp->cum_sum.push_back(s_items);
