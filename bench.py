@@ -749,14 +749,14 @@ def main():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--workload', default='resnet50', choices=sorted(WORKLOADS) + ['noisy_kfac', 'resnet50_train'])
     ap.add_argument('--factor-streams', type=int, default=None,
-                    help='side streams for the factor products (library default: 3; 0 = none)')
+                    help='side streams for the factor products (library default: 2; 0 = none)')
     ap.add_argument('--factor-mode', default=None, choices=['grouped', 'eager'],
                     help='grouped (library default): the hooks queue their factor products and one '
                          'engine call runs them all; eager: a launch sequence per product, on the '
                          'side streams')
     ap.add_argument('--factor-flush-work', default=None,
                     help='grouped mode: multiply-adds of queued products from which the queue runs '
-                         'without waiting for a reader (library default: 1e11); "none": never')
+                         'without waiting for a reader (library default: 2.5e11); "none": never')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--factored-min-dim', type=int, default=None,
                     help='rows from which update_inv keeps an inverse as its triangular factor '

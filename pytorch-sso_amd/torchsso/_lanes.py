@@ -35,10 +35,10 @@ import threading
 
 import torch
 
-_count = 3
+_count = 2
 _mode = 'grouped'
 _lock = threading.Lock()
-_flush_work = 1e11
+_flush_work = 2.5e11
 
 
 class _Queue(object):

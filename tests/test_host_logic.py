@@ -610,7 +610,7 @@ def test_factor_side_streams_host_logic():
         torchsso.join_factor_streams()        # nothing pending: no device is touched
     finally:
         torchsso.set_factor_streams(before)
-    assert torchsso.factor_streams() == 3     # the default
+    assert torchsso.factor_streams() == 2     # the default
 
 
 def test_factor_mode_host_logic():
