@@ -54,7 +54,7 @@ class _Queue(object):
 
 _deferred = {}     # device index -> _Queue
 _calls = {}        # device index -> engine calls made so far (deals them to the side streams)
-_inflight = {}     # device index -> list of (event, items) of calls the side streams may still run
+_inflight = {}     # device index -> list of (event, items, addresses written) of calls the side streams may still run
 _streams = {}      # device index -> list of (torch.cuda.Stream, torch.cuda.Event for the fork)
 _pending = {}      # device index -> set of lane indices with work since the last join
 
@@ -179,13 +179,24 @@ def _run_deferred(only=None):
                 for t in keep:
                     if t is not None:
                         t.record_stream(target)
+        jobs = [job for job, _, _ in items]
         if side is not None:
             with _lock:
                 fork.record(cur)
                 side.wait_event(fork)
+                # a call still in flight on ANOTHER side stream that writes a buffer this
+                # call reads or adds to (factors accumulated over MC samples): wait for it
+                touched = set()
+                for job in jobs:
+                    touched.add(job.C)
+                    if job.C_prev:
+                        touched.add(job.C_prev)
+                for done, _, written in _inflight.get(i, []):
+                    if not touched.isdisjoint(written):
+                        side.wait_event(done)
         for st in others:
             target.wait_stream(st)
-        _ops.factor_grouped([job for job, _, _ in items], device, stream=side)
+        _ops.factor_grouped(jobs, device, stream=side)
         if side is not None:
             # the tensors stay referenced until the caller's stream has been made to wait
             # for the side stream (join), or until the side stream is seen to have passed
@@ -193,7 +204,7 @@ def _run_deferred(only=None):
             done.record(side)
             with _lock:
                 held = [h for h in _inflight.get(i, []) if not h[0].query()]
-                held.append((done, items))
+                held.append((done, items, set(job.C for job in jobs)))
                 _inflight[i] = held
                 _pending.setdefault(i, set()).add(lane)
 

@@ -266,6 +266,7 @@ class KronCurvature(Curvature):
         KronCurvature._lanes_dealt += 1
         self._next = [None, None]        # receives the next running average
         self._jobs = [None, None]        # grouped mode: (signature, engine job, d, work) per factor
+        self._acc_into = None            # (TensorAccumulator, weight): see accumulate_into
         self._fresh = [False, False]     # _next[i] holds the next average (hook ran since the last step)
         self._prev_ok = [False, False]   # _next[i] holds the average before the current one
 
@@ -313,6 +314,16 @@ class KronCurvature(Curvature):
 
     # ---- raw factors ------------------------------------------------------------
 
+    def accumulate_into(self, accumulator, weight):
+        """Until `accumulator` is None again, the hooks add `weight` times each new factor to
+        the buffers of `accumulator` (a TensorAccumulator of [A, G]) in the epilogue of the
+        factor product itself, instead of storing the raw factor for somebody to add up
+        afterwards (the accumulation over MC samples or micro-steps of
+        optim/secondorder.py:175-182 and optim/vi.py:211-220 of the reference): no pass over
+        the factors, and nothing has to wait for the products before the running sum is
+        used.  `data`, `A` and `G` are None while this is on."""
+        self._acc_into = None if accumulator is None else (accumulator, float(weight))
+
     def _build_factor(self, idx, source, kind, scale, add_bias=False, **geometry):
         """Builds factor `idx` (0: A, 1: G) as  scale * P^T P  from the contiguous tensor
         `source` (`kind`: 'linear', 'conv_a' with the convolution's geometry, 'conv_g'):
@@ -328,9 +339,16 @@ class KronCurvature(Curvature):
             if out is None or out.shape != prev.shape:
                 out = torch.empty_like(prev)
             alpha, b = beta * scale, 1. - beta
+        elif self._acc_into is not None:
+            accumulator, weight = self._acc_into
+            d = self._factor_dim(idx, source, kind, add_bias, geometry)
+            out, fresh = accumulator.slot(idx, 2, (d, d), source)
+            prev = None
+            alpha, b = scale * weight, 0. if fresh else 1.
         else:
             prev, out = None, None
             alpha, b = scale, 0.
+        accumulating = not fused and self._acc_into is not None
         if _lanes.mode() == 'grouped' and device.type == 'cuda':
             # (the job object of this factor is reused from pass to pass: the engine copies
             # it when the queue runs, and a second product of a queued factor runs the queue)
@@ -371,6 +389,10 @@ class KronCurvature(Curvature):
             self._fresh[idx] = True
             self._prev_ok[idx] = False
             raw = None
+        elif accumulating:
+            raw = None
+            self._fresh[idx] = False
+            self._prev_ok[idx] = False
         else:
             raw = out
             self._fresh[idx] = False

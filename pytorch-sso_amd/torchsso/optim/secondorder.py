@@ -240,6 +240,19 @@ class SecondOrderOptimizer(Optimizer):
                             precondition=self.precondition_grad)
         return loss
 
+    def _begin_accumulation(self, weight):
+        """Before forward / backward passes whose factors will be accumulated with `weight`:
+        the Kronecker curvatures add their factors to the group's accumulator in the factor
+        products themselves (KronCurvature.accumulate_into), so `_accumulate` has only the
+        gradients and the diagonal curvatures left.  Used where no user code runs between the
+        passes that could ask for a single pass's factor (the MC loop of VIOptimizer.step);
+        accumulation over micro-steps, between which the caller has the floor, adds up stored
+        factors as the reference does."""
+        for group in self.param_groups:
+            curv = group['curv']
+            if curv is not None and curv.kind == 'kron' and not curv.fuse_ema:
+                curv.accumulate_into(group['acc_curv'], weight)
+
     def _accumulate(self, weight):
         """Adds weight * (current gradients, current curvature data) of every group to the
         group's accumulators (reference: secondorder.py:175-182, vi.py:211-220)."""
@@ -248,7 +261,7 @@ class SecondOrderOptimizer(Optimizer):
             accs.append(group['acc_grads'])
             datas.append([p.grad.data for p in group['params']])
             curv = group['curv']
-            if curv is not None:
+            if curv is not None and getattr(curv, '_acc_into', None) is None:
                 accs.append(group['acc_curv'])
                 datas.append(curv.data)
         TensorAccumulator.update_many(accs, datas, scale=weight)   # one launch for all layers
@@ -290,6 +303,8 @@ class SecondOrderOptimizer(Optimizer):
             curv = group['curv']
             if curv is not None:
                 curv.data = group['acc_curv'].get()
+                if curv.kind == 'kron':
+                    curv.accumulate_into(None, 0.)
 
     # ------------------------------------------------------------ update tail
 

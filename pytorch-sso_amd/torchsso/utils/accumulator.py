@@ -71,6 +71,23 @@ class TensorAccumulator(object):
             _ops.axpby_batched([x for src, _ in dsts_old for x in src],
                                [y for _, have in dsts_old for y in have], scale, 1.)
 
+    def slot(self, index, count, shape, like):
+        """(buffer, fresh) for tensor `index` of a list accumulation of `count` tensors whose
+        producers add into it themselves (a factor kernel with an accumulating epilogue):
+        `fresh` tells the producer that the buffer is new and must be written, not added to.
+        Every slot has to be filled before `get`."""
+        if self._accumulation is None:
+            self._accumulation = [None] * count
+        acc = self._accumulation
+        assert isinstance(acc, list) and len(acc) == count, 'accumulation of another shape exists'
+        buf = acc[index]
+        fresh = buf is None
+        if fresh:
+            buf = acc[index] = like.new_empty(shape)
+        else:
+            assert tuple(buf.shape) == tuple(shape)
+        return buf, fresh
+
     def update(self, data, scale=1.):
         self.check_type(data)
         if isinstance(data, list):

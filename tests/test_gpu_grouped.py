@@ -239,3 +239,59 @@ def test_second_pass_before_a_read_runs_the_queue():
     assert _lanes.deferred_count() == 1
     assert O.rel_fro(curv.A, O.factor_linear_a(x2.cpu(), True, D)) < TOL
     assert _lanes.deferred_count() == 0
+
+
+def vi_run(mode, steps=3):
+    import torchsso
+    before = torchsso.factor_mode()
+    torchsso.set_factor_mode(mode)
+    try:
+        dev = torch.device('cuda:0')
+        torch.manual_seed(7)
+        model = nn.Sequential(nn.Conv2d(3, 8, 3, padding=1), nn.ReLU(), nn.MaxPool2d(2),
+                              nn.Conv2d(8, 16, 3), nn.ReLU(), nn.Flatten(),
+                              nn.Linear(16 * 2 * 2, 10)).to(dev)
+        x = torch.randn(12, 3, 8, 8, device=dev)
+        y = torch.randint(0, 10, (12,), device=dev)
+        opt = torchsso.optim.VIOptimizer(
+            model, 1000, 'Cov', {'Conv2d': 'Kron', 'Linear': 'Kron'},
+            {'damping': 1e-3, 'ema_decay': 0.9}, lr=1e-2, momentum=0.9, num_mc_samples=3,
+            prior_variance=1, kl_weighting=1, seed=3)
+        seen = []
+
+        def closure():
+            model.zero_grad()
+            out = model(x)
+            loss = F.cross_entropy(out, y)
+            loss.backward()
+            return loss, out
+        for _ in range(steps):
+            opt.step(closure=closure)
+            seen.append([t.clone() for g in opt.param_groups for t in g['curv'].ema])
+        torch.cuda.synchronize()
+        return [p.detach().clone() for p in model.parameters()], seen
+    finally:
+        torchsso.set_factor_mode(before)
+
+
+def test_mc_loop_accumulates_in_the_factor_products():
+    """VIOptimizer: the factors of the MC samples are added up in the epilogue of the factor
+    products (nothing waits for them between the samples).  Same running averages and
+    parameters in grouped and in eager mode over three steps with posterior sampling, and
+    the running average after the first step is the mean over the samples of the factors an
+    independent pass computes (float64 oracle)."""
+    pg, eg = vi_run('grouped')
+    pe, ee = vi_run('eager')
+    for step, (a, b) in enumerate(zip(ee, eg)):
+        for t_e, t_g in zip(a, b):
+            assert O.rel_fro(t_g, t_e.double().cpu()) < 2e-5, step
+    for a, b in zip(pe, pg):
+        assert O.rel_fro(b, a.double().cpu()) < 1e-4
+    # first step: no posterior yet, every MC sample sees the same parameters, so the mean
+    # over the samples is the factor of one pass
+    torch.manual_seed(7)
+    model = nn.Sequential(nn.Conv2d(3, 8, 3, padding=1), nn.ReLU(), nn.MaxPool2d(2),
+                          nn.Conv2d(8, 16, 3), nn.ReLU(), nn.Flatten(), nn.Linear(16 * 2 * 2, 10))
+    x = torch.randn(12, 3, 8, 8, device='cuda:0').cpu()
+    A0 = O.factor_conv_a(x, (3, 3), (1, 1), (1, 1), (1, 1), True, D)
+    assert O.rel_fro(eg[0][0], A0) < TOL
