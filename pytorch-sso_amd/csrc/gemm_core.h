@@ -384,6 +384,44 @@ __device__ __forceinline__ void gemm_tile(const OPP& P, const OPQ& Q, int m0, in
   gemm_tile_cfg<2, 2>(P, Q, m0, n0, kbeg, kend, same, epi, smem);
 }
 
+// ---------------------------------------------------------------------------
+// A tile whose reduction was cut into `nparts` pieces, each computed by a workgroup of its
+// own that stored its raw 128x128 partial (EpiPartial) at parts + piece * 128 * 128: a
+// workgroup of a LATER launch adds the pieces up in order and hands every element to the
+// epilogue.  (Finishing in the same launch, by the piece that arrives last, was measured:
+// the device-wide fences it needs write back and invalidate the whole L2 of an XCD each
+// time, and the operand panels that the other workgroups share through that L2 with them.)
+// ---------------------------------------------------------------------------
+template <class EPI>
+__device__ __forceinline__ void splitk_sum(const float* parts, int nparts, int m0, int n0,
+                                           const EPI& epi) {
+  constexpr int TILE = BM * BN;
+  constexpr int PER_THREAD = TILE / 4 / NTHREADS;      // float4 groups per thread: 16
+  // piece by piece, the 16 loads of a thread in flight together
+  v4f acc[PER_THREAD];
+#pragma unroll
+  for (int i = 0; i < PER_THREAD; ++i)
+    acc[i] = *reinterpret_cast<const v4f*>(parts + 4 * ((int)threadIdx.x + NTHREADS * i));
+  for (int q = 1; q < nparts; ++q) {
+    const float* p = parts + (size_t)q * TILE;
+    v4f v[PER_THREAD];
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i)
+      v[i] = *reinterpret_cast<const v4f*>(p + 4 * ((int)threadIdx.x + NTHREADS * i));
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i) acc[i] += v[i];
+  }
+#pragma unroll
+  for (int i = 0; i < PER_THREAD; ++i) {
+    const int e = 4 * ((int)threadIdx.x + NTHREADS * i);
+    const int row = m0 + (e >> 7), col = n0 + (e & (BN - 1));
+    epi.store(row, col, acc[i].x);
+    epi.store(row, col + 1, acc[i].y);
+    epi.store(row, col + 2, acc[i].z);
+    epi.store(row, col + 3, acc[i].w);
+  }
+}
+
 // Workgroups are handed to the 8 XCDs round-robin in dispatch order, and each
 // XCD has its own L2.  This maps the dispatch index `id` of a 1-D problem of
 // `total` work items so that every XCD walks a CONTIGUOUS range of items:

@@ -28,6 +28,7 @@ struct LayerDesc {
   int dG, dA, dAw;       // dAw = dA - (has bias)
   float scale;
   int flags;         // factored preconditioning: bit 0 L is Wg, bit 1 R is Wa (else the inverses)
+  float* parts;      // pieces of the tiles whose reduction is cut (see tile_item)
 };
 
 constexpr int LAYER_CHUNK = 32;
@@ -107,18 +108,51 @@ struct EpiSplit {
 // products with its own operand layouts.
 // ---------------------------------------------------------------------------
 
+// A reduction against a triangular operand of T blocks is up to T blocks long, and a launch
+// lasts at least as long as its longest tile: a 4608-deep tile is 150 MFLOP on ONE compute
+// unit.  Where that is longer than the launch would take if its work were spread evenly
+// (few layers, or few tiles: the driver decides per product), the reductions are cut into
+// pieces of at most `pb` blocks, each a work item of the same launch that stores a raw
+// partial tile; a second, short launch adds the pieces of every cut tile up in order and
+// applies the epilogue (precond_finish_kernel).  Piece j exists for the tiles whose
+// reduction is longer than j * pb blocks: tfast - j * pb values of `fast`.  pb == 0: no
+// reduction is cut.
+__host__ __device__ inline int piece_count(int blocks, int pb) {
+  return pb > 0 ? (blocks + pb - 1) / pb : 1;
+}
+// work items of a layer in one product: tiles x pieces
+__host__ __device__ inline int piece_items(int tslow, int tfast, bool tri, int pb) {
+  if (!tri || pb <= 0) return tslow * tfast;
+  int n = 0;
+  for (int j = 0; j * pb < tfast; ++j) n += tslow * (tfast - j * pb);
+  return n;
+}
+
 // (slow, fast) tile indices of work item `local` of a layer with tslow x tfast tiles.
 // `tri`: the reduction length depends on `fast`; it grows with it if `grows`.
 struct TileItem {
   int slow, fast;
+  int piece, pieces;     // which piece of the tile's reduction, of how many
 };
 __device__ __forceinline__ TileItem tile_item(int local, int tslow, int tfast, bool tri,
-                                              bool grows) {
+                                              bool grows, int pb) {
   TileItem it;
+  it.piece = 0;
+  it.pieces = 1;
   if (tri) {
+    // piece j of all tiles that have one, then piece j + 1; within a piece the longest
+    // reductions first
+    int j = 0;
+    if (pb > 0)
+      while (local >= tslow * (tfast - j * pb)) {
+        local -= tslow * (tfast - j * pb);
+        ++j;
+      }
     const int rank = local / tslow;
     it.slow = local - rank * tslow;
     it.fast = grows ? tfast - 1 - rank : rank;
+    it.piece = j;
+    it.pieces = piece_count(grows ? it.fast + 1 : tfast - it.fast, pb);
   } else {
     const int item = xcd_remap(local, tslow * tfast);
     it.slow = item / tfast;
@@ -127,14 +161,46 @@ __device__ __forceinline__ TileItem tile_item(int local, int tslow, int tfast, b
   return it;
 }
 
+// One tile of a product: the whole reduction [k0, k1) into `epi`, or one piece of it as a
+// raw partial into the layer's piece area (tile `tile_id`, room for `max_pieces` each).
+template <class OPP, class OPQ, class EPI>
+__device__ __forceinline__ void tile_or_piece(const LayerDesc& m, const TileItem& it, int tile_id,
+                                              int max_pieces, int pb, const OPP& P, const OPQ& Q,
+                                              int m0, int n0, int M, int N, int k0, int k1,
+                                              const EPI& epi, float* smem) {
+  if (it.pieces == 1) {
+    EPI e = epi;
+    gemm_tile(P, Q, m0, n0, k0, k1, false, e, smem);
+    return;
+  }
+  const int kbeg = k0 + it.piece * (pb * BM);
+  const int kend = min(k1, kbeg + pb * BM);
+  float* parts = m.parts + ((size_t)tile_id * max_pieces + it.piece) * (BM * BN);
+  EpiPartial part{parts, m0, n0, M, N, BN};
+  gemm_tile(P, Q, m0, n0, kbeg, kend, false, part, smem);
+}
+
 // where the products of a layer between the first and the last put their result
 __device__ __forceinline__ float* second_half(const LayerDesc& m) {
   return m.Tt + (size_t)m.dG * m.dA;
 }
 
+// where the second, third and fourth product of a layer put their result
+__device__ __forceinline__ EpiSplit second_epilogue(const LayerDesc& m) {
+  return m.flags == 0 ? EpiSplit{m.outW, m.outb, nullptr, nullptr, m.dG, m.dA, m.dAw, 1.f}
+                      : EpiSplit{second_half(m), nullptr, nullptr, nullptr, m.dG, m.dA, m.dA, 1.f};
+}
+__device__ __forceinline__ EpiSplit third_epilogue(const LayerDesc& m) {
+  return (m.flags & 1) ? EpiSplit{m.Tt, nullptr, nullptr, nullptr, m.dG, m.dA, m.dA, 1.f}
+                       : EpiSplit{m.outW, m.outb, nullptr, nullptr, m.dG, m.dA, m.dAw, 1.f};
+}
+__device__ __forceinline__ EpiSplit fourth_epilogue(const LayerDesc& m) {
+  return EpiSplit{m.outW, m.outb, nullptr, nullptr, m.dG, m.dA, m.dAw, 1.f};
+}
+
 template <bool SAMPLE>
 __global__ __launch_bounds__(NTHREADS, 3) void precond_first_kernel(const LayerDesc* table,
-                                                                 const WorkList wl) {
+                                                                 const WorkList wl, int pb) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   int layer, local;
   work_find(wl, layer, local);
@@ -150,17 +216,18 @@ __global__ __launch_bounds__(NTHREADS, 3) void precond_first_kernel(const LayerD
     gemm_tile(P, Q, bi * BM, bj * BN, bj * BN, m.dG, false, epi, smem);
   } else {
     const bool tri = m.flags & 1;
-    const TileItem it = tile_item(local, ta, tg, tri, true);
+    const TileItem it = tile_item(local, ta, tg, tri, true, pb);
     const int bi = it.slow, bj = it.fast;            // bi over dA, bj over dG
     DenseKM P{m.V, m.vb, m.dAw, m.dA, m.vb ? 2 : 0};
     DenseKM Q{m.L, nullptr, m.dG, m.dG, 0};
-    gemm_tile(P, Q, bi * BM, bj * BN, 0, tri ? min(m.dG, (bj + 1) * BN) : m.dG, false, epi, smem);
+    tile_or_piece(m, it, bi + ta * bj, piece_count(tg, pb), pb, P, Q, bi * BM, bj * BN, m.dA, m.dG,
+                  0, tri ? min(m.dG, (bj + 1) * BN) : m.dG, epi, smem);
   }
 }
 
 template <bool SAMPLE>
 __global__ __launch_bounds__(NTHREADS, 3) void precond_second_kernel(const LayerDesc* table,
-                                                                 const WorkList wl) {
+                                                                 const WorkList wl, int pb) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   int layer, local;
   work_find(wl, layer, local);
@@ -176,59 +243,137 @@ __global__ __launch_bounds__(NTHREADS, 3) void precond_second_kernel(const Layer
     gemm_tile(P, Q, bi * BM, bj * BN, 0, min(m.dA, (bj + 1) * BN), false, epi, smem);
   } else {
     const bool tri = m.flags & 2;
-    const TileItem it = tile_item(local, tg, ta, tri, true);
+    const TileItem it = tile_item(local, tg, ta, tri, true, pb);
     const int bi = it.slow, bj = it.fast;            // bi over dG, bj over dA
-    const EpiSplit epi = m.flags == 0
-        ? EpiSplit{m.outW, m.outb, nullptr, nullptr, m.dG, m.dA, m.dAw, 1.f}
-        : EpiSplit{second_half(m), nullptr, nullptr, nullptr, m.dG, m.dA, m.dA, 1.f};
-    gemm_tile(P, Q, bi * BM, bj * BN, 0, tri ? min(m.dA, (bj + 1) * BN) : m.dA, false, epi, smem);
+    tile_or_piece(m, it, bi + tg * bj, piece_count(ta, pb), pb, P, Q, bi * BM, bj * BN, m.dG, m.dA,
+                  0, tri ? min(m.dA, (bj + 1) * BN) : m.dA, second_epilogue(m), smem);
   }
 }
 
 // third product, layers whose R is the factor Ya:  X' = X Ya^T, reduction a >= j
 __global__ __launch_bounds__(NTHREADS, 3) void precond_third_kernel(const LayerDesc* table,
-                                                                const WorkList wl) {
+                                                                const WorkList wl, int pb) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   int layer, local;
   work_find(wl, layer, local);
   const LayerDesc m = table[layer];
   const int ta = tiles128(m.dA), tg = tiles128(m.dG);
-  const TileItem it = tile_item(local, tg, ta, true, false);
+  const TileItem it = tile_item(local, tg, ta, true, false, pb);
   const int bi = it.slow, bj = it.fast;              // bi over dG, bj over dA
   DenseMK P{second_half(m), m.dA, m.dG};
   DenseMK Q{m.R, m.dA, m.dA};
-  const EpiSplit epi = (m.flags & 1)
-      ? EpiSplit{m.Tt, nullptr, nullptr, nullptr, m.dG, m.dA, m.dA, 1.f}
-      : EpiSplit{m.outW, m.outb, nullptr, nullptr, m.dG, m.dA, m.dAw, 1.f};
-  gemm_tile(P, Q, bi * BM, bj * BN, bj * BN, m.dA, false, epi, smem);
+  tile_or_piece(m, it, bi + tg * bj, piece_count(ta, pb), pb, P, Q, bi * BM, bj * BN, m.dG, m.dA,
+                bj * BN, m.dA, third_epilogue(m), smem);
 }
 
 // fourth product, layers whose L is the factor Yg:  U = Yg X', reduction k >= i
 __global__ __launch_bounds__(NTHREADS, 3) void precond_fourth_kernel(const LayerDesc* table,
-                                                                 const WorkList wl) {
+                                                                 const WorkList wl, int pb) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   int layer, local;
   work_find(wl, layer, local);
   const LayerDesc m = table[layer];
   const int ta = tiles128(m.dA), tg = tiles128(m.dG);
-  const TileItem it = tile_item(local, ta, tg, true, false);
+  const TileItem it = tile_item(local, ta, tg, true, false, pb);
   const int bi = it.fast, bj = it.slow;              // bi over dG, bj over dA
   DenseMK P{m.L, m.dG, m.dG};
   DenseKM Q{(m.flags & 2) ? m.Tt : second_half(m), nullptr, m.dA, m.dA, 0};
-  EpiSplit epi{m.outW, m.outb, nullptr, nullptr, m.dG, m.dA, m.dAw, 1.f};
-  gemm_tile(P, Q, bi * BM, bj * BN, bi * BM, m.dG, false, epi, smem);
+  tile_or_piece(m, it, bj + ta * bi, piece_count(tg, pb), pb, P, Q, bi * BM, bj * BN, m.dG, m.dA,
+                bi * BM, m.dG, fourth_epilogue(m), smem);
+}
+
+// The tiles of product `product` (0..3) whose reduction was cut: pieces added up in order,
+// result through the product's epilogue.  One work item per tile of the layers that take
+// part with a triangular operand; a tile of one piece was finished by its product.
+__global__ __launch_bounds__(NTHREADS) void precond_finish_kernel(const LayerDesc* table,
+                                                                  const WorkList wl, int product,
+                                                                  int pb) {
+  int layer, local;
+  work_find(wl, layer, local);
+  const LayerDesc m = table[layer];
+  const int ta = tiles128(m.dA), tg = tiles128(m.dG);
+  // (slow, fast) as the product numbers them; `local` = slow + tslow * fast = the tile id
+  const bool over_g = product == 0 || product == 3;      // the reduction runs over dG
+  const int tslow = over_g ? ta : tg, tfast = over_g ? tg : ta;
+  const int fast = local / tslow, slow = local - fast * tslow;
+  const bool grows = product < 2;
+  const int pieces = piece_count(grows ? fast + 1 : tfast - fast, pb);
+  if (pieces == 1) return;
+  const float* parts = m.parts + (size_t)local * piece_count(tfast, pb) * (BM * BN);
+  // rows of the result: dA for the first product (T^T), dG for the others
+  int bi, bj;
+  if (product == 0) { bi = slow; bj = fast; }          // bi over dA, bj over dG
+  else if (product == 3) { bi = fast; bj = slow; }     // bi over dG, bj over dA
+  else { bi = slow; bj = fast; }                       // bi over dG, bj over dA
+  if (product == 0)
+    splitk_sum(parts, pieces, bi * BM, bj * BN, EpiStore{m.Tt, m.dG, m.dA, m.dG, 1.f, 0.f, false});
+  else if (product == 1)
+    splitk_sum(parts, pieces, bi * BM, bj * BN, second_epilogue(m));
+  else if (product == 2)
+    splitk_sum(parts, pieces, bi * BM, bj * BN, third_epilogue(m));
+  else
+    splitk_sum(parts, pieces, bi * BM, bj * BN, fourth_epilogue(m));
 }
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 constexpr int PRODUCTS = 4;
 
+// Blocks per piece of the cut reductions of a product (0: none is cut).  `work` = sum over
+// tiles of their reduction length in blocks, `longest` = the longest of them: with the work
+// spread evenly over the chip's resident workgroups (3 per CU) a launch would last
+// work / 768 block times; it cannot end before its longest tile does.
+constexpr int MIN_PIECE_BLOCKS = 4;
+static int piece_blocks(long work, int longest) {
+  const long even = work / 768 + 1;
+  if (longest <= MIN_PIECE_BLOCKS || 3 * (long)longest <= 4 * even) return 0;
+  const long pb = std::max<long>(MIN_PIECE_BLOCKS, even / 2);
+  return pb >= longest ? 0 : (int)pb;
+}
+
+// Piece size of each product from the shape of its launch.  flags == nullptr: every side of
+// every layer is a triangular factor (what the scratch is sized for).
+static void plan_pieces(int layers, const int* dG, const int* dA, const int* flags, bool any_tri,
+                        int (&pbs)[4]) {
+  for (int product = 0; product < 4; ++product) {
+    long work = 0;
+    int longest = 0;
+    const bool over_g = product == 0 || product == 3;
+    for (int l = 0; any_tri && l < layers; ++l) {
+      const int ta = cdiv(dA[l], BN), tg = cdiv(dG[l], BM);
+      const int f = flags ? flags[l] : 3;
+      const int tslow = over_g ? ta : tg, tfast = over_g ? tg : ta;
+      const bool tri = over_g ? (f & 1) : (f & 2);
+      if (product >= 2 && !tri) continue;
+      work += tri ? (long)tslow * tfast * (tfast + 1) / 2 : (long)tslow * tfast * tfast;
+      if (tri) longest = std::max(longest, tfast);
+    }
+    pbs[product] = any_tri ? piece_blocks(work, longest) : 0;
+  }
+}
+
+// floats of the piece area of a layer under the piece sizes `pbs`: room for the pieces of
+// the longest reduction, for every tile
+static size_t piece_floats(int dG, int dA, const int (&pbs)[4]) {
+  const int ta = cdiv(dA, BN), tg = cdiv(dG, BM);
+  int most = 1;
+  for (int product = 0; product < 4; ++product) {
+    const bool over_g = product == 0 || product == 3;
+    most = std::max(most, piece_count(over_g ? tg : ta, pbs[product]));
+  }
+  return most > 1 ? (size_t)ta * tg * most * (BM * BN) : 0;
+}
+
 // scratch: one descriptor table per product, then per layer dG*dA floats (twice that when
-// `factored`: a layer with a factored side keeps two results in flight)
+// `factored`: a layer with a factored side keeps two results in flight) and its piece area
 static size_t precond_workspace(int layers, const int* dG, const int* dA, bool factored) {
   size_t bytes = PRODUCTS * align256((size_t)layers * sizeof(LayerDesc));
-  for (int l = 0; l < layers; ++l)
+  int pbs[4];
+  plan_pieces(layers, dG, dA, nullptr, factored, pbs);
+  for (int l = 0; l < layers; ++l) {
     bytes += align256((size_t)(factored ? 2 : 1) * dG[l] * dA[l] * sizeof(float));
+    if (factored) bytes += align256(piece_floats(dG[l], dA[l], pbs) * sizeof(float));
+  }
   return bytes;
 }
 
@@ -252,17 +397,46 @@ static int run_layers(int layers, const int* dG, const int* dA, const float* con
   // fourth, dA for the second and third), through a descriptor table of its own.
   const size_t table_bytes = align256((size_t)layers * sizeof(LayerDesc));
   char* tbase = (char*)workspace + PRODUCTS * table_bytes;
-  std::vector<size_t> toff(layers);
+  // pieces as large as the scratch was sized for, at least (the query assumed that every
+  // side is a triangular factor), and none where it left no room
+  int pbs_room[4], pbs[PRODUCTS];
+  plan_pieces(layers, dG, dA, nullptr, flags != nullptr && !sample, pbs_room);
+  plan_pieces(layers, dG, dA, flags, flags != nullptr && !sample, pbs);
+  for (int product = 0; product < PRODUCTS; ++product)
+    pbs[product] = pbs[product] > 0 && pbs_room[product] > 0
+                       ? std::max(pbs[product], pbs_room[product]) : 0;
+  std::vector<size_t> toff(layers), poff(layers);
   size_t off = 0;
   for (int l = 0; l < layers; ++l) {
     toff[l] = off;
     off += align256((size_t)(flags ? 2 : 1) * dG[l] * dA[l] * sizeof(float));
+    poff[l] = off;
+    if (flags) off += align256(piece_floats(dG[l], dA[l], pbs_room) * sizeof(float));
   }
-  // work items of layer l in a product: its tiles, or none where it takes no part
-  auto items = [&](int product, int l) {
+  // per product: is the reduction of layer l against a triangular operand, over how many
+  // blocks (tfast), with how many tiles across (tslow)
+  auto shape = [&](int product, int l, bool& takes_part, bool& tri, int& tslow, int& tfast) {
     const int ta = cdiv(dA[l], BN), tg = cdiv(dG[l], BM);
     const bool gfac = flags && (flags[l] & 1), afac = flags && (flags[l] & 2);
-    return (product < 2 || (product == 2 ? afac : gfac)) ? ta * tg : 0;
+    const bool over_g = product == 0 || product == 3;
+    tslow = over_g ? ta : tg;
+    tfast = over_g ? tg : ta;
+    tri = over_g ? gfac : afac;
+    takes_part = product < 2 || tri;
+  };
+  // work items of layer l in a product: its tiles x pieces, or none where it takes no part
+  auto items = [&](int product, int l) {
+    bool part, tri;
+    int tslow, tfast;
+    shape(product, l, part, tri, tslow, tfast);
+    return part ? piece_items(tslow, tfast, tri, pbs[product]) : 0;
+  };
+  // ... and in the launch that finishes the cut tiles of the product
+  auto finish_items = [&](int product, int l) {
+    bool part, tri;
+    int tslow, tfast;
+    shape(product, l, part, tri, tslow, tfast);
+    return part && tri && piece_count(tfast, pbs[product]) > 1 ? tslow * tfast : 0;
   };
   std::vector<int> order(layers);
   for (int product = 0; product < PRODUCTS; ++product) {
@@ -291,12 +465,14 @@ static int run_layers(int layers, const int* dG, const int* dA, const float* con
         d.dAw = dA[l] - (has_bias[l] ? 1 : 0);
         d.scale = scale;
         d.flags = flags ? flags[l] : 0;
+        d.parts = flags ? (float*)(tbase + poff[l]) : nullptr;
       }
       hipLaunchKernelGGL(layer_setup_kernel, dim3(1), dim3(LAYER_CHUNK), 0, stream, chunk,
                          table, s0, cnt);
     }
     // every launch of a product is enqueued before any of the next one (stream order is
     // the dependency)
+    const int pb = pbs[product];
     for (int s0 = 0; s0 < layers; s0 += WL_MAX) {
       WorkList wl;
       wl.first = s0;
@@ -307,17 +483,30 @@ static int run_layers(int layers, const int* dG, const int* dA, const float* con
       if (wl.cum[wl.n] == 0) continue;
       const dim3 grid(wl.cum[wl.n]);
       if (product == 0) {
-        if (sample) KFAC_LAUNCH_TILE2(precond_first_kernel<true>, grid, stream, table, wl);
-        else KFAC_LAUNCH_TILE2(precond_first_kernel<false>, grid, stream, table, wl);
+        if (sample) KFAC_LAUNCH_TILE2(precond_first_kernel<true>, grid, stream, table, wl, pb);
+        else KFAC_LAUNCH_TILE2(precond_first_kernel<false>, grid, stream, table, wl, pb);
       } else if (product == 1) {
-        if (sample) KFAC_LAUNCH_TILE2(precond_second_kernel<true>, grid, stream, table, wl);
-        else KFAC_LAUNCH_TILE2(precond_second_kernel<false>, grid, stream, table, wl);
+        if (sample) KFAC_LAUNCH_TILE2(precond_second_kernel<true>, grid, stream, table, wl, pb);
+        else KFAC_LAUNCH_TILE2(precond_second_kernel<false>, grid, stream, table, wl, pb);
       } else if (product == 2) {
-        KFAC_LAUNCH_TILE2(precond_third_kernel, grid, stream, table, wl);
+        KFAC_LAUNCH_TILE2(precond_third_kernel, grid, stream, table, wl, pb);
       } else {
-        KFAC_LAUNCH_TILE2(precond_fourth_kernel, grid, stream, table, wl);
+        KFAC_LAUNCH_TILE2(precond_fourth_kernel, grid, stream, table, wl, pb);
       }
     }
+    if (pb > 0)
+      for (int s0 = 0; s0 < layers; s0 += WL_MAX) {
+        WorkList wl;
+        wl.first = s0;
+        wl.n = std::min(WL_MAX, layers - s0);
+        wl.cum[0] = 0;
+        for (int i = 0; i < wl.n; ++i)
+          wl.cum[i + 1] = wl.cum[i] + finish_items(product, order[s0 + i]);
+        for (int i = wl.n + 1; i <= WL_MAX; ++i) wl.cum[i] = wl.cum[wl.n];
+        if (wl.cum[wl.n] == 0) continue;
+        hipLaunchKernelGGL(precond_finish_kernel, dim3(wl.cum[wl.n]), dim3(NTHREADS), 0, stream,
+                           table, wl, product, pb);
+      }
   }
   return launch_status();
 }
