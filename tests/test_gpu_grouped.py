@@ -295,3 +295,51 @@ def test_mc_loop_accumulates_in_the_factor_products():
     x = torch.randn(12, 3, 8, 8, device='cuda:0').cpu()
     A0 = O.factor_conv_a(x, (3, 3), (1, 1), (1, 1), (1, 1), True, D)
     assert O.rel_fro(eg[0][0], A0) < TOL
+
+
+def test_queue_runs_on_a_work_threshold_and_across_streams():
+    """The queue also runs when the collected work passes the threshold (here: every product
+    by itself), and products queued under another stream than the one that reads the factors
+    wait for that stream's work: same factors as the eager mode either way."""
+    import torchsso
+    from torchsso import _lanes
+    dev = torch.device('cuda:0')
+    before = _lanes.flush_work()
+
+    def factors(mode, work, side_stream):
+        torchsso.set_factor_mode(mode)
+        torchsso.set_factor_flush_work(work)
+        torch.manual_seed(11)
+        conv = nn.Conv2d(6, 10, 3, padding=1).to(dev)
+        lin = nn.Linear(10 * 8 * 8, 7).to(dev)
+        cc = torchsso.KronCovConv2d(conv, ema_decay=1.)
+        cl = torchsso.KronCovLinear(lin, ema_decay=1.)
+        x = torch.randn(16, 6, 8, 8, device=dev)
+        torch.cuda.synchronize()
+        if side_stream:
+            s = torch.cuda.Stream()
+            with torch.cuda.stream(s):
+                # a slow producer in front of the layers: the products must wait for it
+                big = torch.randn(4096, 4096, device=dev)
+                for _ in range(6):
+                    big = big @ big * 1e-3
+                x2 = x + big[:1, :1].reshape(1, 1, 1, 1) * 0
+                out = lin(conv(x2).flatten(1))
+                out.sum().backward()
+        else:
+            out = lin(conv(x).flatten(1))
+            out.sum().backward()
+        res = [cc.A.clone(), cc.G.clone(), cl.A.clone(), cl.G.clone()]     # read on the default stream
+        torch.cuda.synchronize()
+        return res
+    try:
+        ref = factors('eager', before, False)
+        for work, side in ((1., False), (None, False), (before, True), (1., True)):
+            got = factors('grouped', work, side)
+            for a, b in zip(ref, got):
+                assert torch.isfinite(b).all()
+                assert O.rel_fro(b, a.double().cpu()) < 1e-5, (work, side)
+        assert _lanes.deferred_count() == 0
+    finally:
+        torchsso.set_factor_mode('grouped')
+        torchsso.set_factor_flush_work(before)
