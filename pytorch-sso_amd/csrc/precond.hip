@@ -122,7 +122,8 @@ __host__ __device__ inline int piece_count(int blocks, int pb) {
 }
 // work items of a layer in one product: tiles x pieces
 __host__ __device__ inline int piece_items(int tslow, int tfast, bool tri, int pb) {
-  if (!tri || pb <= 0) return tslow * tfast;
+  if (pb <= 0) return tslow * tfast;
+  if (!tri) return tslow * tfast * piece_count(tfast, pb);    // dense: all reductions tfast blocks
   int n = 0;
   for (int j = 0; j * pb < tfast; ++j) n += tslow * (tfast - j * pb);
   return n;
@@ -154,7 +155,11 @@ __device__ __forceinline__ TileItem tile_item(int local, int tslow, int tfast, b
     it.piece = j;
     it.pieces = piece_count(grows ? it.fast + 1 : tfast - it.fast, pb);
   } else {
-    const int item = xcd_remap(local, tslow * tfast);
+    // a dense operand: every reduction is tfast blocks long; piece after piece
+    const int tiles = tslow * tfast;
+    it.pieces = piece_count(tfast, pb);
+    it.piece = local / tiles;
+    const int item = xcd_remap(local - it.piece * tiles, tiles);
     it.slow = item / tfast;
     it.fast = item - it.slow * tfast;
   }
@@ -190,6 +195,9 @@ __device__ __forceinline__ EpiSplit second_epilogue(const LayerDesc& m) {
   return m.flags == 0 ? EpiSplit{m.outW, m.outb, nullptr, nullptr, m.dG, m.dA, m.dAw, 1.f}
                       : EpiSplit{second_half(m), nullptr, nullptr, nullptr, m.dG, m.dA, m.dA, 1.f};
 }
+__device__ __forceinline__ EpiSplit sample_epilogue(const LayerDesc& m) {
+  return EpiSplit{m.outW, m.outb, m.meanW, m.meanb, m.dG, m.dA, m.dAw, m.scale};
+}
 __device__ __forceinline__ EpiSplit third_epilogue(const LayerDesc& m) {
   return (m.flags & 1) ? EpiSplit{m.Tt, nullptr, nullptr, nullptr, m.dG, m.dA, m.dA, 1.f}
                        : EpiSplit{m.outW, m.outb, nullptr, nullptr, m.dG, m.dA, m.dAw, 1.f};
@@ -208,12 +216,13 @@ __global__ __launch_bounds__(NTHREADS, 3) void precond_first_kernel(const LayerD
   const int ta = tiles128(m.dA), tg = tiles128(m.dG);
   EpiStore epi{m.Tt, m.dG, m.dA, m.dG, 1.f, 0.f, false};
   if (SAMPLE) {
-    const int item = xcd_remap(local, ta * tg);
-    const int bi = item / tg, bj = item - bi * tg;   // bi over dA, bj over dG
     // noise E is a plain dG x dA matrix; U_G is upper triangular: L(k, i) = U_G[i][k], k >= i
+    const TileItem it = tile_item(local, ta, tg, true, false, pb);
+    const int bi = it.slow, bj = it.fast;            // bi over dA, bj over dG
     DenseKM P{m.V, nullptr, m.dA, m.dA, 0};
     DenseMK Q{m.L, m.dG, m.dG};
-    gemm_tile(P, Q, bi * BM, bj * BN, bj * BN, m.dG, false, epi, smem);
+    tile_or_piece(m, it, bi + ta * bj, piece_count(tg, pb), pb, P, Q, bi * BM, bj * BN, m.dA, m.dG,
+                  bj * BN, m.dG, epi, smem);
   } else {
     const bool tri = m.flags & 1;
     const TileItem it = tile_item(local, ta, tg, tri, true, pb);
@@ -236,11 +245,11 @@ __global__ __launch_bounds__(NTHREADS, 3) void precond_second_kernel(const Layer
   DenseKM P{m.Tt, nullptr, m.dG, m.dG, 0};
   DenseKM Q{m.R, nullptr, m.dA, m.dA, 0};
   if (SAMPLE) {
-    const int item = xcd_remap(local, ta * tg);
-    const int bi = item / ta, bj = item - bi * ta;   // bi over dG, bj over dA
-    EpiSplit epi{m.outW, m.outb, m.meanW, m.meanb, m.dG, m.dA, m.dAw, m.scale};
     // U_A is upper triangular: rows a > j are zero, so the sum stops at the tile's last column
-    gemm_tile(P, Q, bi * BM, bj * BN, 0, min(m.dA, (bj + 1) * BN), false, epi, smem);
+    const TileItem it = tile_item(local, tg, ta, true, true, pb);
+    const int bi = it.slow, bj = it.fast;            // bi over dG, bj over dA
+    tile_or_piece(m, it, bi + tg * bj, piece_count(ta, pb), pb, P, Q, bi * BM, bj * BN, m.dG, m.dA,
+                  0, min(m.dA, (bj + 1) * BN), sample_epilogue(m), smem);
   } else {
     const bool tri = m.flags & 2;
     const TileItem it = tile_item(local, tg, ta, tri, true, pb);
@@ -287,7 +296,7 @@ __global__ __launch_bounds__(NTHREADS, 3) void precond_fourth_kernel(const Layer
 // part with a triangular operand; a tile of one piece was finished by its product.
 __global__ __launch_bounds__(NTHREADS) void precond_finish_kernel(const LayerDesc* table,
                                                                   const WorkList wl, int product,
-                                                                  int pb) {
+                                                                  int pb, int sample) {
   int layer, local;
   work_find(wl, layer, local);
   const LayerDesc m = table[layer];
@@ -296,8 +305,9 @@ __global__ __launch_bounds__(NTHREADS) void precond_finish_kernel(const LayerDes
   const bool over_g = product == 0 || product == 3;      // the reduction runs over dG
   const int tslow = over_g ? ta : tg, tfast = over_g ? tg : ta;
   const int fast = local / tslow, slow = local - fast * tslow;
-  const bool grows = product < 2;
-  const int pieces = piece_count(grows ? fast + 1 : tfast - fast, pb);
+  const bool grows = sample ? product == 1 : product < 2;
+  const bool tri = sample || (m.flags & (over_g ? 1 : 2));
+  const int pieces = piece_count(!tri ? tfast : (grows ? fast + 1 : tfast - fast), pb);
   if (pieces == 1) return;
   const float* parts = m.parts + (size_t)local * piece_count(tfast, pb) * (BM * BN);
   // rows of the result: dA for the first product (T^T), dG for the others
@@ -308,7 +318,7 @@ __global__ __launch_bounds__(NTHREADS) void precond_finish_kernel(const LayerDes
   if (product == 0)
     splitk_sum(parts, pieces, bi * BM, bj * BN, EpiStore{m.Tt, m.dG, m.dA, m.dG, 1.f, 0.f, false});
   else if (product == 1)
-    splitk_sum(parts, pieces, bi * BM, bj * BN, second_epilogue(m));
+    splitk_sum(parts, pieces, bi * BM, bj * BN, sample ? sample_epilogue(m) : second_epilogue(m));
   else if (product == 2)
     splitk_sum(parts, pieces, bi * BM, bj * BN, third_epilogue(m));
   else
@@ -334,19 +344,19 @@ static int piece_blocks(long work, int longest) {
 // Piece size of each product from the shape of its launch.  flags == nullptr: every side of
 // every layer is a triangular factor (what the scratch is sized for).
 static void plan_pieces(int layers, const int* dG, const int* dA, const int* flags, bool any_tri,
-                        int (&pbs)[4]) {
+                        int (&pbs)[4], bool sample = false) {
   for (int product = 0; product < 4; ++product) {
     long work = 0;
     int longest = 0;
     const bool over_g = product == 0 || product == 3;
-    for (int l = 0; any_tri && l < layers; ++l) {
+    for (int l = 0; any_tri && !(sample && product >= 2) && l < layers; ++l) {
       const int ta = cdiv(dA[l], BN), tg = cdiv(dG[l], BM);
       const int f = flags ? flags[l] : 3;
       const int tslow = over_g ? ta : tg, tfast = over_g ? tg : ta;
       const bool tri = over_g ? (f & 1) : (f & 2);
       if (product >= 2 && !tri) continue;
       work += tri ? (long)tslow * tfast * (tfast + 1) / 2 : (long)tslow * tfast * tfast;
-      if (tri) longest = std::max(longest, tfast);
+      longest = std::max(longest, tfast);
     }
     pbs[product] = any_tri ? piece_blocks(work, longest) : 0;
   }
@@ -368,11 +378,13 @@ static size_t piece_floats(int dG, int dA, const int (&pbs)[4]) {
 // `factored`: a layer with a factored side keeps two results in flight) and its piece area
 static size_t precond_workspace(int layers, const int* dG, const int* dA, bool factored) {
   size_t bytes = PRODUCTS * align256((size_t)layers * sizeof(LayerDesc));
+  // (the piece area is there for both queries: posterior sampling, which shares the query of
+  // the explicit preconditioning, multiplies by triangular factors as well)
   int pbs[4];
-  plan_pieces(layers, dG, dA, nullptr, factored, pbs);
+  plan_pieces(layers, dG, dA, nullptr, true, pbs);
   for (int l = 0; l < layers; ++l) {
     bytes += align256((size_t)(factored ? 2 : 1) * dG[l] * dA[l] * sizeof(float));
-    if (factored) bytes += align256(piece_floats(dG[l], dA[l], pbs) * sizeof(float));
+    bytes += align256(piece_floats(dG[l], dA[l], pbs) * sizeof(float));
   }
   return bytes;
 }
@@ -399,9 +411,11 @@ static int run_layers(int layers, const int* dG, const int* dA, const float* con
   char* tbase = (char*)workspace + PRODUCTS * table_bytes;
   // pieces as large as the scratch was sized for, at least (the query assumed that every
   // side is a triangular factor), and none where it left no room
+  const std::vector<int> no_flags(layers, 0);     // explicit inverses on both sides
   int pbs_room[4], pbs[PRODUCTS];
-  plan_pieces(layers, dG, dA, nullptr, flags != nullptr && !sample, pbs_room);
-  plan_pieces(layers, dG, dA, flags, flags != nullptr && !sample, pbs);
+  const int* const real_flags = flags ? flags : (sample ? nullptr : no_flags.data());
+  plan_pieces(layers, dG, dA, nullptr, true, pbs_room);
+  plan_pieces(layers, dG, dA, real_flags, true, pbs, sample);
   for (int product = 0; product < PRODUCTS; ++product)
     pbs[product] = pbs[product] > 0 && pbs_room[product] > 0
                        ? std::max(pbs[product], pbs_room[product]) : 0;
@@ -411,18 +425,18 @@ static int run_layers(int layers, const int* dG, const int* dA, const float* con
     toff[l] = off;
     off += align256((size_t)(flags ? 2 : 1) * dG[l] * dA[l] * sizeof(float));
     poff[l] = off;
-    if (flags) off += align256(piece_floats(dG[l], dA[l], pbs_room) * sizeof(float));
+    off += align256(piece_floats(dG[l], dA[l], pbs_room) * sizeof(float));
   }
   // per product: is the reduction of layer l against a triangular operand, over how many
   // blocks (tfast), with how many tiles across (tslow)
   auto shape = [&](int product, int l, bool& takes_part, bool& tri, int& tslow, int& tfast) {
     const int ta = cdiv(dA[l], BN), tg = cdiv(dG[l], BM);
-    const bool gfac = flags && (flags[l] & 1), afac = flags && (flags[l] & 2);
+    const bool gfac = sample || (flags && (flags[l] & 1)), afac = sample || (flags && (flags[l] & 2));
     const bool over_g = product == 0 || product == 3;
     tslow = over_g ? ta : tg;
     tfast = over_g ? tg : ta;
     tri = over_g ? gfac : afac;
-    takes_part = product < 2 || tri;
+    takes_part = product < 2 || (tri && !sample);
   };
   // work items of layer l in a product: its tiles x pieces, or none where it takes no part
   auto items = [&](int product, int l) {
@@ -436,7 +450,7 @@ static int run_layers(int layers, const int* dG, const int* dA, const float* con
     bool part, tri;
     int tslow, tfast;
     shape(product, l, part, tri, tslow, tfast);
-    return part && tri && piece_count(tfast, pbs[product]) > 1 ? tslow * tfast : 0;
+    return part && piece_count(tfast, pbs[product]) > 1 ? tslow * tfast : 0;
   };
   std::vector<int> order(layers);
   for (int product = 0; product < PRODUCTS; ++product) {
@@ -465,7 +479,7 @@ static int run_layers(int layers, const int* dG, const int* dA, const float* con
         d.dAw = dA[l] - (has_bias[l] ? 1 : 0);
         d.scale = scale;
         d.flags = flags ? flags[l] : 0;
-        d.parts = flags ? (float*)(tbase + poff[l]) : nullptr;
+        d.parts = (float*)(tbase + poff[l]);
       }
       hipLaunchKernelGGL(layer_setup_kernel, dim3(1), dim3(LAYER_CHUNK), 0, stream, chunk,
                          table, s0, cnt);
@@ -505,7 +519,7 @@ static int run_layers(int layers, const int* dG, const int* dA, const float* con
         for (int i = wl.n + 1; i <= WL_MAX; ++i) wl.cum[i] = wl.cum[wl.n];
         if (wl.cum[wl.n] == 0) continue;
         hipLaunchKernelGGL(precond_finish_kernel, dim3(wl.cum[wl.n]), dim3(NTHREADS), 0, stream,
-                           table, wl, product, pb);
+                           table, wl, product, pb, sample ? 1 : 0);
       }
   }
   return launch_status();
