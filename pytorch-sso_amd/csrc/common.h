@@ -54,6 +54,22 @@ double conv_a_taps_grouped_executed_flops(int count, const TapsJob* jobs);
 int conv_a_taps_grouped(int count, const TapsJob* jobs, void* workspace, size_t workspace_bytes,
                         hipStream_t stream);
 
+// Blocks per piece of the cut reductions of a launch of 128x128 tiles (0: none is cut).
+// `work` = sum over the tiles of their reduction length in blocks, `longest` = the longest
+// of them: with the work spread evenly over the chip's resident workgroups (3 per CU) the
+// launch would last work / 768 block times, and it cannot end before its longest tile does
+// (which shares its compute unit with two other workgroups until the launch thins out).
+// Where the longest tile is the longer of the two, reductions are cut into pieces that are
+// work items of the same launch and store raw partial tiles; a short launch afterwards adds
+// the pieces of every cut tile up in order (splitk_sum).
+constexpr int MIN_PIECE_BLOCKS = 4;
+inline int piece_blocks(long work, int longest) {
+  const long even = work / 768 + 1;
+  if (longest <= MIN_PIECE_BLOCKS || 3 * (long)longest <= 4 * even) return 0;
+  const long pb = even / 2 > MIN_PIECE_BLOCKS ? even / 2 : MIN_PIECE_BLOCKS;
+  return pb >= longest ? 0 : (int)pb;
+}
+
 inline int launch_status() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? KFAC_OK : KFAC_ERR_LAUNCH;

@@ -392,9 +392,15 @@ __device__ __forceinline__ void gemm_tile(const OPP& P, const OPQ& Q, int m0, in
 // the device-wide fences it needs write back and invalidate the whole L2 of an XCD each
 // time, and the operand panels that the other workgroups share through that L2 with them.)
 // ---------------------------------------------------------------------------
+// pieces of a reduction of `blocks` 128-blocks cut at `pb` blocks (pb <= 0: not cut)
+__host__ __device__ inline int piece_count(int blocks, int pb) {
+  return pb > 0 ? (blocks + pb - 1) / pb : 1;
+}
+
+// (`stride`: floats from one piece of the tile to the next)
 template <class EPI>
 __device__ __forceinline__ void splitk_sum(const float* parts, int nparts, int m0, int n0,
-                                           const EPI& epi) {
+                                           const EPI& epi, size_t stride = BM * BN) {
   constexpr int TILE = BM * BN;
   constexpr int PER_THREAD = TILE / 4 / NTHREADS;      // float4 groups per thread: 16
   // piece by piece, the 16 loads of a thread in flight together
@@ -403,7 +409,7 @@ __device__ __forceinline__ void splitk_sum(const float* parts, int nparts, int m
   for (int i = 0; i < PER_THREAD; ++i)
     acc[i] = *reinterpret_cast<const v4f*>(parts + 4 * ((int)threadIdx.x + NTHREADS * i));
   for (int q = 1; q < nparts; ++q) {
-    const float* p = parts + (size_t)q * TILE;
+    const float* p = parts + (size_t)q * stride;
     v4f v[PER_THREAD];
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i)

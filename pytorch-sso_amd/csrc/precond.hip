@@ -117,9 +117,6 @@ struct EpiSplit {
 // applies the epilogue (precond_finish_kernel).  Piece j exists for the tiles whose
 // reduction is longer than j * pb blocks: tfast - j * pb values of `fast`.  pb == 0: no
 // reduction is cut.
-__host__ __device__ inline int piece_count(int blocks, int pb) {
-  return pb > 0 ? (blocks + pb - 1) / pb : 1;
-}
 // work items of a layer in one product: tiles x pieces
 __host__ __device__ inline int piece_items(int tslow, int tfast, bool tri, int pb) {
   if (pb <= 0) return tslow * tfast;
@@ -328,18 +325,6 @@ __global__ __launch_bounds__(NTHREADS) void precond_finish_kernel(const LayerDes
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 constexpr int PRODUCTS = 4;
-
-// Blocks per piece of the cut reductions of a product (0: none is cut).  `work` = sum over
-// tiles of their reduction length in blocks, `longest` = the longest of them: with the work
-// spread evenly over the chip's resident workgroups (3 per CU) a launch would last
-// work / 768 block times; it cannot end before its longest tile does.
-constexpr int MIN_PIECE_BLOCKS = 4;
-static int piece_blocks(long work, int longest) {
-  const long even = work / 768 + 1;
-  if (longest <= MIN_PIECE_BLOCKS || 3 * (long)longest <= 4 * even) return 0;
-  const long pb = std::max<long>(MIN_PIECE_BLOCKS, even / 2);
-  return pb >= longest ? 0 : (int)pb;
-}
 
 // Piece size of each product from the shape of its launch.  flags == nullptr: every side of
 // every layer is a triangular factor (what the scratch is sized for).
