@@ -2,12 +2,15 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
                     [--workload resnet50|alexnet_fc|convnet|mlp|noisy_kfac|resnet50_train]
-                    [--factor-streams N] [--no-cpu-baseline] [--copy-calibration]
+                    [--factor-mode grouped|eager] [--factor-streams N] [--factor-flush-work W]
+                    [--explicit-inverse] [--no-cpu-baseline] [--copy-calibration]
 
 A "step" is one pass of the K-FAC hot path over one batch of synthetic input,
 driven through the public torchsso API: for every layer the two Kronecker
-factors are built from that layer's input and output gradient (what the
-forward / backward hooks do), then SecondOrderOptimizer.step() runs the running
+factors are built from that layer's input and output gradient (the forward hooks
+in layer order, then the backward hooks in reverse order, as in a training pass;
+they queue the products, which run in a few grouped engine calls), then
+SecondOrderOptimizer.step() runs the running
 average, the pi-damped inversion of all factors, the preconditioning of all
 gradients and the parameter update.  The default workload is BASELINE config 3:
 the 53 convolutions + fc of a ResNet-50 at batch 32, 224x224 (real per-layer
@@ -320,7 +323,7 @@ class LayerSet(object):
             n += sum(t.numel() * 4 for t in lst)
         return n
 
-    # -- the three phases of a step -----------------------------------------
+    # -- the parts of a step ---------------------------------------------------
     def build_factors(self, kinds=('conv', 'linear', 'bn')):
         """The hooks of one training pass: the forward hooks in layer order, then the backward
         hooks in reverse order."""
@@ -339,8 +342,8 @@ class LayerSet(object):
         self.flat_grad.copy_(self.flat_raw)
 
     def step(self):
-        # the factor products go to the side streams first; the copy that stands in for the
-        # backward pass's fresh gradients then runs beside them, as a backward pass would
+        # the factor products go to the side streams; the copy that stands in for the
+        # backward pass's fresh gradients runs beside them, as a backward pass would
         self.build_factors()
         self.restore_grads()
         self.opt.step()

@@ -26,9 +26,12 @@ deterministic and each stream has its own scratch.
 Grouped mode (`set_mode('grouped')`, the default) goes one step further: a hook only
 describes its product (`defer`) and keeps the tensor it reads alive; the first reader of
 factor data (`join()`, as before) hands all products collected so far to ONE engine call,
-which runs them as a handful of launches holding the work items of all layers.  The
-side streams are not used then.  `set_mode('eager')` runs every product in its hook, on
-the side streams, as described above.
+which runs them as a handful of launches holding the work items of all layers.  The queue
+also runs at the first backward hook of a pass (the input factors then run beside the
+backward pass), when a factor that is still queued gets a second product, and when the
+collected work passes `flush_work()`; the engine calls take turns on the side streams, and
+calls in flight that touch the same buffer are ordered by an event.  `set_mode('eager')`
+runs every product in its hook, on the side streams, as described above.
 """
 import atexit
 import threading

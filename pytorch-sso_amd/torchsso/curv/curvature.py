@@ -12,8 +12,9 @@ mechanics, none in results:
   engine routine is launched once per step, not once per layer;
 * `ema` is updated in place and `inv` / `std` buffers are reused from step to
   step (the reference allocates new tensors each time);
-* the Kronecker factor products are enqueued on side streams (torchsso._lanes) and
-  joined by whoever reads factor data first;
+* the hooks queue the Kronecker factor products, and whoever reads factor data first has
+  them all run in one grouped engine call on a side stream (torchsso._lanes; in eager mode
+  every hook enqueues its own product on a side stream);
 * the output gradient is taken with a tensor hook on the module output instead
   of the deprecated module backward hook (same tensor, and it also works with
   an in-place activation after the module).
