@@ -15,12 +15,18 @@
 //   XCD (own L2) walks a contiguous run of (split, tile) pairs, tile fastest, as in
 //   the single-product kernel.
 //
+// The input factor of a convolution that is not pointwise reads a copy of its input:
+// zero-padded, one plane per row phase of the stride and per kernel column
+// (conv_planes_kernel, one launch for all such products of the call).  The operand then
+// needs no bounds test and reads consecutive addresses along the reduction.
+//
 // Products whose input exceeds the 1 GiB addressing window of an operand, and the
 // stride-1 k x k layers served by the correlation kernels, are handed to their
 // single-product routines on the same stream.
 #include <string.h>
 
 #include <algorithm>
+#include <type_traits>
 #include <vector>
 
 #include "common.h"
@@ -135,6 +141,60 @@ __global__ __launch_bounds__(256) void reduce_tile_grouped_kernel(const RdJob* _
                        tile, rem / CB, rem % CB);
 }
 
+// One convolution input and its copy in planes (see ConvP).  Only the row phases that
+// some kernel tap reads are written (a 1x1 convolution of stride 2 reads one of two).
+constexpr int MAX_PLANES = 32;
+constexpr int PLANE_ITEM = 8192;      // elements of the copy per workgroup
+struct PlaneJob {
+  const float* x;
+  float* out;
+  int C, H, W, sh, sw, ph, pw, dw, KW, Hs, OW, nused, chunks, ones, image;
+  FastDiv by_ow, by_area, by_chunks, by_c;
+  unsigned char used[MAX_PLANES];     // ry * KW + kw of the planes to write
+};
+
+// item = (channel image (n, c), chunk of its used planes): PLANE_ITEM elements, in order
+__global__ __launch_bounds__(256) void conv_planes_kernel(const PlaneJob* __restrict__ jobs,
+                                                          const int* __restrict__ cum, int njobs) {
+  const int j = find_job(cum, njobs, blockIdx.x);
+  const PlaneJob& jb = jobs[j];
+  const int local = blockIdx.x - cum[j];
+  const int img = jb.by_chunks.div(local);
+  const int chunk = local - img * jb.chunks;
+  const int n = jb.by_c.div(img), c = img - n * jb.C;
+  const int H = jb.H, W = jb.W, OW = jb.OW, area = jb.Hs * OW, planes = jb.sh * jb.KW;
+  const float* __restrict__ src = jb.x + (size_t)img * H * W;
+  float* __restrict__ dst = jb.out + (size_t)n * jb.image + (size_t)c * planes * area;
+  const int total = jb.nused * area;
+  const int e1 = min(total, (chunk + 1) * PLANE_ITEM);
+  // four elements per thread and trip, so that four loads are in flight
+  for (int e0 = chunk * PLANE_ITEM + threadIdx.x; e0 < e1; e0 += 4 * 256) {
+    float v[4];
+    int at[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int e = e0 + 256 * q;
+      const int u = jb.by_area.div(e);
+      const int idx = e - u * area;
+      const int plane = jb.used[u & (MAX_PLANES - 1)];
+      const int ry = plane / jb.KW, kw = plane - ry * jb.KW;
+      const int ys = jb.by_ow.div(idx);
+      const int ow = idx - ys * OW;
+      const int y = ys * jb.sh + ry - jb.ph, x = ow * jb.sw + kw * jb.dw - jb.pw;
+      const bool in = e < e1 && (unsigned)y < (unsigned)H && (unsigned)x < (unsigned)W;
+      at[q] = e < e1 ? plane * area + idx : -1;
+      v[q] = in ? src[y * W + x] : 0.f;
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      if (at[q] >= 0) dst[at[q]] = v[q];
+  }
+  if (jb.ones && c == 0 && chunk == 0) {
+    float* __restrict__ one = jb.out + (size_t)n * jb.image + (size_t)jb.C * planes * area;
+    for (int idx = threadIdx.x; idx < jb.ones; idx += 256) one[idx] = 1.f;
+  }
+}
+
 // ---- host side -----------------------------------------------------------------
 
 // Items of a grouped launch are dispatched longest first and the launch holds many of
@@ -179,17 +239,20 @@ static long launch_target(int w, double total_units) {
   return t;
 }
 
-enum Path { P_DENSE, P_CONVG, P_CONVA, P_TAPS, P_SINGLE, P_BAD };
+enum Path { P_DENSE, P_CONVG, P_CONVA, P_CONVP, P_TAPS, P_SINGLE, P_BAD };
+constexpr int SYRK_PATHS = 4;     // the first four: one launch each per tile size
 
 struct Classified {
   Path path;
   int d;
   long K;
   int OH, OW;
+  int Hs;                // P_CONVP: rows of a plane of the copy
+  size_t copy_bytes;     // P_CONVP: 0 when the input itself serves
 };
 
 static Classified classify(const kfac_factor_job& j) {
-  Classified c{P_BAD, 0, 0, 0, 0};
+  Classified c{P_BAD, 0, 0, 0, 0, 0, 0};
   if (j.rows <= 0 || j.c <= 0) return c;
   const int bias = j.add_bias ? 1 : 0;
   if (j.kind == KFAC_FACTOR_LINEAR) {
@@ -230,6 +293,19 @@ static Classified classify(const kfac_factor_job& j) {
     c.path = P_TAPS;
   } else {
     c.path = P_CONVA;
+    // the copy in planes, where it fits the addressing window of an operand
+    c.Hs = c.OH + (j.kh - 1) * j.dh / j.sh;
+    const int64_t copy =
+        j.rows * ((int64_t)j.c * j.sh * j.kw * c.Hs * c.OW + (bias ? c.OH * c.OW : 0)) * 4;
+    // (a pointwise convolution with a stride reads so little per product that the copy
+    // costs more than the bounds tests)
+    if (j.kh * j.kw > 1 && j.sh * j.kw <= MAX_PLANES && copy <= MAX_OPERAND_BYTES) {
+      c.path = P_CONVP;
+      // (a k x 1 kernel, stride 1, no padding, no bias: one plane, Hs = H, OW = W)
+      const bool as_is =
+          j.sh == 1 && j.sw == 1 && j.ph == 0 && j.pw == 0 && j.kw == 1 && !bias;
+      c.copy_bytes = as_is ? 0 : (size_t)copy;
+    }
   }
   return c;
 }
@@ -269,7 +345,10 @@ struct GroupedPlan {
   size_t table_bytes = 0, partial_floats = 0, single_bytes = 0;
   double executed_flops = 0.;
   // members of each launch, longest items first
-  std::vector<int> members[3][2];       // [P_DENSE | P_CONVG | P_CONVA][w - 1]
+  std::vector<int> members[SYRK_PATHS][2];   // [P_DENSE | P_CONVG | P_CONVA | P_CONVP][w - 1]
+  std::vector<size_t> copy_off;         // P_CONVP with a copy: bytes, from the copy area
+  std::vector<int> copies;              // the products that read a copy
+  size_t copy_bytes = 0;
   std::vector<int> reduce_many[2], reduce_tile[2];   // [w - 1]
   std::vector<int> singles;             // P_SINGLE, in call order
   std::vector<int> taps;                // P_TAPS, in call order
@@ -296,6 +375,7 @@ static GroupedPlan make_plan(int count, const kfac_factor_job* jobs) {
   gp.cls.resize(count);
   gp.plans.resize(count);
   gp.partial_off.assign(count, 0);
+  gp.copy_off.assign(count, 0);
   for (int i = 0; i < count; ++i) {
     const Classified c = classify(jobs[i]);
     gp.cls[i] = c;
@@ -320,8 +400,13 @@ static GroupedPlan make_plan(int count, const kfac_factor_job* jobs) {
     }
     const int w = c.d <= 256 ? 1 : 2;
     gp.members[c.path][w - 1].push_back(i);
+    if (c.path == P_CONVP && c.copy_bytes) {
+      gp.copies.push_back(i);
+      gp.copy_off[i] = gp.copy_bytes;
+      gp.copy_bytes += align_up(c.copy_bytes, 256);
+    }
   }
-  for (int path = 0; path < 3; ++path)
+  for (int path = 0; path < SYRK_PATHS; ++path)
     for (int w = 0; w < 2; ++w) {
       double units = 0.;
       for (int i : gp.members[path][w]) {
@@ -342,7 +427,7 @@ static GroupedPlan make_plan(int count, const kfac_factor_job* jobs) {
         gp.executed_flops += (double)p.ntiles * (double)((c.K + 15) / 16) * 16 * 2.0 * p.ts * p.ts;
       }
     }
-  for (int path = 0; path < 3; ++path)
+  for (int path = 0; path < SYRK_PATHS; ++path)
     for (int w = 0; w < 2; ++w) {
       auto& m = gp.members[path][w];
       std::stable_sort(m.begin(), m.end(),
@@ -352,9 +437,11 @@ static GroupedPlan make_plan(int count, const kfac_factor_job* jobs) {
     gp.table_bytes += table_size<SyJob<DenseKM>>(gp.members[P_DENSE][w].size());
     gp.table_bytes += table_size<SyJob<ConvG>>(gp.members[P_CONVG][w].size());
     gp.table_bytes += table_size<SyJob<ConvA>>(gp.members[P_CONVA][w].size());
+    gp.table_bytes += table_size<SyJob<ConvP>>(gp.members[P_CONVP][w].size());
     gp.table_bytes += table_size<RdJob>(gp.reduce_many[w].size());
     gp.table_bytes += table_size<RdJob>(gp.reduce_tile[w].size());
   }
+  gp.table_bytes += table_size<PlaneJob>(gp.copies.size());
   gp.table_bytes = align_up(gp.table_bytes, 256);
   if (!gp.taps.empty()) {
     const std::vector<TapsJob> tj = taps_jobs(gp, jobs);
@@ -413,7 +500,7 @@ static const GroupedPlan& cached_plan(int count, const kfac_factor_job* jobs) {
 
 static size_t plan_workspace(const GroupedPlan& gp) {
   return gp.table_bytes + align_up(gp.partial_floats * sizeof(float), 256) + gp.taps_bytes +
-         gp.single_bytes;
+         gp.single_bytes + gp.copy_bytes;
 }
 
 // host image of the device tables, filled section by section
@@ -446,6 +533,11 @@ ConvA make_op<ConvA>(const kfac_factor_job& j, const Classified& c) {
                j.add_bias ? 1 : 0);
 }
 
+template <>
+ConvP make_op<ConvP>(const kfac_factor_job& j, const Classified& c) {
+  return ConvP(j.x, j.c, j.kh, j.kw, j.sh, j.dh, c.Hs, c.OH, c.OW, c.d, j.add_bias ? 1 : 0);
+}
+
 struct Launch {
   size_t jobs_off, cum_off;
   int njobs, items;
@@ -453,7 +545,7 @@ struct Launch {
 
 template <class OP>
 static Launch fill_syrk(TableWriter& tw, const GroupedPlan& gp, const std::vector<int>& members,
-                        const kfac_factor_job* jobs, float* partials) {
+                        const kfac_factor_job* jobs, float* partials, const char* copies) {
   if (members.empty()) return Launch{0, 0, 0, 0};
   std::vector<SyJob<OP>> tab;
   std::vector<int> cum;
@@ -463,6 +555,9 @@ static Launch fill_syrk(TableWriter& tw, const GroupedPlan& gp, const std::vecto
     const kfac_factor_job& j = jobs[i];
     SyJob<OP> s;
     s.op = make_op<OP>(j, gp.cls[i]);
+    if constexpr (std::is_same<OP, ConvP>::value) {
+      if (gp.cls[i].copy_bytes) s.op.p = (const float*)(copies + gp.copy_off[i]);
+    }
     s.C = j.C;
     s.Cin = j.C_prev;
     s.ws = partials + gp.partial_off[i];
@@ -506,6 +601,52 @@ static Launch fill_reduce(TableWriter& tw, const GroupedPlan& gp, const std::vec
   l.jobs_off = tw.put(tab);
   l.cum_off = tw.put(cum);
   l.njobs = (int)members.size();
+  l.items = items;
+  return l;
+}
+
+// the copies in planes of all products that read one
+static Launch fill_planes(TableWriter& tw, const GroupedPlan& gp, const kfac_factor_job* jobs,
+                          char* copies) {
+  if (gp.copies.empty()) return Launch{0, 0, 0, 0};
+  std::vector<PlaneJob> tab;
+  std::vector<int> cum;
+  int items = 0;
+  for (int i : gp.copies) {
+    const kfac_factor_job& j = jobs[i];
+    const Classified& c = gp.cls[i];
+    PlaneJob pj;
+    memset(&pj, 0, sizeof(pj));
+    pj.x = j.x;
+    pj.out = (float*)(copies + gp.copy_off[i]);
+    pj.C = j.c;
+    pj.H = j.H; pj.W = j.W;
+    pj.sh = j.sh; pj.sw = j.sw;
+    pj.ph = j.ph; pj.pw = j.pw;
+    pj.dw = j.dw; pj.KW = j.kw;
+    pj.Hs = c.Hs; pj.OW = c.OW;
+    bool seen[MAX_PLANES] = {};
+    for (int kh = 0; kh < j.kh; ++kh) seen[kh * j.dh % j.sh] = true;
+    for (int ry = 0; ry < j.sh; ++ry)
+      for (int kw = 0; kw < j.kw && seen[ry]; ++kw)
+        pj.used[pj.nused++] = (unsigned char)(ry * j.kw + kw);
+    const int area = c.Hs * c.OW;
+    pj.chunks = cdiv(pj.nused * area, PLANE_ITEM);
+    pj.ones = j.add_bias ? c.OH * c.OW : 0;
+    pj.image = j.c * j.sh * j.kw * area + pj.ones;
+    pj.by_ow = FastDiv((unsigned)c.OW);
+    pj.by_area = FastDiv((unsigned)area);
+    pj.by_chunks = FastDiv((unsigned)pj.chunks);
+    pj.by_c = FastDiv((unsigned)j.c);
+    tab.push_back(pj);
+    cum.push_back(items);
+    items += (int)j.rows * j.c * pj.chunks;
+  }
+  cum.push_back(items);
+  Launch l;
+  l.jobs_off = tw.put(tab);
+  l.cum_off = tw.put(cum);
+  l.njobs = (int)gp.copies.size();
   l.items = items;
   return l;
 }
@@ -561,18 +702,25 @@ int kfac_factor_grouped(int count, const kfac_factor_job* jobs, void* workspace,
   float* partials = (float*)(table + gp.table_bytes);
   char* taps_ws = (char*)partials + align_up(gp.partial_floats * sizeof(float), 256);
   char* single_ws = taps_ws + gp.taps_bytes;
+  char* copies = single_ws + gp.single_bytes;
 
   TableWriter tw;
-  Launch sy[3][2], rm[2], rt[2];
+  Launch sy[SYRK_PATHS][2], rm[2], rt[2];
   for (int w = 0; w < 2; ++w) {
-    sy[P_DENSE][w] = fill_syrk<DenseKM>(tw, gp, gp.members[P_DENSE][w], jobs, partials);
-    sy[P_CONVG][w] = fill_syrk<ConvG>(tw, gp, gp.members[P_CONVG][w], jobs, partials);
-    sy[P_CONVA][w] = fill_syrk<ConvA>(tw, gp, gp.members[P_CONVA][w], jobs, partials);
+    sy[P_DENSE][w] = fill_syrk<DenseKM>(tw, gp, gp.members[P_DENSE][w], jobs, partials, copies);
+    sy[P_CONVG][w] = fill_syrk<ConvG>(tw, gp, gp.members[P_CONVG][w], jobs, partials, copies);
+    sy[P_CONVA][w] = fill_syrk<ConvA>(tw, gp, gp.members[P_CONVA][w], jobs, partials, copies);
+    sy[P_CONVP][w] = fill_syrk<ConvP>(tw, gp, gp.members[P_CONVP][w], jobs, partials, copies);
     rm[w] = fill_reduce(tw, gp, gp.reduce_many[w], jobs, partials, true);
     rt[w] = fill_reduce(tw, gp, gp.reduce_tile[w], jobs, partials, false);
   }
+  const Launch pl = fill_planes(tw, gp, jobs, copies);
   if (tw.words.size() * 4 > gp.table_bytes) return KFAC_ERR_LAUNCH;     // (cannot happen)
   upload_table(tw.words.data(), tw.words.size() * 4, table, stream);
+  if (pl.njobs)
+    hipLaunchKernelGGL(conv_planes_kernel, dim3(pl.items), dim3(256), 0, stream,
+                       (const PlaneJob*)(table + pl.jobs_off), (const int*)(table + pl.cum_off),
+                       pl.njobs);
   for (int i : gp.singles) {
     const int st = run_single(jobs[i], gp.single_bytes ? single_ws : nullptr, gp.single_bytes,
                               stream_);
@@ -584,9 +732,11 @@ int kfac_factor_grouped(int count, const kfac_factor_job* jobs, void* workspace,
     if (st != KFAC_OK) return st;
   }
   bool ok = true;
+  ok = ok && launch_syrk_group<ConvP, 2>(sy[P_CONVP][1], table, stream);
   ok = ok && launch_syrk_group<ConvA, 2>(sy[P_CONVA][1], table, stream);
   ok = ok && launch_syrk_group<ConvG, 2>(sy[P_CONVG][1], table, stream);
   ok = ok && launch_syrk_group<DenseKM, 2>(sy[P_DENSE][1], table, stream);
+  ok = ok && launch_syrk_group<ConvP, 1>(sy[P_CONVP][0], table, stream);
   ok = ok && launch_syrk_group<ConvA, 1>(sy[P_CONVA][0], table, stream);
   ok = ok && launch_syrk_group<ConvG, 1>(sy[P_CONVG][0], table, stream);
   ok = ok && launch_syrk_group<DenseKM, 1>(sy[P_DENSE][0], table, stream);
