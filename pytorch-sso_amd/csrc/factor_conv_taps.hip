@@ -86,21 +86,14 @@ struct TapPlanDev {
   short pair_jobs[MAX_PAIR_JOBS];
 };
 static_assert(sizeof(TapPlanDev) <= 3800, "plan must fit the kernel argument buffer");
-// work item `item` of one layer's plan -> (job, split, tile), and that tile's product
+// the product of one work item: tile `tile` of job j over its k-split `split`
 template <int W>
-__device__ __forceinline__ void corr_item(const float* x, int nimg, int C, int H, int Wd,
-                                          const TapPlanDev& plan, int tiles_side, float* ws,
-                                          int item, float* smem) {
+__device__ __forceinline__ void corr_product(const float* x, int nimg, int C, int H, int Wd,
+                                             const TapPlanDev& plan, int tiles_side, float* ws,
+                                             int j, int split, int tile, float* smem) {
   constexpr int TS = 64 * W;
   constexpr int KC = Cfg<W, W>::KC;
-  int j = -1;
-#pragma unroll
-  for (int q = 0; q < MAX_JOBS; ++q) j += plan.item0[q] <= item ? 1 : 0;
   const JobDesc jd = plan.jobs[j];
-  const int ntiles = tiles_side * tiles_side;
-  const int local = item - plan.item0[j];
-  const int split = local / ntiles;
-  const int tile = local - split * ntiles;
   const int bi = tile / tiles_side, bj = tile - bi * tiles_side;
   const int K = nimg * jd.hh * jd.ww;
   const int kbeg = split * jd.cps * KC;
@@ -117,12 +110,43 @@ __device__ __forceinline__ void corr_item(const float* x, int nimg, int C, int H
   gemm_tile_cfg<W, W>(P, Q, bi * TS, bj * TS, kbeg, kend, false, epi, smem);
 }
 
+// work item `item` of one layer's plan -> (job, split, tile), job by job
+template <int W>
+__device__ __forceinline__ void corr_item(const float* x, int nimg, int C, int H, int Wd,
+                                          const TapPlanDev& plan, int tiles_side, float* ws,
+                                          int item, float* smem) {
+  int j = -1;
+#pragma unroll
+  for (int q = 0; q < MAX_JOBS; ++q) j += plan.item0[q] <= item ? 1 : 0;
+  const int ntiles = tiles_side * tiles_side;
+  const int local = item - plan.item0[j];
+  const int split = local / ntiles;
+  corr_product<W>(x, nimg, C, H, Wd, plan, tiles_side, ws, j, split, local - split * ntiles, smem);
+}
+
 template <int W>
 __global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void corr_kernel(
     const float* x, int nimg, int C, int H, int Wd, const TapPlanDev plan, int tiles_side,
     float* ws) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   corr_item<W>(x, nimg, C, H, Wd, plan, tiles_side, ws, blockIdx.x, smem);
+}
+
+// The items of a layer in the order of a grouped launch, as a table of (job, k-split)
+// entries (tile fastest within an entry).  The jobs with many splits (the interior
+// products, one per displacement) come first, k-split by k-split: a run of consecutive
+// entries then reads one region of the input under all displacements, and
+// xcd_remap_range gives every XCD such a run, so that the region is fetched into one L2
+// once (job by job, the whole input streams through every L2 once per displacement).  The
+// short jobs (edge strips) follow job by job and are dealt round-robin: a launch of this
+// kind is resident all at once, a compute unit holds 5 or 6 of its items, and the units
+// with one more should get a short one.
+struct TapOrder {
+  int first;            // of this layer's entries in the table
+  int main_items;       // items (entries x tiles) that are remapped per XCD
+};
+__host__ __device__ __forceinline__ unsigned order_entry(int job, int split) {
+  return (unsigned)job | ((unsigned)split << 8);
 }
 
 // One layer of a grouped call: its tensors, and where its plan's partials and block sums live.
@@ -149,12 +173,20 @@ __device__ __forceinline__ int find_layer(const int* __restrict__ cum, int n, in
 template <int W>
 __global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void corr_grouped_kernel(
     const TapLayer* __restrict__ layers, const TapPlanDev* __restrict__ plans,
+    const TapOrder* __restrict__ order, const unsigned* __restrict__ entries,
     const int* __restrict__ index, const int* __restrict__ cum, int nlayers) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   const int k = find_layer(cum, nlayers, blockIdx.x);
   const int l = index[k];
   const TapLayer& L = layers[l];
-  corr_item<W>(L.x, L.n, L.C, L.H, L.W, plans[l], L.tiles_side, L.ws, blockIdx.x - cum[k], smem);
+  const TapOrder o = order[l];
+  int v = blockIdx.x - cum[k];
+  if (v < o.main_items) v = xcd_remap_range(blockIdx.x, cum[k], o.main_items);
+  const int ntiles = L.tiles_side * L.tiles_side;
+  const int e = v / ntiles;
+  const unsigned entry = entries[o.first + e];
+  corr_product<W>(L.x, L.n, L.C, L.H, L.W, plans[l], L.tiles_side, L.ws, (int)(entry & 255u),
+                  (int)(entry >> 8), v - e * ntiles, smem);
 }
 
 // B[pair][c][c'] = sum over the pair's jobs and their k-splits, in a fixed order.
@@ -550,16 +582,41 @@ struct TapsShape {
 struct TapsGroupPlan {
   std::vector<TapsShape> shapes;
   std::vector<TapPlanHost> plans;
+  std::vector<TapOrder> orders;
+  std::vector<unsigned> entries;
   std::vector<size_t> ws_off;          // floats, per layer, from the partial area
   std::vector<int> members[2];         // layers by tile size (w - 1), longest items first
   std::vector<int> cum_corr[2], cum_sum, cum_il;
-  size_t layers_off, plans_off, index_off[2], cum_corr_off[2], cum_sum_off, cum_il_off;
+  size_t layers_off, plans_off, orders_off, entries_off, index_off[2], cum_corr_off[2], cum_sum_off, cum_il_off;
   size_t table_bytes, partial_floats;
   double executed_flops;
   bool ok;
 };
 
 static size_t pad16(size_t v) { return (v + 15) / 16 * 16; }
+
+// appends the layer's entries to `entries`; the interior products are the jobs at least
+// half as long as the longest
+static TapOrder make_order(const TapPlanHost& hp, std::vector<unsigned>& entries) {
+  TapOrder o;
+  o.first = (int)entries.size();
+  const TapPlanDev& pd = hp.dev;
+  const int J = pd.njobs, ntiles = hp.tiles_side * hp.tiles_side;
+  long longest = 0;
+  for (int j = 0; j < J; ++j) longest = std::max(longest, (long)pd.jobs[j].splits * pd.jobs[j].cps);
+  auto interior = [&](int j) { return 2L * pd.jobs[j].splits * pd.jobs[j].cps >= longest; };
+  int smax = 0;
+  for (int j = 0; j < J; ++j)
+    if (interior(j)) smax = std::max(smax, (int)pd.jobs[j].splits);
+  for (int s = 0; s < smax; ++s)
+    for (int j = 0; j < J; ++j)
+      if (interior(j) && s < pd.jobs[j].splits) entries.push_back(order_entry(j, s));
+  o.main_items = ((int)entries.size() - o.first) * ntiles;
+  for (int j = 0; j < J; ++j)
+    if (!interior(j))
+      for (int s = 0; s < pd.jobs[j].splits; ++s) entries.push_back(order_entry(j, s));
+  return o;
+}
 
 // chunks per item of a grouped launch (one-wave 64-wide tiles / four-wave 128-wide tiles);
 // measured flat between 48 and 192
@@ -598,6 +655,7 @@ static TapsGroupPlan* make_taps_group_plan(int count, const TapsJob* jobs) {
       gp->ok = false;
       return gp;
     }
+    gp->orders.push_back(make_order(hp, gp->entries));
     gp->ws_off.push_back(gp->partial_floats);
     gp->partial_floats += (hp.partial_floats + 63) / 64 * 64;
     gp->members[hp.w - 1].push_back(i);
@@ -634,6 +692,10 @@ static TapsGroupPlan* make_taps_group_plan(int count, const TapsJob* jobs) {
   off += pad16((size_t)count * sizeof(TapLayer));
   gp->plans_off = off;
   off += pad16((size_t)count * sizeof(TapPlanDev));
+  gp->orders_off = off;
+  off += pad16((size_t)count * sizeof(TapOrder));
+  gp->entries_off = off;
+  off += pad16(gp->entries.size() * sizeof(unsigned));
   for (int w = 0; w < 2; ++w) {
     gp->index_off[w] = off;
     off += pad16(gp->members[w].size() * sizeof(int));
@@ -704,6 +766,8 @@ int conv_a_taps_grouped(int count, const TapsJob* jobs, void* workspace, size_t 
                          j.kh * j.kw, hp.tiles_side, j.alpha, j.beta};
     plans[i] = hp.dev;
   }
+  memcpy(img.data() + gp.orders_off, gp.orders.data(), (size_t)count * sizeof(TapOrder));
+  memcpy(img.data() + gp.entries_off, gp.entries.data(), gp.entries.size() * sizeof(unsigned));
   for (int w = 0; w < 2; ++w) {
     if (!gp.members[w].empty())
       memcpy(img.data() + gp.index_off[w], gp.members[w].data(), gp.members[w].size() * sizeof(int));
@@ -714,18 +778,20 @@ int conv_a_taps_grouped(int count, const TapsJob* jobs, void* workspace, size_t 
   upload_table(img.data(), img.size(), table, stream);
   const TapLayer* dl = (const TapLayer*)(table + gp.layers_off);
   const TapPlanDev* dp = (const TapPlanDev*)(table + gp.plans_off);
+  const TapOrder* dord = (const TapOrder*)(table + gp.orders_off);
+  const unsigned* dent = (const unsigned*)(table + gp.entries_off);
   if (!gp.members[1].empty()) {
     constexpr int lds = Cfg<2, 2>::SMEM_FLOATS * (int)sizeof(float);
     if (!enable_large_lds((const void*)corr_grouped_kernel<2>, lds)) return KFAC_ERR_LAUNCH;
     hipLaunchKernelGGL(corr_grouped_kernel<2>, dim3(gp.cum_corr[1].back()), dim3(256), lds, stream,
-                       dl, dp, (const int*)(table + gp.index_off[1]),
+                       dl, dp, dord, dent, (const int*)(table + gp.index_off[1]),
                        (const int*)(table + gp.cum_corr_off[1]), (int)gp.members[1].size());
   }
   if (!gp.members[0].empty()) {
     constexpr int lds = Cfg<1, 1>::SMEM_FLOATS * (int)sizeof(float);
     if (!enable_large_lds((const void*)corr_grouped_kernel<1>, lds)) return KFAC_ERR_LAUNCH;
     hipLaunchKernelGGL(corr_grouped_kernel<1>, dim3(gp.cum_corr[0].back()), dim3(64), lds, stream,
-                       dl, dp, (const int*)(table + gp.index_off[0]),
+                       dl, dp, dord, dent, (const int*)(table + gp.index_off[0]),
                        (const int*)(table + gp.cum_corr_off[0]), (int)gp.members[0].size());
   }
   hipLaunchKernelGGL(block_sum_grouped_kernel, dim3(gp.cum_sum.back()), dim3(256), 0, stream, dl, dp,

@@ -65,23 +65,6 @@ __device__ __forceinline__ int find_job(const int* __restrict__ cum, int njobs, 
   return lo;
 }
 
-// Workgroups go to the 8 XCDs round-robin by dispatch index g.  The n items of one
-// product occupy the dispatch indices [c0, c0 + n); this permutation of [0, n) gives
-// every XCD a contiguous run of them.
-__device__ __forceinline__ int xcd_remap_range(int g, int c0, int n) {
-  const int s = c0 & 7;
-  const int v = g - c0 + s;        // index in a virtual range that starts at a multiple of 8
-  const int x = v & 7;
-  const int tv = n + s;
-  int base = 0;
-#pragma unroll
-  for (int y = 0; y < 8; ++y) {
-    const int cnt = ((tv - y + 7) >> 3) - (y < s ? 1 : 0);
-    base += y < x ? cnt : 0;
-  }
-  return base + (v >> 3) - (x < s ? 1 : 0);
-}
-
 template <class OP, int W>
 __global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void syrk_grouped_kernel(
     const SyJob<OP>* __restrict__ jobs, const int* __restrict__ cum, int njobs) {

@@ -438,6 +438,24 @@ __device__ __forceinline__ int xcd_remap(int id, int total) {
   return base + (id >> 3);
 }
 
+// Workgroups go to the 8 XCDs round-robin by dispatch index g.  The n items of one
+// product occupy the dispatch indices [c0, c0 + n); this permutation of [0, n) gives
+// every XCD a contiguous run of them.
+__device__ __forceinline__ int xcd_remap_range(int g, int c0, int n) {
+  const int s = c0 & 7;
+  const int v = g - c0 + s;        // index in a virtual range that starts at a multiple of 8
+  const int x = v & 7;
+  const int tv = n + s;
+  int base = 0;
+#pragma unroll
+  for (int y = 0; y < 8; ++y) {
+    const int cnt = ((tv - y + 7) >> 3) - (y < s ? 1 : 0);
+    base += y < x ? cnt : 0;
+  }
+  return base + (v >> 3) - (x < s ? 1 : 0);
+}
+
+
 // Batched launches (one for many matrices or layers of different sizes) use a 1-D
 // grid of exactly the workgroups needed: cum[i] is the first work item of the i-th
 // listed matrix (table index first + i), cum[n] the grid size.  (A rectangular grid
