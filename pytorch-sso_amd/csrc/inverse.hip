@@ -737,35 +737,60 @@ __host__ __device__ inline int merge_tiles(int T, int depth) {
   return total;
 }
 
-// Tile `local` of the merges at `depth`.  Each XCD (own L2) takes a contiguous run of the
-// tiles, walked so that a run holds every reduction length in equal measure and
-// neighbouring tiles share an operand panel: the reduction of the first product grows
-// with the column of the tile, so its tiles go row by row (a row shares the U12 panel);
-// that of the second shrinks with the row, so its tiles go column by column (a column
-// shares the W panel); within a row / column the longest comes first.
+// Tile `local` of the merges at `depth`, longest reduction first: a launch lasts at least
+// as long as its longest tile (up to T/2 blocks on ONE compute unit, shared with two other
+// workgroups), so those start first and the launch ends on its one-block tiles.  The
+// reduction of the first product grows with the column of the tile (`fast` = column, the
+// tiles of a column share the Y22 panel), that of the second shrinks with the row (`fast`
+// = row, its tiles share the Y11 panel).  The halves of all segments of a depth differ by
+// at most one block, so rank r (0 = longest) holds one tile per `slow` index of every
+// segment, except the last rank, which only the longer segments have.
 __device__ __forceinline__ MergeTile merge_tile(const MatDesc& m, int depth, int local,
                                                 bool by_column) {
   MergeTile t;
   t.valid = false;
-  const int T = m.T;
-  const int total = merge_tiles(T, depth);
-  if (local >= total) return t;
-  int item = xcd_remap(local, total);
-  Segment sg = segment(0, depth, T);
-  for (int P = 0; item >= sg.tiles(); sg = segment(++P, depth, T)) item -= sg.tiles();
-  const int rows = sg.mid - sg.p0, cols = sg.p1 - sg.mid;
-  if (by_column) {
-    t.jt = item / rows;
-    t.it = item - t.jt * rows;
-  } else {
-    t.it = item / cols;
-    t.jt = cols - 1 - (item - t.it * cols);
+  const int T = m.T, nseg = 1 << depth;
+  int fmax = 0, s_all = 0, s_top = 0;
+  for (int P = 0; P < nseg; ++P) {
+    const Segment sg = segment(P, depth, T);
+    const int rows = sg.mid - sg.p0, cols = sg.p1 - sg.mid;
+    const int f = by_column ? rows : cols, sl = by_column ? cols : rows;
+    if (f == 0 || sl == 0) continue;
+    if (f > fmax) { fmax = f; s_top = 0; }
+    if (f == fmax) s_top += sl;
+    s_all += sl;
   }
-  t.X1 = sg.p0 * DB;
-  t.b1 = rows * DB;
-  t.X2 = sg.mid * DB;
-  t.b2 = min(cols * DB, m.n - t.X2);
-  t.valid = true;
+  if (fmax == 0) return t;
+  const int full = (fmax - 1) * s_all;
+  if (local >= full + s_top) return t;
+  int r, q;
+  if (local < full) {
+    r = local / s_all;
+    q = local - r * s_all;
+  } else {
+    r = fmax - 1;
+    q = local - full;
+  }
+  for (int P = 0; P < nseg; ++P) {
+    const Segment sg = segment(P, depth, T);
+    const int rows = sg.mid - sg.p0, cols = sg.p1 - sg.mid;
+    const int f = by_column ? rows : cols, sl = by_column ? cols : rows;
+    if (f == 0 || sl == 0 || f <= r) continue;
+    if (q >= sl) { q -= sl; continue; }
+    if (by_column) {
+      t.it = r;
+      t.jt = q;
+    } else {
+      t.it = q;
+      t.jt = f - 1 - r;
+    }
+    t.X1 = sg.p0 * DB;
+    t.b1 = rows * DB;
+    t.X2 = sg.mid * DB;
+    t.b2 = min(cols * DB, m.n - t.X2);
+    t.valid = true;
+    return t;
+  }
   return t;
 }
 
