@@ -120,8 +120,10 @@ typedef struct kfac_factor_job {
 } kfac_factor_job;
 
 /* Scratch for kfac_factor_grouped on this list (`jobs` is a HOST array): the device
- * tables of its launches, the k-split partials of all products at once, and the scratch
- * of the products that go through their single-product routine. */
+ * tables of its launches, the k-split partials of all products at once, the zero-padded
+ * copies of the inputs of strided / padded k x k convolutions (about 1.5 x such an input
+ * for a 3x3 kernel of stride 2), and the scratch of the products that go through their
+ * single-product routine. */
 size_t kfac_factor_grouped_workspace_bytes(int count, const kfac_factor_job* jobs);
 
 /* Every product of the list, C_i = alpha_i * P_i^T P_i + beta_i * C_prev_i, with the same
@@ -134,8 +136,9 @@ size_t kfac_factor_grouped_workspace_bytes(int count, const kfac_factor_job* job
  * layer by layer) and hands them over before the first reader of a factor: a launch per
  * layer drains and refills the chip a hundred times per step.  The outputs C_i must be
  * distinct buffers, and no C_i may be an input or C_prev of another product of the call.
- * Stride-1 k x k convolution inputs (the correlation kernels) and inputs above 1 GiB run
- * through their single-product routines on the same stream. */
+ * Stride-1 k x k convolution inputs go through the correlation kernels (all such layers
+ * of the call in one launch each); inputs above 1 GiB run through their single-product
+ * routines on the same stream. */
 int kfac_factor_grouped(int count, const kfac_factor_job* jobs, void* workspace,
                         size_t workspace_bytes, void* stream);
 
