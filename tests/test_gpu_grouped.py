@@ -44,10 +44,11 @@ CASES = [
     ('conv_a', (4, 48, 8, 8), ((1, 1), (1, 1), (0, 0), (1, 1)), False),     # pointwise: dense read
     ('conv_a', (3, 300, 7, 7), ((1, 1), (1, 1), (0, 0), (1, 1)), False),
     ('conv_a', (3, 20, 8, 8), ((1, 1), (2, 2), (0, 0), (1, 1)), False),     # pointwise with stride
-    ('conv_a', (3, 6, 13, 10), ((3, 2), (3, 2), (2, 1), (1, 1)), True),     # stride phases that differ per axis
-    ('conv_a', (2, 7, 12, 12), ((3, 3), (2, 2), (2, 2), (2, 2)), False),    # dilation = stride: one phase read
+    ('conv_a', (3, 6, 13, 10), ((3, 2), (3, 2), (2, 1), (1, 1)), True),     # strides that differ per axis
+    ('conv_a', (2, 7, 12, 12), ((3, 3), (2, 2), (2, 2), (2, 2)), False),    # dilation = stride: one row phase read
     ('conv_a', (2, 5, 15, 14), ((3, 3), (2, 3), (0, 1), (3, 2)), True),     # dilated and strided
-    ('conv_a', (3, 4, 17, 17), ((2, 2), (5, 5), (1, 1), (1, 1)), False),    # 25 stride phases: im2col with bounds tests
+    ('conv_a', (3, 4, 17, 17), ((2, 2), (5, 5), (1, 1), (1, 1)), False),    # stride larger than the kernel
+    ('conv_a', (3, 4, 17, 17), ((2, 7), (5, 1), (1, 3), (1, 1)), False),    # 35 planes: im2col with bounds tests instead
     ('conv_a', (4, 40, 10, 10), ((5, 5), (1, 1), (2, 2), (1, 1)), True),    # stride 1, padded copy, 128-wide tiles
     ('conv_a', (8, 64, 14, 14), ((3, 3), (1, 1), (1, 1), (1, 1)), False),   # correlation kernels
     ('conv_a', (4, 256, 14, 14), ((3, 3), (1, 1), (1, 1), (1, 1)), False),
