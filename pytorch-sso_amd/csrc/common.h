@@ -70,6 +70,14 @@ inline int piece_blocks(long work, int longest) {
   return pb >= longest ? 0 : (int)pb;
 }
 
+// Tiles' worth of MFMA work in the T(T+1)/2 upper tiles of a symmetric product with T tiles
+// per side: a diagonal tile leaves out its 32x32 blocks below the diagonal, 6 of 16 for a
+// 128-wide tile of four waves, 1 of 4 for a 64-wide tile of one.
+inline double syrk_tile_units(int T, int w) {
+  const double diag = w == 2 ? 10. / 16. : 3. / 4.;
+  return (double)T * (T - 1) / 2 + T * diag;
+}
+
 inline int launch_status() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? KFAC_OK : KFAC_ERR_LAUNCH;

@@ -143,10 +143,10 @@ __global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void syrk_kernel(OP op,
   if (kend > K) kend = K;
   if (splits == 1) {
     EpiStore epi{C, d, d, d, alpha, beta, bi != bj, Cin};
-    gemm_tile_cfg<W, W>(op, op, bi * TS, bj * TS, kbeg, kend, bi == bj, epi, smem);
+    gemm_tile_cfg<W, W, true>(op, op, bi * TS, bj * TS, kbeg, kend, bi == bj, epi, smem);
   } else {
     EpiPartial epi{ws + ((size_t)split * ntiles + tile) * (TS * TS), bi * TS, bj * TS, d, d, TS};
-    gemm_tile_cfg<W, W>(op, op, bi * TS, bj * TS, kbeg, kend, bi == bj, epi, smem);
+    gemm_tile_cfg<W, W, true>(op, op, bi * TS, bj * TS, kbeg, kend, bi == bj, epi, smem);
   }
 }
 
@@ -225,12 +225,13 @@ static int64_t slice_len(int64_t total, int64_t elems_per_unit) {
 }
 
 // MFMA flops one launch_syrk executes: every (tile, split) workgroup runs whole chunks of
-// KC reduction steps on a full ts x ts tile (padding and the k tail included).
+// KC reduction steps on a full ts x ts tile (padding and the k tail included); a diagonal
+// tile leaves out its 32x32 blocks below the diagonal.
 static double syrk_executed_flops(int d, int64_t K) {
   const SyrkPlan p = plan_syrk(d, (long)K);
   const int kc = p.w == 1 ? Cfg<1, 1>::KC : Cfg<2, 2>::KC;
   const double chunks = (double)((K + kc - 1) / kc);
-  return (double)p.ntiles * chunks * kc * 2.0 * p.ts * p.ts;
+  return syrk_tile_units(p.T, p.w) * chunks * kc * 2.0 * p.ts * p.ts;
 }
 
 double kfac_factor_executed_flops(int d, int64_t K) {

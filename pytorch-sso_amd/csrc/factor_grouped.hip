@@ -88,10 +88,10 @@ __global__ __launch_bounds__(64 * W * W, W == 2 ? 3 : 1) void syrk_grouped_kerne
   const OP op = jb.op;
   if (splits == 1) {
     EpiStore epi{jb.C, d, d, d, jb.alpha, jb.beta, bi != bj, jb.Cin};
-    gemm_tile_cfg<W, W>(op, op, bi * TS, bj * TS, kbeg, kend, bi == bj, epi, smem);
+    gemm_tile_cfg<W, W, true>(op, op, bi * TS, bj * TS, kbeg, kend, bi == bj, epi, smem);
   } else {
     EpiPartial epi{jb.ws + ((size_t)split * ntiles + tile) * (TS * TS), bi * TS, bj * TS, d, d, TS};
-    gemm_tile_cfg<W, W>(op, op, bi * TS, bj * TS, kbeg, kend, bi == bj, epi, smem);
+    gemm_tile_cfg<W, W, true>(op, op, bi * TS, bj * TS, kbeg, kend, bi == bj, epi, smem);
   }
 }
 
@@ -407,7 +407,8 @@ static GroupedPlan make_plan(int count, const kfac_factor_job* jobs) {
           gp.reduce_many[w].push_back(i);
         else if (p.splits > 1)
           gp.reduce_tile[w].push_back(i);
-        gp.executed_flops += (double)p.ntiles * (double)((c.K + 15) / 16) * 16 * 2.0 * p.ts * p.ts;
+        gp.executed_flops +=
+            syrk_tile_units(p.T, p.w) * (double)((c.K + 15) / 16) * 16 * 2.0 * p.ts * p.ts;
       }
     }
   for (int path = 0; path < SYRK_PATHS; ++path)

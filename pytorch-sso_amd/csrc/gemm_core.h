@@ -241,11 +241,40 @@ __device__ __forceinline__ void acc_coords(int m0, int n0, int a, int b, int i, 
   col = n0 + (wave % WN) * 64 + 32 * b + r;
 }
 
-template <int WM, int WN, class OPP, class OPQ, class EPI>
-__device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0, int n0,
-                                              int kbeg, int kend, bool same, EPI& epi,
-                                              float* smem) {
+// The MFMAs of k-steps [S0, S1) of a 16-deep slice.  A diagonal tile of a symmetric product
+// is symmetric itself: with SKIP its 32x32 blocks below the diagonal are not computed, and
+// the blocks above it are stored twice.  A wave's 64x64 quadrant then holds all four of its
+// blocks (quadrant above the diagonal), three (quadrant on it) or none (below it).  The
+// tile takes as long as before (one wave still has four blocks), but the matrix cores it
+// leaves alone serve the other workgroups of its compute unit; a launch with few
+// workgroups per unit has nothing to gain and only pays for the mirrored stores.
+enum { WAVE_FULL = 0, WAVE_DIAG = 1, WAVE_NONE = 2 };
+template <int S0, int S1, bool SKIP>
+__device__ __forceinline__ void mma_slice(const float (&fa)[2][8], const float (&fb)[2][8],
+                                          v16f (&acc)[2][2], int mode) {
+  if (!SKIP || mode == WAVE_FULL) {
+#pragma unroll
+    for (int s = S0; s < S1; ++s)
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a][s], fb[b][s], acc[a][b], 0, 0, 0);
+  } else if (mode == WAVE_DIAG) {
+#pragma unroll
+    for (int s = S0; s < S1; ++s) {
+      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[0][s], fb[0][s], acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[0][s], fb[1][s], acc[0][1], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[1][s], fb[1][s], acc[1][1], 0, 0, 0);
+    }
+  }
+}
+
+template <int WM, int WN, bool SAME, bool SKIP, class OPP, class OPQ, class EPI>
+__device__ __forceinline__ void gemm_tile_impl(const OPP& P, const OPQ& Q, int m0, int n0,
+                                               int kbeg, int kend, EPI& epi, float* smem) {
   typedef Cfg<WM, WN> C;
+  constexpr bool same = SAME;
   const int t = threadIdx.x & (C::NT - 1);
   const int lane = t & 63;
   const int wave = t >> 6;
@@ -253,6 +282,8 @@ __device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0
   const int h = lane >> 5;
   const int wm = (wave / WN) * 64;
   const int wn = (wave % WN) * 64;
+  static_assert(SAME || !SKIP, "only a diagonal tile of a symmetric product has blocks to skip");
+  const int mode = !SKIP ? WAVE_FULL : (wm < wn ? WAVE_FULL : (wm == wn ? WAVE_DIAG : WAVE_NONE));
 
   v16f acc[2][2];
 #pragma unroll
@@ -297,42 +328,31 @@ __device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0
 #pragma unroll
     for (int sl = 0; sl < KC / 16; ++sl) {
       float fa[2][8], fb[2][8];
-      load_frags<OPP::layout, C::TM, C::LDS_MK>(tpc, wm, r, h, 16 * sl, fa);
-      if (same)
-        load_frags<OPP::layout, C::TM, C::LDS_MK>(tpc, wn, r, h, 16 * sl, fb);
-      else
-        load_frags<OPQ::layout, C::TN, C::LDS_MK>(tqc, wn, r, h, 16 * sl, fb);
+      if (!SKIP || mode != WAVE_NONE) {
+        load_frags<OPP::layout, C::TM, C::LDS_MK>(tpc, wm, r, h, 16 * sl, fa);
+        if (same)
+          load_frags<OPP::layout, C::TM, C::LDS_MK>(tpc, wn, r, h, 16 * sl, fb);
+        else
+          load_frags<OPQ::layout, C::TN, C::LDS_MK>(tqc, wn, r, h, 16 * sl, fb);
+      }
       if (sl == KC / 16 - 1) {
-#pragma unroll
-        for (int s = 0; s < 4; ++s)
-#pragma unroll
-          for (int a = 0; a < 2; ++a)
-#pragma unroll
-            for (int b = 0; b < 2; ++b)
-              acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a][s], fb[b][s], acc[a][b], 0, 0, 0);
+        mma_slice<0, 4, SKIP>(fa, fb, acc, mode);
         if (more) {
           sp.commit(tpn);
           if (!same) sq.commit(tpn + C::P_FLOATS);
         }
-#pragma unroll
-        for (int s = 4; s < 8; ++s)
-#pragma unroll
-          for (int a = 0; a < 2; ++a)
-#pragma unroll
-            for (int b = 0; b < 2; ++b)
-              acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a][s], fb[b][s], acc[a][b], 0, 0, 0);
+        mma_slice<4, 8, SKIP>(fa, fb, acc, mode);
       } else {
-#pragma unroll
-        for (int s = 0; s < 8; ++s)
-#pragma unroll
-          for (int a = 0; a < 2; ++a)
-#pragma unroll
-            for (int b = 0; b < 2; ++b)
-              acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a][s], fb[b][s], acc[a][b], 0, 0, 0);
+        mma_slice<0, 8, SKIP>(fa, fb, acc, mode);
       }
     }
     __syncthreads();
   }
+
+  // A diagonal tile of a symmetric product: the blocks above the tile's diagonal are
+  // stored at their mirror position too, the blocks below it were not computed.
+  auto computed = [&](int a, int b) { return !SKIP || (wm + 32 * a <= wn + 32 * b); };
+  auto mirrored = [&](int a, int b) { return SKIP && (wm + 32 * a < wn + 32 * b); };
 
   if constexpr (reading_epilogue<EPI>::value) {
     // C = alpha*acc + beta*C_old: the old values are loaded 32 at a time ahead of the
@@ -348,7 +368,7 @@ __device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0
           for (int i = 0; i < 16; ++i) {
             int row, col;
             acc_coords<WM, WN>(m0, n0, a, b, i, row, col);
-            old[b * 16 + i] = epi.fetch(row, col);
+            old[b * 16 + i] = computed(a, b) ? epi.fetch(row, col) : 0.f;
           }
 #pragma unroll
         for (int b = 0; b < 2; ++b)
@@ -356,7 +376,9 @@ __device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0
           for (int i = 0; i < 16; ++i) {
             int row, col;
             acc_coords<WM, WN>(m0, n0, a, b, i, row, col);
-            epi.store_with(row, col, acc[a][b][i], old[b * 16 + i]);
+            if (computed(a, b)) epi.store_with(row, col, acc[a][b][i], old[b * 16 + i]);
+            // (the old values are symmetric like the new ones)
+            if (mirrored(a, b)) epi.store_with(col, row, acc[a][b][i], old[b * 16 + i]);
           }
       }
       return;
@@ -370,11 +392,29 @@ __device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0
       for (int i = 0; i < 16; ++i) {
         int row, col;
         acc_coords<WM, WN>(m0, n0, a, b, i, row, col);
-        if constexpr (indexed_epilogue<EPI>::value)
+        if constexpr (indexed_epilogue<EPI>::value) {
+          static_assert(!SKIP, "indexed epilogues do not take skipped blocks");
           epi.store_at((a * 2 + b) * 16 + i, acc[a][b][i]);     // index known at compile time
-        else
-          epi.store(row, col, acc[a][b][i]);
+        } else {
+          if (computed(a, b)) epi.store(row, col, acc[a][b][i]);
+          if (mirrored(a, b)) epi.store(col, row, acc[a][b][i]);
+        }
       }
+}
+
+// SKIP_LOWER: a diagonal tile (`same`) leaves out its blocks below the diagonal.
+template <int WM, int WN, bool SKIP_LOWER = false, class OPP, class OPQ, class EPI>
+__device__ __forceinline__ void gemm_tile_cfg(const OPP& P, const OPQ& Q, int m0, int n0,
+                                              int kbeg, int kend, bool same, EPI& epi,
+                                              float* smem) {
+  if constexpr (std::is_same<OPP, OPQ>::value) {
+    if (same) {
+      gemm_tile_impl<WM, WN, true, SKIP_LOWER && !indexed_epilogue<EPI>::value>(
+          P, Q, m0, n0, kbeg, kend, epi, smem);
+      return;
+    }
+  }
+  gemm_tile_impl<WM, WN, false, false>(P, Q, m0, n0, kbeg, kend, epi, smem);
 }
 
 // default configuration: 128x128 tile, 256 threads
