@@ -50,6 +50,11 @@ CASES = [
     ('conv_a', (3, 4, 17, 17), ((2, 2), (5, 5), (1, 1), (1, 1)), False),    # stride larger than the kernel
     ('conv_a', (3, 4, 17, 17), ((2, 7), (5, 1), (1, 3), (1, 1)), False),    # 35 planes: im2col with bounds tests instead
     ('conv_a', (4, 40, 10, 10), ((5, 5), (1, 1), (2, 2), (1, 1)), True),    # stride 1, padded copy, 128-wide tiles
+    ('conv_a', (1, 1, 5, 5), ((3, 3), (2, 2), (1, 1), (1, 1)), True),       # one sample, one channel
+    ('conv_a', (2, 3, 4, 9), ((4, 3), (1, 3), (0, 0), (1, 1)), False),      # one output row
+    ('conv_a', (3, 2, 8, 3), ((2, 3), (2, 2), (0, 0), (1, 1)), True),       # one output column
+    ('conv_a', (2, 2, 3, 3), ((5, 5), (1, 1), (2, 2), (1, 1)), True),       # kernel larger than the image
+    ('conv_a', (5, 8, 6, 1), ((3, 1), (2, 1), (1, 0), (1, 1)), False),      # images one pixel wide
     ('conv_a', (8, 64, 14, 14), ((3, 3), (1, 1), (1, 1), (1, 1)), False),   # correlation kernels
     ('conv_a', (4, 256, 14, 14), ((3, 3), (1, 1), (1, 1), (1, 1)), False),
     ('conv_g', (16, 64, 56, 56), None, False),      # one 64-wide tile, very long reduction
