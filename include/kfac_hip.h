@@ -56,7 +56,9 @@ size_t kfac_factor_workspace_bytes(int d, int64_t K);
  * bias) and :61-67 with the n^2 rescale of curvature.py:154-155,299-300
  * (G, alpha = n, add_bias = 0).  beta != 0 fuses the accumulation of
  * utils/accumulator.py:23-38 or the running average of curvature.py:185-186
- * into the GEMM epilogue; with beta == 0, neither C nor C_prev is read. */
+ * into the GEMM epilogue; with beta == 0, neither C nor C_prev is read.  C_prev is
+ * taken to be symmetric (what these routines write is, to the bit): only its
+ * upper triangle is read, and C is written symmetric. */
 int kfac_factor_linear(const float* x, int64_t rows, int f, int64_t ldx, int add_bias,
                        float alpha, float beta, const float* C_prev, float* C,
                        void* workspace, size_t workspace_bytes, void* stream);
