@@ -243,12 +243,14 @@ __device__ __forceinline__ void acc_coords(int m0, int n0, int a, int b, int i, 
 
 // The MFMAs of k-steps [S0, S1) of a 16-deep slice.  A diagonal tile of a symmetric product
 // is symmetric itself: with SKIP its 32x32 blocks below the diagonal are not computed, and
-// the blocks above it are stored twice.  A wave's 64x64 quadrant then holds all four of its
-// blocks (quadrant above the diagonal), three (quadrant on it) or none (below it).  The
-// tile takes as long as before (one wave still has four blocks), but the matrix cores it
-// leaves alone serve the other workgroups of its compute unit; a launch with few
-// workgroups per unit has nothing to gain and only pays for the mirrored stores.
-enum { WAVE_FULL = 0, WAVE_DIAG = 1, WAVE_NONE = 2 };
+// the blocks above it are stored twice.  The 10 blocks of a 128-wide tile are dealt 3, 2, 2, 3
+// over its four waves: the waves on the diagonal quadrants take the three blocks of theirs,
+// and the quadrant above the diagonal is shared by the wave that owns it (upper two blocks)
+// and the wave of the quadrant below the diagonal (lower two), so the tile is done in three
+// quarters of the time.  The single wave of a 64-wide tile takes its three blocks.  The
+// matrix cores this leaves alone serve the other workgroups of the compute unit; a launch
+// with few workgroups per unit has little to gain and pays for the mirrored stores.
+enum { WAVE_FULL = 0, WAVE_DIAG = 1, WAVE_ROW0 = 2, WAVE_ROW1 = 3 };
 template <int S0, int S1, bool SKIP>
 __device__ __forceinline__ void mma_slice(const float (&fa)[2][8], const float (&fb)[2][8],
                                           v16f (&acc)[2][2], int mode) {
@@ -267,7 +269,28 @@ __device__ __forceinline__ void mma_slice(const float (&fa)[2][8], const float (
       acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[0][s], fb[1][s], acc[0][1], 0, 0, 0);
       acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[1][s], fb[1][s], acc[1][1], 0, 0, 0);
     }
+  } else if (mode == WAVE_ROW0) {
+#pragma unroll
+    for (int s = S0; s < S1; ++s) {
+      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[0][s], fb[0][s], acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[0][s], fb[1][s], acc[0][1], 0, 0, 0);
+    }
+  } else {
+#pragma unroll
+    for (int s = S0; s < S1; ++s) {
+      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[1][s], fb[0][s], acc[1][0], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[1][s], fb[1][s], acc[1][1], 0, 0, 0);
+    }
   }
+}
+
+// acc_coords for a wave whose quadrant starts at (wm, wn) of the tile
+__device__ __forceinline__ void quad_coords(int m0, int n0, int wm, int wn, int a, int b, int i,
+                                            int& row, int& col) {
+  const int lane = threadIdx.x & 63;
+  const int r = lane & 31, h = lane >> 5;
+  row = m0 + wm + 32 * a + 8 * (i >> 2) + 4 * h + (i & 3);
+  col = n0 + wn + 32 * b + r;
 }
 
 template <int WM, int WN, bool SAME, bool SKIP, class OPP, class OPQ, class EPI>
@@ -280,10 +303,22 @@ __device__ __forceinline__ void gemm_tile_impl(const OPP& P, const OPQ& Q, int m
   const int wave = t >> 6;
   const int r = lane & 31;
   const int h = lane >> 5;
-  const int wm = (wave / WN) * 64;
-  const int wn = (wave % WN) * 64;
+  int wm = (wave / WN) * 64;
+  int wn = (wave % WN) * 64;
   static_assert(SAME || !SKIP, "only a diagonal tile of a symmetric product has blocks to skip");
-  const int mode = !SKIP ? WAVE_FULL : (wm < wn ? WAVE_FULL : (wm == wn ? WAVE_DIAG : WAVE_NONE));
+  static_assert(!SKIP || (WM == WN && WM <= 2), "skipping is written for 64- and 128-wide tiles");
+  int mode = WAVE_FULL;
+  if (SKIP) {
+    if (wm == wn) {
+      mode = WAVE_DIAG;
+    } else if (wm < wn) {
+      mode = WAVE_ROW0;
+    } else {             // the quadrant below the diagonal: the lower half of the one above
+      mode = WAVE_ROW1;
+      wm = 0;
+      wn = 64;
+    }
+  }
 
   v16f acc[2][2];
 #pragma unroll
@@ -328,7 +363,7 @@ __device__ __forceinline__ void gemm_tile_impl(const OPP& P, const OPQ& Q, int m
 #pragma unroll
     for (int sl = 0; sl < KC / 16; ++sl) {
       float fa[2][8], fb[2][8];
-      if (!SKIP || mode != WAVE_NONE) {
+      {
         load_frags<OPP::layout, C::TM, C::LDS_MK>(tpc, wm, r, h, 16 * sl, fa);
         if (same)
           load_frags<OPP::layout, C::TM, C::LDS_MK>(tpc, wn, r, h, 16 * sl, fb);
@@ -351,8 +386,10 @@ __device__ __forceinline__ void gemm_tile_impl(const OPP& P, const OPQ& Q, int m
 
   // A diagonal tile of a symmetric product: the blocks above the tile's diagonal are
   // stored at their mirror position too, the blocks below it were not computed.
-  auto computed = [&](int a, int b) { return !SKIP || (wm + 32 * a <= wn + 32 * b); };
-  auto mirrored = [&](int a, int b) { return SKIP && (wm + 32 * a < wn + 32 * b); };
+  auto computed = [&](int a, int b) {
+    return !SKIP || (mode == WAVE_DIAG ? a <= b : a == (mode == WAVE_ROW0 ? 0 : 1));
+  };
+  auto mirrored = [&](int a, int b) { return SKIP && computed(a, b) && (wm + 32 * a < wn + 32 * b); };
 
   if constexpr (reading_epilogue<EPI>::value) {
     // C = alpha*acc + beta*C_old: the old values are loaded 32 at a time ahead of the
@@ -367,7 +404,7 @@ __device__ __forceinline__ void gemm_tile_impl(const OPP& P, const OPQ& Q, int m
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
             int row, col;
-            acc_coords<WM, WN>(m0, n0, a, b, i, row, col);
+            quad_coords(m0, n0, wm, wn, a, b, i, row, col);
             old[b * 16 + i] = computed(a, b) ? epi.fetch(row, col) : 0.f;
           }
 #pragma unroll
@@ -375,7 +412,7 @@ __device__ __forceinline__ void gemm_tile_impl(const OPP& P, const OPQ& Q, int m
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
             int row, col;
-            acc_coords<WM, WN>(m0, n0, a, b, i, row, col);
+            quad_coords(m0, n0, wm, wn, a, b, i, row, col);
             if (computed(a, b)) epi.store_with(row, col, acc[a][b][i], old[b * 16 + i]);
             // (the old values are symmetric like the new ones)
             if (mirrored(a, b)) epi.store_with(col, row, acc[a][b][i], old[b * 16 + i]);
@@ -391,7 +428,7 @@ __device__ __forceinline__ void gemm_tile_impl(const OPP& P, const OPQ& Q, int m
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         int row, col;
-        acc_coords<WM, WN>(m0, n0, a, b, i, row, col);
+        quad_coords(m0, n0, wm, wn, a, b, i, row, col);
         if constexpr (indexed_epilogue<EPI>::value) {
           static_assert(!SKIP, "indexed epilogues do not take skipped blocks");
           epi.store_at((a * 2 + b) * 16 + i, acc[a][b][i]);     // index known at compile time
