@@ -121,139 +121,10 @@ __global__ __launch_bounds__(256) void inv_copy_damp_kernel(const MatDesc* table
 // ---------------------------------------------------------------------------
 constexpr int DB = 128;          // diagonal block size
 constexpr int DLD = DB + 1;      // LDS leading dimension
-constexpr int WLD = 65;
-constexpr int DIAG_SMEM_BYTES = (2 * DB * DLD + 64 * WLD) * (int)sizeof(float);
+constexpr int DIAG_SMEM_BYTES = 2 * DB * DLD * (int)sizeof(float);
 
-// One wave runs the 32 elimination steps of the 32-row strip at row c0 of S on two
-// column blocks at once: lanes 0-31 hold the columns of the diagonal leaf
-// (c0 .. c0+31), lanes 32-63 the columns pcol .. pcol+31 of the same rows (a
-// block of the row panel to the right; pcol < 0: none, the lanes shadow the leaf).
-// Lane j keeps its column in registers.  Each step needs row c of the leaf in every
-// lane: the leaf lanes write their element to a 64-float LDS buffer private to
-// the wave and all lanes read the row back with broadcast ds_read_b128.  The steps
-// are software-pipelined: step c first finishes element c+1 of the column, publishes
-// it (two buffers alternate) and issues the reads of row c+1, and only then applies
-// row c to the rest of the column, so the LDS round trip of the next row runs under
-// those FMAs (scheduling barriers keep the compiler from moving them in front of the
-// store); the pivot itself comes through v_readlane and does not wait for LDS.
-// The panel columns see the same eliminations as the leaf columns, so the strip ends
-// up holding U[q][*] without a triangular solve.  Several waves may run this on the
-// same leaf with different panel blocks (the leaf is then factored redundantly; only
-// `owner` writes it out, as a dense 32x32 copy `ubuf`, which the caller copies over
-// the leaf in S once all waves are past reading it, and which feeds the back
-// substitution).
 __device__ __forceinline__ float lane_value(float v, int src_lane) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src_lane));
-}
-
-__device__ __forceinline__ void read_row(const lds_f* rowbuf, int first, float (&row)[32]) {
-#pragma unroll
-  for (int g = first / 4; g < 8; ++g) {
-    const v4f v = *(const lds_f4*)(rowbuf + 4 * g);
-    row[4 * g + 0] = v.x;
-    row[4 * g + 1] = v.y;
-    row[4 * g + 2] = v.z;
-    row[4 * g + 3] = v.w;
-  }
-}
-
-__device__ __forceinline__ void chol_strip_32(lds_f* S, lds_f* rowbuf, lds_f* ubuf, int c0,
-                                              int pcol, bool owner, int row_base, int* info) {
-  const int lane = threadIdx.x & 63;
-  const int j = lane & 31;
-  const bool leaf = lane < 32;
-  const int col = (leaf || pcol < 0) ? c0 + j : pcol + j;
-  float a[32];
-#pragma unroll
-  for (int i = 0; i < 32; ++i) a[i] = S[(c0 + i) * DLD + col];
-  int bad = 0;
-  // A[c][c0 + j] after the updates of the earlier steps; the panel lanes write into
-  // the unused second half of the buffer, so that the store is unconditional
-  float row[32];
-  rowbuf[lane] = a[0];
-  __builtin_amdgcn_wave_barrier();
-  read_row(rowbuf, 0, row);
-  float piv = lane_value(a[0], 0);
-  // 1/sqrt in one instruction: the next step's pivot waits on this chain
-  float rd = __builtin_amdgcn_rsqf(piv);
-  float f = a[0] * (rd * rd);
-#pragma unroll
-  for (int c = 0; c < 32; ++c) {
-    if (!(piv > 0.f) && bad == 0) bad = row_base + c0 + c + 1;
-    float next[32];
-    float pivn = 0.f, rdn = 0.f, fn = 0.f;
-    if (c + 1 < 32) {
-      // the chain from step to step: element c+1, its store, the reads of row c+1
-      a[c + 1] = fmaf(-row[c + 1], f, a[c + 1]);
-      lds_f* const nb = rowbuf + 64 * ((c + 1) & 1);
-      nb[lane] = a[c + 1];
-      __builtin_amdgcn_wave_barrier();
-      read_row(nb, c + 1, next);
-      // nothing may be scheduled in front of that store: the rest of this step is
-      // what runs while the row travels through LDS
-      __builtin_amdgcn_sched_barrier(0);
-      pivn = lane_value(a[c + 1], c + 1);
-      rdn = __builtin_amdgcn_rsqf(pivn);
-      fn = a[c + 1] * (rdn * rdn);
-    }
-#pragma unroll
-    for (int i = c + 2; i < 32; ++i) a[i] = fmaf(-row[i], f, a[i]);   // A[i][col] -= U[c][i] U[c][col]
-    const float u = a[c] * rd;
-    a[c] = leaf ? (j > c ? u : (j == c ? piv * rd : 0.f)) : u;
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = c + 1; i < 32; ++i) row[i] = next[i];
-    piv = pivn;
-    rd = rdn;
-    f = fn;
-  }
-  if (owner && bad != 0 && lane == 0) {
-    if (*info == 0) *info = bad;
-  }
-  if (leaf) {
-    if (owner) {
-#pragma unroll
-      for (int i = 0; i < 32; ++i) ubuf[i * 32 + j] = (i <= j) ? a[i] : 0.f;
-    }
-  } else if (pcol >= 0) {
-#pragma unroll
-    for (int i = 0; i < 32; ++i) S[(c0 + i) * DLD + pcol + j] = a[i];
-  }
-}
-
-// One wave: Y = U^-1 of the 32x32 upper-triangular leaf in ubuf (dense, row-major),
-// written to Yb at (c0, c0).  Column j of Y in lane j, row i of U broadcast.
-__device__ __forceinline__ void backsub_32(const lds_f* ubuf, lds_f* Yb, int c0) {
-  const int lane = threadIdx.x & 63;
-  const int j = lane & 31;
-  float y[32];
-#pragma unroll
-  for (int i = 31; i >= 0; --i) {
-    float row[32];
-#pragma unroll
-    for (int g = i / 4; g < 8; ++g) {
-      const v4f v = *(const lds_f4*)(ubuf + i * 32 + 4 * g);
-      row[4 * g + 0] = v.x;
-      row[4 * g + 1] = v.y;
-      row[4 * g + 2] = v.z;
-      row[4 * g + 3] = v.w;
-    }
-    // y[i+1] was finished last: it enters the sum last, so that only one FMA and
-    // one multiply separate consecutive rows; two partial sums shorten the rest
-    float s0 = (j == i) ? 1.f : 0.f, s1 = 0.f;
-#pragma unroll
-    for (int k = 31; k > i + 1; k -= 2) {
-      s0 = fmaf(-row[k], y[k], s0);
-      if (k - 1 > i + 1) s1 = fmaf(-row[k - 1], y[k - 1], s1);
-    }
-    float s = s0 + s1;
-    if (i + 1 < 32) s = fmaf(-row[i + 1], y[i + 1], s);
-    y[i] = s * __builtin_amdgcn_rcpf(row[i]);
-  }
-  if (lane < 32) {
-#pragma unroll
-    for (int i = 0; i < 32; ++i) Yb[(c0 + i) * DLD + c0 + j] = (i <= j) ? y[i] : 0.f;
-  }
 }
 
 // One wave: acc(32x32) = sum_{k<K} A(k, i) * B(k, j) with operands in LDS,
@@ -283,165 +154,258 @@ __device__ __forceinline__ v16f lds_mma32(const lds_f* a, int a_ks, int a_is, co
   return acc;
 }
 
-// store / subtract a 32x32 result block at c[row*ld + col]
-__device__ __forceinline__ void lds_put32(lds_f* c, int ld, const v16f& acc, float scale) {
-  const int lane = threadIdx.x & 63;
-  const int r = lane & 31, h = lane >> 5;
-#pragma unroll
-  for (int t = 0; t < 16; ++t) c[(8 * (t >> 2) + 4 * h + (t & 3)) * ld + r] = scale * acc[t];
-}
-__device__ __forceinline__ void lds_sub32(lds_f* c, int ld, const v16f& acc) {
-  const int lane = threadIdx.x & 63;
-  const int r = lane & 31, h = lane >> 5;
-#pragma unroll
-  for (int t = 0; t < 16; ++t) c[(8 * (t >> 2) + 4 * h + (t & 3)) * ld + r] -= acc[t];
-}
-
-// In-LDS off-diagonal inverse block:  Y12 = -Y11 * (U12 * Y22) for the pair
-// X1 = [s1, s1+b), X2 = [s1+b, s1+2b), b = 32 or 64; W is a b x b scratch.
-// 32x32 result blocks are dealt round-robin to the 4 waves.
-__device__ __forceinline__ void tri_pair(const lds_f* S, lds_f* Yb, lds_f* Wt, int s1, int b,
-                                         int wave_first, int wave_count) {
-  const int s2 = s1 + b;
-  const int wave = (int)(threadIdx.x >> 6) - wave_first;
-  const int nb = b / 32;
-  // W[i][j] = sum_k U12[i][k] * Y22[k][j]     (Y22 is zero below its diagonal)
-  for (int blk = wave; blk < nb * nb && wave >= 0; blk += wave_count) {
-    const int bi = blk / nb, bj = blk - bi * nb;
-    const v16f acc = lds_mma32(S + (s1 + 32 * bi) * DLD + s2, 1, DLD,
-                               Yb + s2 * DLD + s2 + 32 * bj, DLD, 1, 32 * (bj + 1));
-    lds_put32(Wt + 32 * bi * WLD + 32 * bj, WLD, acc, 1.f);
-  }
-  __syncthreads();
-  // Y12[i][j] = - sum_{k} Y11[i][k] * W[k][j]  (Y11 is zero below its diagonal)
-  for (int blk = wave; blk < nb * nb && wave >= 0; blk += wave_count) {
-    const int bi = blk / nb, bj = blk - bi * nb;
-    const v16f acc = lds_mma32(Yb + (s1 + 32 * bi) * DLD + s1 + 32 * bi, 1, DLD,
-                               Wt + 32 * bi * WLD + 32 * bj, WLD, 1, b - 32 * bi);
-    lds_put32(Yb + (s1 + 32 * bi) * DLD + s2 + 32 * bj, DLD, acc, -1.f);
-  }
-  __syncthreads();
+// The elimination of a 32-row strip, two rows per step, on 32x32 blocks that live in the
+// accumulator registers of v_mfma_f32_32x32x2_f32: element t of lane (r = lane & 31,
+// h = lane >> 5) is (row 8*(t/4) + 4*h + t%4, column r), so row c of a block is ONE register
+// (index 4*(c/8) + c%4) in the 32 lanes of half (c/4)%2, lane = column, and rows c, c+1
+// (c even) are neighbouring registers in the same half.
+//   L: the diagonal leaf, a full symmetric 32x32 block (Schur complement of the rows above);
+//   P: the same rows of another 32 columns (a block of the row panel, or of [ . | identity]).
+// A step finishes rows c and c+1:  with the 2x2 pivot block [p00 p01; p01 p11] of L,
+//   w0 = L[c] / sqrt(p00),  u01 = p01 / sqrt(p00),  w1 = (L[c+1] - u01 w0) / sqrt(p11 - u01^2)
+// are rows c, c+1 of U (the same combination y0, y1 of P's rows: those rows of the second
+// block), and the rows below get  X[i][j] -= w0[i] y0[j] + w1[i] y1[j]  as ONE rank-2 matrix
+// instruction per block: its reduction slot 0 is the lanes 0-31 of the operand registers,
+// slot 1 the lanes 32-63, so (w0 | w1) in the two halves of one register is the B operand
+// (lane = column j) and, negated and zeroed in the lanes i <= c+1, the A operand (lane = row
+// i; by the symmetry of L its rows are its columns).  Both rows live in one half, so one
+// v_permlane32_swap moves the second into the other half; apart from that and the three
+// pivot entries (v_readlane) no value changes lanes.  The chain from step to step is
+//   matrix instruction -> pivots -> two 1/sqrt -> w1 -> swap -> matrix instruction.
+// The finished rows go to LDS as they are made (`leaf_out`: where U_qq goes, `dummy` for a
+// wave that only needs the multipliers; `blk_out`: the second block's rows; `dummy`: a
+// 32x32 block of LDS that nothing reads).
+// With P = rows of the panel the strip ends as U[q][*] = U_qq^-T A[q][*] without a
+// triangular solve; with P = [pending | identity] as the rows of U^-T.
+// `bad`: 1-based row of the first non-positive pivot (row1 = that of the strip's first row).
+template <int H>
+__device__ __forceinline__ float pair_operand(float x0, float x1) {
+  // both valid in the lanes of half H -> x0 in lanes 0-31, x1 in lanes 32-63
+  // (the instruction swaps lanes 32-63 of its first register with lanes 0-31 of its second)
+  const auto sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x0),
+                                                   __builtin_bit_cast(unsigned, x1), false, false);
+  return __builtin_bit_cast(float, H ? sw[1] : sw[0]);
 }
 
-// Factors and inverts diagonal block p of matrix m (one workgroup of 256 threads with
-// DIAG_SMEM_BYTES of LDS at dsm).
+template <int C>
+__device__ __forceinline__ void elim_pair(v16f& L, v16f& P, lds_f* leaf_out, lds_f* blk_out,
+                                          lds_f* dummy, int r, int& bad, int row1) {
+  constexpr int T = 4 * (C >> 3) + (C & 3), H = (C >> 2) & 1;
+  const float v0 = L[T], v1 = L[T + 1];
+  const float p00 = lane_value(v0, 32 * H + C);
+  const float p01 = lane_value(v0, 32 * H + C + 1);
+  const float p11 = lane_value(v1, 32 * H + C + 1);
+  const float r0 = __builtin_amdgcn_rsqf(p00);
+  const float u01 = p01 * r0;
+  const float d = fmaf(-u01, u01, p11);
+  const float r1 = __builtin_amdgcn_rsqf(d);
+  const float w0 = v0 * r0;
+  const float w1 = fmaf(-u01, w0, v1) * r1;
+  const float y0 = P[T] * r0;
+  const float y1 = fmaf(-u01, y0, P[T + 1]) * r1;
+  if (C < 30) {
+    const float xb = pair_operand<H>(w0, w1);
+    const float pb = pair_operand<H>(y0, y1);
+    const float xa = r > C + 1 ? -xb : 0.f;
+    L = __builtin_amdgcn_mfma_f32_32x32x2f32(xa, xb, L, 0, 0, 0);
+    P = __builtin_amdgcn_mfma_f32_32x32x2f32(xa, pb, P, 0, 0, 0);
+  }
+  // off the chain: the finished rows, and the pivot check.  The lanes of the other half
+  // hold unfinished rows: they write to a block of LDS that nothing reads, so that the
+  // stores need no branch.
+  if (!(p00 > 0.f) && bad == 0) bad = row1 + C;
+  if (!(d > 0.f) && bad == 0) bad = row1 + C + 1;
+  const bool mine = ((threadIdx.x >> 5) & 1) == H;
+  lds_f* const lo = (mine ? leaf_out : dummy) + r;
+  lds_f* const bo = (mine ? blk_out : dummy) + r;
+  lo[C * DLD] = r >= C ? w0 : 0.f;
+  lo[(C + 1) * DLD] = r >= C + 1 ? w1 : 0.f;
+  bo[C * DLD] = y0;
+  bo[(C + 1) * DLD] = y1;
+}
+
+template <int C>
+__device__ __forceinline__ void elim_from(v16f& L, v16f& P, lds_f* leaf_out, lds_f* blk_out,
+                                          lds_f* dummy, int r, int& bad, int row1) {
+  if constexpr (C < 32) {
+    elim_pair<C>(L, P, leaf_out, blk_out, dummy, r, bad, row1);
+    elim_from<C + 2>(L, P, leaf_out, blk_out, dummy, r, bad, row1);
+  }
+}
+
+// L -= A^T A,  P -= A^T B  for 32 finished rows:  A(k, i) = a[k*DLD + i], B(k, j) = b[k*DLD + j]
+// (one read of A serves both products; `with_p` false: L only)
+__device__ __forceinline__ void strip_update(v16f& L, v16f& P, const lds_f* a, const lds_f* b,
+                                             bool with_p) {
+  const int lane = threadIdx.x & 63;
+  const int r = lane & 31, h = lane >> 5;
+  const lds_f* pa = a + h * DLD + r;
+  const lds_f* pb = b + h * DLD + r;
+  float av[16], bv[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    av[i] = pa[2 * i * DLD];
+    bv[i] = with_p ? pb[2 * i * DLD] : 0.f;
+  }
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const float na = -av[i];
+    L = __builtin_amdgcn_mfma_f32_32x32x2f32(na, av[i], L, 0, 0, 0);
+    if (with_p) P = __builtin_amdgcn_mfma_f32_32x32x2f32(na, bv[i], P, 0, 0, 0);
+  }
+}
+
+// Factors and inverts diagonal block p of matrix m: one workgroup of DIAG_THREADS threads
+// (8 waves) with DIAG_SMEM_BYTES of LDS at dsm: S, the block (upper triangle, finished
+// rows of U replacing it strip by strip), and Z, the rows of U_pp^-T.
+// Four strips of 32 rows.  In strip q each of the waves 0-3 holds the leaf (its own copy:
+// the multipliers of a step come from it) and ONE further block of the same rows: a block
+// of the row panel to the right of the leaf (3 - q of them), or a block of the same rows of
+// Z (q + 1 of them, the last one starting as the identity).  That is four blocks in every
+// strip, one per wave, and the inverse Y_pp = Z^T is complete when the last strip is: no back
+// substitution, no doubling.  The rows of strip q meet the update by strip q-1 in registers,
+// on the way in (one 32-deep product per block); the rows further down get it in LDS from
+// the waves 4-7 while strip q is eliminated, and those waves also write the finished rows of
+// strip q-1 to global memory meanwhile, so that only the last strip's are left at the end.
+constexpr int DIAG_THREADS = 512;
+
 __device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, float* dsm) {
   lds_f* const S = (lds_f*)dsm;
-  lds_f* const Yb = S + DB * DLD;
-  lds_f* const Wt = S + 2 * DB * DLD;
+  lds_f* const Z = S + DB * DLD;
   const int n = m.n;
   const int r0 = p * DB;
   const int nb = min(DB, n - r0);
   const int t = threadIdx.x;
   const int wave = t >> 6;
+  const int lane = t & 63;
+  const int r = lane & 31, h = lane >> 5;
 
-  // load the upper triangle; pad with the identity up to 128.  32 loads are
-  // issued before the first is used, so the block costs 2 memory round trips
-  // instead of 64.
+  // load the upper triangle; pad with the identity up to 128.  All 32 loads of a thread are
+  // issued before the first is used: one memory round trip for the block.
   // (raw buffer loads: no 64-bit address per element, and the elements outside the
   // triangle cost no memory access)
-  const __amdgpu_buffer_rsrc_t rs = make_rsrc(m.U + (size_t)r0 * n + r0);
-  for (int e0 = 0; e0 < DB * DB; e0 += 256 * 32) {
+  {
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(m.U + (size_t)r0 * n + r0);
     float v[32];
 #pragma unroll
     for (int u = 0; u < 32; ++u) {
-      const int e = e0 + u * 256 + t;
+      const int e = u * DIAG_THREADS + t;
       const int i = e >> 7, j = e & 127;
       const bool in = i < nb && j < nb && j >= i;
       v[u] = buffer_load(rs, in ? (unsigned)(i * n + j) * 4u : INV_M);
     }
 #pragma unroll
     for (int u = 0; u < 32; ++u) {
-      const int e = e0 + u * 256 + t;
+      const int e = u * DIAG_THREADS + t;
       const int i = e >> 7, j = e & 127;
       const bool in = i < nb && j < nb && j >= i;
       const bool pad = (i >= nb || j >= nb) && i == j;
       S[i * DLD + j] = in ? v[u] : (pad ? 1.f : 0.f);
-      Yb[i * DLD + j] = 0.f;
+      if ((j >> 5) < (i >> 5)) Z[i * DLD + j] = 0.f;     // where the waves 4-7 accumulate
     }
   }
   __syncthreads();
 
-  // Scratch (in Wt, free until the doubling below): two 64-float row buffers per
-  // wave and two dense leaf copies, used alternately.
-  lds_f* const rowbuf = Wt + 128 * wave;
-  lds_f* const ubuf0 = Wt + 512;
-  const int nq = (nb + 31) / 32;
-  // One more turn than there are leaves: the last one only inverts the last leaf
-  // (a second call site would be a second copy of that code, fetched cold).
-  for (int q = 0; q <= nq; ++q) {
-    const int c0 = 32 * q;
-    const int rest = nq - q - 1;     // 32-blocks to the right
-    if (wave < 3) {
-      // waves 0..2: the strip of leaf q, each with one block of the row panel
-      if (q < nq && (wave == 0 || wave < rest))
-        chol_strip_32(S, rowbuf, ubuf0 + 1024 * (q & 1), c0, wave < rest ? c0 + 32 * (wave + 1) : -1,
-                      wave == 0, r0, info + m.out);
-    } else if (q > 0) {
-      // wave 3, meanwhile: inverse of the previous leaf (off the critical path)
-      backsub_32(ubuf0 + 1024 * ((q - 1) & 1), Yb, c0 - 32);
-    }
-    __syncthreads();
-    if (q == nq) break;
-    if (wave == 0 && (t & 32) == 0) {
-      // the factored leaf replaces A[q][q] now that no wave reads the original any more
-      const lds_f* ub = ubuf0 + 1024 * (q & 1);
-#pragma unroll
-      for (int i = 0; i < 32; ++i) S[(c0 + i) * DLD + c0 + t] = ub[i * 32 + t];
-    }
-    if (rest > 0) {
-      // trailing update: A[i][j] -= U[q][i]^T U[q][j], q < i <= j
-      const int nblk = rest * (rest + 1) / 2;
-      for (int blk = wave; blk < nblk; blk += 4) {
-        int bi, bj;
-        upper_tile(blk, rest, bi, bj);
-        const int ci = c0 + 32 * (bi + 1), cj = c0 + 32 * (bj + 1);
-        const v16f acc = lds_mma32(S + c0 * DLD + ci, DLD, 1, S + c0 * DLD + cj, DLD, 1, 32);
-        lds_sub32(S + ci * DLD + cj, DLD, acc);
-      }
-      __syncthreads();
-    }
-  }
-
-  // inverse of the whole block by doubling: 32 -> 64 -> 128
-  if (nq > 1) {
-    // the two level-32 pairs use disjoint data: waves 0-1 take the first, 2-3 the second
-    // (both calls contain the same two barriers, reached by every wave)
-    if (nq > 3) {
-      const int s1 = wave < 2 ? 0 : 64;
-      tri_pair(S, Yb, Wt + (wave < 2 ? 0 : 32 * WLD), s1, 32, wave < 2 ? 0 : 2, 2);
-    } else {
-      tri_pair(S, Yb, Wt, 0, 32, 0, 4);
-    }
-  }
-  if (nq > 2) tri_pair(S, Yb, Wt, 0, 64, 0, 4);
-
-  // write U_pp and Y_pp back, 16 LDS reads in flight per thread
   typedef __attribute__((address_space(1))) float global_f;
   global_f* const gU = (global_f*)(m.U + (size_t)r0 * n + r0);
   global_f* const gY = (global_f*)(m.Y + (size_t)r0 * n + r0);
-  for (int e0 = 0; e0 < DB * DB; e0 += 256 * 16) {
-    float u[16], y[16];
+  // rows [32 qs, 32 qs + 32) of U and the same columns of Y = Z^T, by `nthr` threads
+  auto write_strip = [&](int qs, int tid, int nthr) {
+    for (int e0 = 0; e0 < 32 * DB; e0 += 8 * nthr) {
+      float u[8], y[8];
 #pragma unroll
-    for (int k = 0; k < 16; ++k) {
-      const int e = e0 + k * 256 + t;
-      const int i = e >> 7, j = e & 127;
-      u[k] = S[i * DLD + j];
-      y[k] = Yb[i * DLD + j];
-    }
+      for (int k = 0; k < 8; ++k) {
+        const int e = e0 + k * nthr + tid;
+        const int iu = 32 * qs + (e >> 7), ju = e & 127;      // U[iu][ju]
+        const int iy = e >> 5, jy = 32 * qs + (e & 31);       // Y[iy][jy] = Z[jy][iy]
+        u[k] = S[iu * DLD + ju];
+        y[k] = iy <= jy ? Z[jy * DLD + iy] : 0.f;
+      }
 #pragma unroll
-    for (int k = 0; k < 16; ++k) {
-      const int e = e0 + k * 256 + t;
-      const int i = e >> 7, j = e & 127;
-      if (i < nb && j < nb) {
-        gU[i * n + j] = u[k];
-        gY[i * n + j] = y[k];
+      for (int k = 0; k < 8; ++k) {
+        const int e = e0 + k * nthr + tid;
+        const int iu = 32 * qs + (e >> 7), ju = e & 127;
+        const int iy = e >> 5, jy = 32 * qs + (e & 31);
+        if (iu < nb && ju < nb) gU[iu * n + ju] = u[k];
+        if (iy < nb && jy < nb) gY[iy * n + jy] = y[k];
       }
     }
+  };
+
+  const int nq = (nb + 31) / 32;
+  for (int q = 0; q < nq; ++q) {
+    const int c0 = 32 * q;
+    const int rest = nq - q - 1;       // 32-blocks of the row panel to the right of the leaf
+    const bool strip_wave = wave < 4 && wave < nq;
+    const bool panel = wave < rest;    // this wave's second block: panel block jb, or block s
+    const int jb = q + 1 + wave;       // of the rows of Z
+    const int s = wave - rest;
+    v16f L, P;
+    if (strip_wave) {
+      // the leaf, read symmetrically from the upper triangle
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = 8 * (e >> 2) + 4 * h + (e & 3);
+        L[e] = row <= r ? S[(c0 + row) * DLD + c0 + r] : S[(c0 + r) * DLD + c0 + row];
+      }
+      const lds_f* const src = panel ? S + c0 * DLD + 32 * jb : Z + c0 * DLD + 32 * s;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = 8 * (e >> 2) + 4 * h + (e & 3);
+        P[e] = (panel || s < q) ? src[row * DLD + r] : (row == r ? 1.f : 0.f);
+      }
+      if (q > 0) {
+        // the update by the strip above (the earlier ones are in LDS already)
+        const lds_f* const above = S + (c0 - 32) * DLD;
+        strip_update(L, P, above + c0, panel ? above + 32 * jb : Z + (c0 - 32) * DLD + 32 * s,
+                     panel || s < q);
+      }
+    }
+    __syncthreads();      // every wave has read the leaf
+    if (wave < 4) {
+      if (strip_wave) {
+        int bad = 0;
+        // (block (0, 3) of Z, above its diagonal, is never used; the lane's column made
+        // opaque per strip, so that the lane masks derived from it are computed where they
+        // are used instead of being kept, and spilled, across the loop over the strips)
+        lds_f* const dummy = Z + 96;
+        int rr = r;
+        asm volatile("" : "+v"(rr));
+        elim_from<0>(L, P, wave == 0 ? S + c0 * DLD + c0 : dummy,
+                     panel ? S + c0 * DLD + 32 * jb : Z + c0 * DLD + 32 * s, dummy, rr, bad,
+                     r0 + c0 + 1);
+        if (wave == 0 && bad != 0 && lane == 0) {
+          int* const out = info + m.out;
+          if (*out == 0) *out = bad;
+        }
+      }
+    } else if (q > 0) {
+      // waves 4-7: strip q-1's update of the rows below strip q, block by block in LDS:
+      //   S(i, j) -= U[q-1][i]^T U[q-1][j]  (i <= j),   Z(i, s) -= U[q-1][i]^T Z[q-1][s]  (s < q)
+      const lds_f* const above = S + (c0 - 32) * DLD;
+      const lds_f* const zabove = Z + (c0 - 32) * DLD;
+      int item = 0;
+      for (int i = q + 1; i < nq; ++i) {
+        for (int jj = i; jj < nq + q; ++jj) {
+          if ((item++ & 3) != wave - 4) continue;
+          const bool in_s = jj < nq;
+          const int col = in_s ? jj : jj - nq;             // block column of S, or of Z
+          const v16f acc = lds_mma32(above + 32 * i, DLD, 1,
+                                     (in_s ? above : zabove) + 32 * col, DLD, 1, 32);
+          lds_f* const c = (in_s ? S : Z) + 32 * i * DLD + 32 * col;
+#pragma unroll
+          for (int e = 0; e < 16; ++e) c[(8 * (e >> 2) + 4 * h + (e & 3)) * DLD + r] -= acc[e];
+        }
+      }
+      write_strip(q - 1, t - 256, 256);
+    }
+    __syncthreads();
   }
+  write_strip(nq - 1, t, DIAG_THREADS);
 }
 
-__global__ __launch_bounds__(256) void potrf_diag_kernel(const MatDesc* table, int p, int* info) {
+__global__ __launch_bounds__(DIAG_THREADS) void potrf_diag_kernel(const MatDesc* table, int p,
+                                                                   int* info) {
   extern __shared__ __attribute__((aligned(16))) float dsm[];
   diag_block(table[blockIdx.x], p, info, dsm);
 }
@@ -521,14 +485,16 @@ __global__ __launch_bounds__(NTHREADS, 3) void potrf_trail_kernel(const MatDesc*
 // the others one tile each.  The launch carries the diagonal block's LDS, so one
 // workgroup runs per CU: the tile workgroups use the CUs that the few diagonal blocks
 // leave idle, for about as long as a diagonal block takes.
-__global__ __launch_bounds__(NTHREADS) void potrf_step_kernel(const MatDesc* table, int p,
-                                                              int* info, int ndiag, int row_lo,
-                                                              int row_hi, const WorkList wl) {
+__global__ __launch_bounds__(DIAG_THREADS) void potrf_step_kernel(const MatDesc* table, int p,
+                                                                   int* info, int ndiag,
+                                                                   int row_lo, int row_hi,
+                                                                   const WorkList wl) {
   extern __shared__ __attribute__((aligned(16))) float dsm[];
   if ((int)blockIdx.x < ndiag) {
     diag_block(table[blockIdx.x], p, info, dsm);
     return;
   }
+  if (threadIdx.x >= NTHREADS) return;       // a tile is the work of four waves
   int mat, local;
   work_find_item(wl, (int)blockIdx.x - ndiag, mat, local);
   const MatDesc m = table[mat];
@@ -1099,14 +1065,14 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
       // (rows p+1 .. Pend-1; row p got it right after panel p-1)
       auto rest_items = [&](int T) { return (std::min(Pend, T) - p - 1) * (T - p - 1); };
       if (p == P0 || total_items(na, rest_items) == 0) {
-        hipLaunchKernelGGL(potrf_diag_kernel, dim3(na), dim3(256), DIAG_SMEM_BYTES, stream,
+        hipLaunchKernelGGL(potrf_diag_kernel, dim3(na), dim3(DIAG_THREADS), DIAG_SMEM_BYTES, stream,
                            table, p, info);
       } else {
         bool first = true;
         for_worklists(na, rest_items, [&](const WorkList& wl, int grid) {
           const int nd = first ? na : 0;
           first = false;
-          hipLaunchKernelGGL(potrf_step_kernel, dim3(nd + grid), dim3(NTHREADS), DIAG_SMEM_BYTES,
+          hipLaunchKernelGGL(potrf_step_kernel, dim3(nd + grid), dim3(DIAG_THREADS), DIAG_SMEM_BYTES,
                              stream, table, p, info, nd, p + 1, Pend, wl);
         });
       }
