@@ -172,12 +172,13 @@ __device__ __forceinline__ v16f lds_mma32(const lds_f* a, int a_ks, int a_is, co
 // v_permlane32_swap moves the second into the other half; apart from that and the three
 // pivot entries (v_readlane) no value changes lanes.  The chain from step to step is
 //   matrix instruction -> pivots -> two 1/sqrt -> w1 -> swap -> matrix instruction.
-// The finished rows go to LDS as they are made (`leaf_out`: where U_qq goes, `dummy` for a
-// wave that only needs the multipliers; `blk_out`: the second block's rows; `dummy`: a
-// 32x32 block of LDS that nothing reads).
+// The finished rows go to LDS as they are made, straight from the operand registers
+// (`leaf_rows`: where U_qq goes, or a block of LDS that nothing reads for a wave that only
+// needs the multipliers; `blk_rows`: the second block's rows).  Below its diagonal U_qq is
+// left with rounding noise there; whoever copies it out writes zeros instead.
+// `pmin`, `piv`: the smallest pivot so far and all 32 of them, for the caller's check.
 // With P = rows of the panel the strip ends as U[q][*] = U_qq^-T A[q][*] without a
 // triangular solve; with P = [pending | identity] as the rows of U^-T.
-// `bad`: 1-based row of the first non-positive pivot (row1 = that of the strip's first row).
 template <int H>
 __device__ __forceinline__ float pair_operand(float x0, float x1) {
   // both valid in the lanes of half H -> x0 in lanes 0-31, x1 in lanes 32-63
@@ -188,8 +189,8 @@ __device__ __forceinline__ float pair_operand(float x0, float x1) {
 }
 
 template <int C>
-__device__ __forceinline__ void elim_pair(v16f& L, v16f& P, lds_f* leaf_out, lds_f* blk_out,
-                                          lds_f* dummy, int r, int& bad, int row1) {
+__device__ __forceinline__ void elim_pair(v16f& L, v16f& P, lds_f* leaf_rows, lds_f* blk_rows,
+                                          int r, float& pmin, float (&piv)[32]) {
   constexpr int T = 4 * (C >> 3) + (C & 3), H = (C >> 2) & 1;
   const float v0 = L[T], v1 = L[T + 1];
   const float p00 = lane_value(v0, 32 * H + C);
@@ -201,73 +202,50 @@ __device__ __forceinline__ void elim_pair(v16f& L, v16f& P, lds_f* leaf_out, lds
   const float r1 = __builtin_amdgcn_rsqf(d);
   const float w0 = v0 * r0;
   const float w1 = fmaf(-u01, w0, v1) * r1;
+  const float xb = pair_operand<H>(w0, w1);
+  const float xa = r > C + 1 ? -xb : 0.f;
+  if (C < 30) L = __builtin_amdgcn_mfma_f32_32x32x2f32(xa, xb, L, 0, 0, 0);
+  // (nothing below moves in front of that instruction: the second block's work belongs in
+  // the wait for its result)
+  __builtin_amdgcn_sched_barrier(0);
   const float y0 = P[T] * r0;
   const float y1 = fmaf(-u01, y0, P[T + 1]) * r1;
-  if (C < 30) {
-    const float xb = pair_operand<H>(w0, w1);
-    const float pb = pair_operand<H>(y0, y1);
-    const float xa = r > C + 1 ? -xb : 0.f;
-    L = __builtin_amdgcn_mfma_f32_32x32x2f32(xa, xb, L, 0, 0, 0);
-    P = __builtin_amdgcn_mfma_f32_32x32x2f32(xa, pb, P, 0, 0, 0);
-  }
-  // off the chain: the finished rows, and the pivot check.  The lanes of the other half
-  // hold unfinished rows: they write to a block of LDS that nothing reads, so that the
-  // stores need no branch.
-  if (!(p00 > 0.f) && bad == 0) bad = row1 + C;
-  if (!(d > 0.f) && bad == 0) bad = row1 + C + 1;
-  const bool mine = ((threadIdx.x >> 5) & 1) == H;
-  lds_f* const lo = (mine ? leaf_out : dummy) + r;
-  lds_f* const bo = (mine ? blk_out : dummy) + r;
-  lo[C * DLD] = r >= C ? w0 : 0.f;
-  lo[(C + 1) * DLD] = r >= C + 1 ? w1 : 0.f;
-  bo[C * DLD] = y0;
-  bo[(C + 1) * DLD] = y1;
+  const float pb = pair_operand<H>(y0, y1);
+  if (C < 30) P = __builtin_amdgcn_mfma_f32_32x32x2f32(xa, pb, P, 0, 0, 0);
+  // the finished rows: the operand registers hold row C in the lanes 0-31 and row C+1 in the
+  // lanes 32-63, so one store writes both (the pointers carry the lane's row and column)
+  leaf_rows[C * DLD] = xb;
+  blk_rows[C * DLD] = pb;
+  pmin = fminf(fminf(pmin, p00), d);
+  piv[C] = p00;
+  piv[C + 1] = d;
+  __builtin_amdgcn_sched_barrier(0);
 }
 
 template <int C>
-__device__ __forceinline__ void elim_from(v16f& L, v16f& P, lds_f* leaf_out, lds_f* blk_out,
-                                          lds_f* dummy, int r, int& bad, int row1) {
+__device__ __forceinline__ void elim_from(v16f& L, v16f& P, lds_f* leaf_rows, lds_f* blk_rows,
+                                          int r, float& pmin, float (&piv)[32]) {
   if constexpr (C < 32) {
-    elim_pair<C>(L, P, leaf_out, blk_out, dummy, r, bad, row1);
-    elim_from<C + 2>(L, P, leaf_out, blk_out, dummy, r, bad, row1);
-  }
-}
-
-// L -= A^T A,  P -= A^T B  for 32 finished rows:  A(k, i) = a[k*DLD + i], B(k, j) = b[k*DLD + j]
-// (one read of A serves both products; `with_p` false: L only)
-__device__ __forceinline__ void strip_update(v16f& L, v16f& P, const lds_f* a, const lds_f* b,
-                                             bool with_p) {
-  const int lane = threadIdx.x & 63;
-  const int r = lane & 31, h = lane >> 5;
-  const lds_f* pa = a + h * DLD + r;
-  const lds_f* pb = b + h * DLD + r;
-  float av[16], bv[16];
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    av[i] = pa[2 * i * DLD];
-    bv[i] = with_p ? pb[2 * i * DLD] : 0.f;
-  }
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const float na = -av[i];
-    L = __builtin_amdgcn_mfma_f32_32x32x2f32(na, av[i], L, 0, 0, 0);
-    if (with_p) P = __builtin_amdgcn_mfma_f32_32x32x2f32(na, bv[i], P, 0, 0, 0);
+    elim_pair<C>(L, P, leaf_rows, blk_rows, r, pmin, piv);
+    elim_from<C + 2>(L, P, leaf_rows, blk_rows, r, pmin, piv);
   }
 }
 
 // Factors and inverts diagonal block p of matrix m: one workgroup of DIAG_THREADS threads
-// (8 waves) with DIAG_SMEM_BYTES of LDS at dsm: S, the block (upper triangle, finished
-// rows of U replacing it strip by strip), and Z, the rows of U_pp^-T.
+// (12 waves) with DIAG_SMEM_BYTES of LDS at dsm: S, the block (upper triangle and the whole
+// diagonal 32-blocks; finished rows of U replace it strip by strip), and Z, the rows of
+// U_pp^-T.
 // Four strips of 32 rows.  In strip q each of the waves 0-3 holds the leaf (its own copy:
 // the multipliers of a step come from it) and ONE further block of the same rows: a block
 // of the row panel to the right of the leaf (3 - q of them), or a block of the same rows of
 // Z (q + 1 of them, the last one starting as the identity).  That is four blocks in every
 // strip, one per wave, and the inverse Y_pp = Z^T is complete when the last strip is: no back
-// substitution, no doubling.  The rows of strip q meet the update by strip q-1 in registers,
-// on the way in (one 32-deep product per block); the rows further down get it in LDS from
-// the waves 4-7 while strip q is eliminated, and those waves also write the finished rows of
-// strip q-1 to global memory meanwhile, so that only the last strip's are left at the end.
-constexpr int DIAG_THREADS = 512;
+// substitution, no doubling.  The updates by finished strips happen in LDS, by the other
+// waves: strip q-1's update of the rows of strip q first (four blocks, waves 4-7: this is
+// on the chain), its update of the rows further down while strip q is eliminated (at most
+// five blocks, waves 4-11); those waves also write the finished rows of strip q-1 to global
+// memory meanwhile, so that only the last strip's are left at the end.
+constexpr int DIAG_THREADS = 768;
 
 __device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, float* dsm) {
   lds_f* const S = (lds_f*)dsm;
@@ -276,29 +254,35 @@ __device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, f
   const int r0 = p * DB;
   const int nb = min(DB, n - r0);
   const int t = threadIdx.x;
-  const int wave = t >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);     // (provably uniform: scalar branches)
   const int lane = t & 63;
   const int r = lane & 31, h = lane >> 5;
+  // the waves that eliminate the strips go first wherever they share a SIMD with the others
+  if (wave < 4) __builtin_amdgcn_s_setprio(3);
 
-  // load the upper triangle; pad with the identity up to 128.  All 32 loads of a thread are
+  // load the upper triangle; pad with the identity up to 128.  All loads of a thread are
   // issued before the first is used: one memory round trip for the block.
   // (raw buffer loads: no 64-bit address per element, and the elements outside the
   // triangle cost no memory access)
   {
     const __amdgpu_buffer_rsrc_t rs = make_rsrc(m.U + (size_t)r0 * n + r0);
-    float v[32];
+    constexpr int PER = (DB * DB + DIAG_THREADS - 1) / DIAG_THREADS;
+    float v[PER];
 #pragma unroll
-    for (int u = 0; u < 32; ++u) {
+    for (int u = 0; u < PER; ++u) {
       const int e = u * DIAG_THREADS + t;
       const int i = e >> 7, j = e & 127;
-      const bool in = i < nb && j < nb && j >= i;
-      v[u] = buffer_load(rs, in ? (unsigned)(i * n + j) * 4u : INV_M);
+      // (the diagonal 32-blocks in full, their lower triangles from the upper one: a strip
+      // reads its leaf as a plain symmetric block)
+      const bool in = i < nb && j < nb && (j >= i || (j >> 5) == (i >> 5));
+      v[u] = buffer_load(rs, in ? (unsigned)(min(i, j) * n + max(i, j)) * 4u : INV_M);
     }
 #pragma unroll
-    for (int u = 0; u < 32; ++u) {
+    for (int u = 0; u < PER; ++u) {
       const int e = u * DIAG_THREADS + t;
+      if (e >= DB * DB) break;
       const int i = e >> 7, j = e & 127;
-      const bool in = i < nb && j < nb && j >= i;
+      const bool in = i < nb && j < nb && (j >= i || (j >> 5) == (i >> 5));
       const bool pad = (i >= nb || j >= nb) && i == j;
       S[i * DLD + j] = in ? v[u] : (pad ? 1.f : 0.f);
       if ((j >> 5) < (i >> 5)) Z[i * DLD + j] = 0.f;     // where the waves 4-7 accumulate
@@ -315,15 +299,16 @@ __device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, f
       float u[8], y[8];
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
-        const int e = e0 + k * nthr + tid;
+        const int e = min(e0 + k * nthr + tid, 32 * DB - 1);
         const int iu = 32 * qs + (e >> 7), ju = e & 127;      // U[iu][ju]
         const int iy = e >> 5, jy = 32 * qs + (e & 31);       // Y[iy][jy] = Z[jy][iy]
-        u[k] = S[iu * DLD + ju];
+        u[k] = iu <= ju ? S[iu * DLD + ju] : 0.f;
         y[k] = iy <= jy ? Z[jy * DLD + iy] : 0.f;
       }
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
         const int e = e0 + k * nthr + tid;
+        if (e >= 32 * DB) break;
         const int iu = 32 * qs + (e >> 7), ju = e & 127;
         const int iy = e >> 5, jy = 32 * qs + (e & 31);
         if (iu < nb && ju < nb) gU[iu * n + ju] = u[k];
@@ -333,6 +318,27 @@ __device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, f
   };
 
   const int nq = (nb + 31) / 32;
+  // Strip qs's update of block row i, by `nw` of the waves from 4 on, block by block in LDS
+  // (item k of the row goes to wave 4 + (first + k) % nw):
+  //   S(i, j) -= U[qs][i]^T U[qs][j]  (i <= j),     Z(i, s) -= U[qs][i]^T Z[qs][s]  (s <= qs)
+  auto update_row = [&](int qs, int i, int first, int nw) {
+    const lds_f* const above = S + 32 * qs * DLD;
+    const lds_f* const zabove = Z + 32 * qs * DLD;
+    for (int k = 0; k < nq - i + qs + 1; ++k) {
+      if ((first + k) % nw != wave - 4) continue;
+      const bool in_s = k < nq - i;
+      const int col = in_s ? i + k : k - (nq - i);         // block column of S, or of Z
+      const v16f acc = lds_mma32(above + 32 * i, DLD, 1, (in_s ? above : zabove) + 32 * col,
+                                 DLD, 1, 32);
+      lds_f* const c = (in_s ? S : Z) + (32 * i + 4 * h) * DLD + 32 * col + r;
+      float old[16];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) old[e] = c[(8 * (e >> 2) + (e & 3)) * DLD];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) c[(8 * (e >> 2) + (e & 3)) * DLD] = old[e] - acc[e];
+    }
+    return nq - i + qs + 1;
+  };
   for (int q = 0; q < nq; ++q) {
     const int c0 = 32 * q;
     const int rest = nq - q - 1;       // 32-blocks of the row panel to the right of the leaf
@@ -340,64 +346,57 @@ __device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, f
     const bool panel = wave < rest;    // this wave's second block: panel block jb, or block s
     const int jb = q + 1 + wave;       // of the rows of Z
     const int s = wave - rest;
-    v16f L, P;
-    if (strip_wave) {
-      // the leaf, read symmetrically from the upper triangle
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = 8 * (e >> 2) + 4 * h + (e & 3);
-        L[e] = row <= r ? S[(c0 + row) * DLD + c0 + r] : S[(c0 + r) * DLD + c0 + row];
-      }
-      const lds_f* const src = panel ? S + c0 * DLD + 32 * jb : Z + c0 * DLD + 32 * s;
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = 8 * (e >> 2) + 4 * h + (e & 3);
-        P[e] = (panel || s < q) ? src[row * DLD + r] : (row == r ? 1.f : 0.f);
-      }
-      if (q > 0) {
-        // the update by the strip above (the earlier ones are in LDS already)
-        const lds_f* const above = S + (c0 - 32) * DLD;
-        strip_update(L, P, above + c0, panel ? above + 32 * jb : Z + (c0 - 32) * DLD + 32 * s,
-                     panel || s < q);
-      }
-    }
-    __syncthreads();      // every wave has read the leaf
+    // the rows of this strip meet the update by the strip above (nq blocks, one per wave)
+    if (wave >= 4 && q > 0) update_row(q - 1, q, 0, 4);
+    __syncthreads();
     if (wave < 4) {
       if (strip_wave) {
-        int bad = 0;
+        v16f L, P;
+        const lds_f* const lsrc = S + (c0 + 4 * h) * DLD + c0 + r;
+        const lds_f* const psrc =
+            (panel ? S + c0 * DLD + 32 * jb : Z + c0 * DLD + 32 * s) + 4 * h * DLD + r;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) L[e] = lsrc[(8 * (e >> 2) + (e & 3)) * DLD];
+        if (panel || s < q) {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) P[e] = psrc[(8 * (e >> 2) + (e & 3)) * DLD];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) P[e] = 8 * (e >> 2) + 4 * h + (e & 3) == r ? 1.f : 0.f;
+        }
         // (block (0, 3) of Z, above its diagonal, is never used; the lane's column made
         // opaque per strip, so that the lane masks derived from it are computed where they
         // are used instead of being kept, and spilled, across the loop over the strips)
-        lds_f* const dummy = Z + 96;
         int rr = r;
         asm volatile("" : "+v"(rr));
-        elim_from<0>(L, P, wave == 0 ? S + c0 * DLD + c0 : dummy,
-                     panel ? S + c0 * DLD + 32 * jb : Z + c0 * DLD + 32 * s, dummy, rr, bad,
-                     r0 + c0 + 1);
-        if (wave == 0 && bad != 0 && lane == 0) {
-          int* const out = info + m.out;
-          if (*out == 0) *out = bad;
-        }
-      }
-    } else if (q > 0) {
-      // waves 4-7: strip q-1's update of the rows below strip q, block by block in LDS:
-      //   S(i, j) -= U[q-1][i]^T U[q-1][j]  (i <= j),   Z(i, s) -= U[q-1][i]^T Z[q-1][s]  (s < q)
-      const lds_f* const above = S + (c0 - 32) * DLD;
-      const lds_f* const zabove = Z + (c0 - 32) * DLD;
-      int item = 0;
-      for (int i = q + 1; i < nq; ++i) {
-        for (int jj = i; jj < nq + q; ++jj) {
-          if ((item++ & 3) != wave - 4) continue;
-          const bool in_s = jj < nq;
-          const int col = in_s ? jj : jj - nq;             // block column of S, or of Z
-          const v16f acc = lds_mma32(above + 32 * i, DLD, 1,
-                                     (in_s ? above : zabove) + 32 * col, DLD, 1, 32);
-          lds_f* const c = (in_s ? S : Z) + 32 * i * DLD + 32 * col;
+        lds_f* const leaf_rows = (wave == 0 ? S + c0 * DLD + c0 : Z + 96) + h * DLD + r;
+        lds_f* const blk_rows = (panel ? S + c0 * DLD + 32 * jb : Z + c0 * DLD + 32 * s) + h * DLD + r;
+        float pmin = 1.f, piv[32];
+        // every wave has its copy of the leaf in registers before wave 0 writes U_qq over it
+        // (the waves 4-7 and the idle ones pass the same barrier below)
+        __syncthreads();
+        elim_from<0>(L, P, leaf_rows, blk_rows, rr, pmin, piv);
+        // LAPACK's info: the first pivot that is not positive.  A NaN anywhere in the leaf
+        // reaches a pivot and from there every later one, so the last pivot stands for them.
+        if (wave == 0 && (!(pmin > 0.f) || !(piv[31] > 0.f))) {
+          int bad = 0;
 #pragma unroll
-          for (int e = 0; e < 16; ++e) c[(8 * (e >> 2) + 4 * h + (e & 3)) * DLD + r] -= acc[e];
+          for (int c = 31; c >= 0; --c)
+            if (!(piv[c] > 0.f)) bad = r0 + c0 + c + 1;
+          int* const out = info + m.out;
+          if (lane == 0 && *out == 0) *out = bad;
         }
+      } else {
+        __syncthreads();
       }
-      write_strip(q - 1, t - 256, 256);
+    } else {
+      __syncthreads();
+      // meanwhile: the strip above's update of the rows further down, and its rows to memory
+      if (q > 0) {
+      int first = 0;
+      for (int i = q + 1; i < nq; ++i) first += update_row(q - 1, i, first, 8);
+      write_strip(q - 1, t - 256, DIAG_THREADS - 256);
+      }
     }
     __syncthreads();
   }
