@@ -22,6 +22,7 @@
 // so small factors ride along with the large ones instead of getting a launch
 // sequence each.
 #include <algorithm>
+#include <cstdlib>
 #include <atomic>
 #include <vector>
 
@@ -461,6 +462,17 @@ __device__ __forceinline__ bool trail_tile(int T, int row_lo, int row_hi, int lo
 // 1.0e-4 (16), because a deeper product accumulates more terms before it meets the
 // entry it nearly cancels.
 constexpr int GROUP_BLOCKS = 4;
+// The last TAIL_BLOCKS diagonal blocks of the largest matrices form one group: the deeper
+// update of the rows beyond a group is a launch that lasts as long as one 512-deep tile
+// (50 us) however few tiles it has, while the rank-128 updates of a short trailing matrix
+// all fit beside the next diagonal block (one workgroup per compute unit there).
+static int tail_blocks() {
+  static const int v = [] {
+    const char* e = getenv("KFAC_TAIL_BLOCKS");
+    return e ? atoi(e) : 12;
+  }();
+  return v;
+}
 
 __global__ __launch_bounds__(NTHREADS, 3) void potrf_trail_kernel(const MatDesc* table, int kb0,
                                                                int nk, int row_lo, int row_hi,
@@ -1052,7 +1064,7 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
   });
 
   for (int P0 = 0, Pend = 0; P0 < Tmax; P0 = Pend) {
-    Pend = std::min(P0 + GROUP_BLOCKS, Tmax);
+    Pend = Tmax - P0 <= tail_blocks() ? Tmax : std::min(P0 + GROUP_BLOCKS, Tmax);
     auto total_items = [&](int count, auto&& items) {
       long sum = 0;
       for (int i = 0; i < count; ++i) sum += std::max(0, (int)items(Ts[i]));
@@ -1062,7 +1074,10 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
       const int na = active(p + 1);
       // diagonal block p; beside it, panel p-1's update of the group's rows beyond p
       // (rows p+1 .. Pend-1; row p got it right after panel p-1)
-      auto rest_items = [&](int T) { return (std::min(Pend, T) - p - 1) * (T - p - 1); };
+      auto rest_items = [&](int T) {
+        const int Tr = T - p - 1;      // (all remaining rows: the upper triangle of tiles)
+        return Pend >= T ? Tr * (Tr + 1) / 2 : (Pend - p - 1) * Tr;
+      };
       if (p == P0 || total_items(na, rest_items) == 0) {
         hipLaunchKernelGGL(potrf_diag_kernel, dim3(na), dim3(DIAG_THREADS), DIAG_SMEM_BYTES, stream,
                            table, p, info);
