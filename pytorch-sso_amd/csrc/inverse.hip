@@ -9,10 +9,11 @@
 //      block in LDS; the row panel is a product with that small inverse; the
 //      trailing update is a symmetric rank-128 product on the MFMA tile engine.
 //      Panels are grouped: the rows of the current group receive each panel's
-//      update at once (the next row before anything else, the others from tile
-//      workgroups that share a launch with the next diagonal block, so that the
-//      chip is not idle while that latency-bound block is factored), the rows
-//      beyond the group receive the whole group in one deeper product;
+//      update in the launch that factors the next diagonal block (that block's
+//      workgroup applies it to its own tile first, tile workgroups to the rest,
+//      so that the chip is not idle while the latency-bound block is factored:
+//      two launches per panel), the rows beyond the group receive the whole group
+//      in one deeper product;
 //   3. Y = U^-1 by recursive doubling over the 128-blocks:
 //      Y12 = -Y11 * U12 * Y22, two MFMA products per level, log2(n/128) levels;
 //   4. dst = Y Y^T on the MFMA tile engine (upper tiles, mirrored).
@@ -139,17 +140,31 @@ __device__ __forceinline__ v16f lds_mma32(const lds_f* a, int a_ks, int a_is, co
   for (int t = 0; t < 16; ++t) acc[t] = 0.f;
   const lds_f* pa = a + h * a_ks + r * a_is;
   const lds_f* pb = b + h * b_ks + r * b_js;
-  // 32 deep at a time: the 32 operand reads are issued together, ahead of the 16 MFMAs
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    float av[16], bv[16];
+  // 32 deep at a time: the 32 operand reads of a slice are issued together, and those of the
+  // next slice before the 16 MFMAs of this one
+  float av[16], bv[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      av[i] = pa[(k0 + 2 * i) * a_ks];
-      bv[i] = pb[(k0 + 2 * i) * b_ks];
+  for (int i = 0; i < 16; ++i) {
+    av[i] = pa[2 * i * a_ks];
+    bv[i] = pb[2 * i * b_ks];
+  }
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    float an[16], bn[16];
+    if (k0 + 32 < K) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        an[i] = pa[(k0 + 32 + 2 * i) * a_ks];
+        bn[i] = pb[(k0 + 32 + 2 * i) * b_ks];
+      }
     }
 #pragma unroll
     for (int i = 0; i < 16; ++i)
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[i], acc, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      av[i] = an[i];
+      bv[i] = bn[i];
+    }
   }
   return acc;
 }
@@ -247,7 +262,10 @@ __device__ __forceinline__ void elim_from(v16f& L, v16f& P, lds_f* leaf_rows, ld
 // memory meanwhile, so that only the last strip's are left at the end.
 constexpr int DIAG_THREADS = 768;
 
-__device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, float* dsm) {
+// `pending`: the row panel above (block row p-1) has not been applied to this block yet
+// (the launch that holds this workgroup applies it to the rest of block row p meanwhile).
+__device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, float* dsm,
+                                           bool pending) {
   lds_f* const S = (lds_f*)dsm;
   lds_f* const Z = S + DB * DLD;
   const int n = m.n;
@@ -266,8 +284,10 @@ __device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, f
   // triangle cost no memory access)
   {
     const __amdgpu_buffer_rsrc_t rs = make_rsrc(m.U + (size_t)r0 * n + r0);
+    // (pending: tile (p-1, p) of U, all of its 128 rows, in the same round trip)
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(m.U + ((size_t)r0 - DB) * n + r0);
     constexpr int PER = (DB * DB + DIAG_THREADS - 1) / DIAG_THREADS;
-    float v[PER];
+    float v[PER], a[PER];
 #pragma unroll
     for (int u = 0; u < PER; ++u) {
       const int e = u * DIAG_THREADS + t;
@@ -276,6 +296,7 @@ __device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, f
       // reads its leaf as a plain symmetric block)
       const bool in = i < nb && j < nb && (j >= i || (j >> 5) == (i >> 5));
       v[u] = buffer_load(rs, in ? (unsigned)(min(i, j) * n + max(i, j)) * 4u : INV_M);
+      if (pending) a[u] = buffer_load(ra, (i < DB && j < nb) ? (unsigned)(i * n + j) * 4u : INV_M);
     }
 #pragma unroll
     for (int u = 0; u < PER; ++u) {
@@ -285,10 +306,26 @@ __device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, f
       const bool in = i < nb && j < nb && (j >= i || (j >> 5) == (i >> 5));
       const bool pad = (i >= nb || j >= nb) && i == j;
       S[i * DLD + j] = in ? v[u] : (pad ? 1.f : 0.f);
-      if ((j >> 5) < (i >> 5)) Z[i * DLD + j] = 0.f;     // where the waves 4-7 accumulate
+      if (pending) Z[i * DLD + j] = a[u];
     }
   }
   __syncthreads();
+  if (pending) {
+    // S -= W^T W, W = tile (p-1, p) of U (in Z for now): the ten 32x32 blocks on and above
+    // the diagonal, one per wave, 128 deep
+    if (wave < 10) {
+      int bi, bj;
+      upper_tile(wave, 4, bi, bj);
+      const v16f acc = lds_mma32(Z + 32 * bi, DLD, 1, Z + 32 * bj, DLD, 1, DB);
+      lds_f* const c = S + (32 * bi + 4 * h) * DLD + 32 * bj + r;
+      float old[16];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) old[e] = c[(8 * (e >> 2) + (e & 3)) * DLD];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) c[(8 * (e >> 2) + (e & 3)) * DLD] = old[e] - acc[e];
+    }
+    // (the loop over the strips starts with a barrier; nothing there reads Z before writing it)
+  }
 
   typedef __attribute__((address_space(1))) float global_f;
   global_f* const gU = (global_f*)(m.U + (size_t)r0 * n + r0);
@@ -331,9 +368,12 @@ __device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, f
       const v16f acc = lds_mma32(above + 32 * i, DLD, 1, (in_s ? above : zabove) + 32 * col,
                                  DLD, 1, 32);
       lds_f* const c = (in_s ? S : Z) + (32 * i + 4 * h) * DLD + 32 * col + r;
+      // (a block of Z below the diagonal starts at zero: its first update, by the strip of
+      // its column, finds it uninitialised)
+      const bool fresh = !in_s && col == qs;
       float old[16];
 #pragma unroll
-      for (int e = 0; e < 16; ++e) old[e] = c[(8 * (e >> 2) + (e & 3)) * DLD];
+      for (int e = 0; e < 16; ++e) old[e] = fresh ? 0.f : c[(8 * (e >> 2) + (e & 3)) * DLD];
 #pragma unroll
       for (int e = 0; e < 16; ++e) c[(8 * (e >> 2) + (e & 3)) * DLD] = old[e] - acc[e];
     }
@@ -406,7 +446,7 @@ __device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, f
 __global__ __launch_bounds__(DIAG_THREADS) void potrf_diag_kernel(const MatDesc* table, int p,
                                                                    int* info) {
   extern __shared__ __attribute__((aligned(16))) float dsm[];
-  diag_block(table[blockIdx.x], p, info, dsm);
+  diag_block(table[blockIdx.x], p, info, dsm, false);
 }
 
 // row panel of the blocked Cholesky: U[p, j] = Ypp^T * A[p, j], j > p
@@ -497,7 +537,7 @@ __global__ __launch_bounds__(DIAG_THREADS) void potrf_step_kernel(const MatDesc*
                                                                    const WorkList wl) {
   extern __shared__ __attribute__((aligned(16))) float dsm[];
   if ((int)blockIdx.x < ndiag) {
-    diag_block(table[blockIdx.x], p, info, dsm);
+    diag_block(table[blockIdx.x], p, info, dsm, true);
     return;
   }
   if (threadIdx.x >= NTHREADS) return;       // a tile is the work of four waves
@@ -506,24 +546,23 @@ __global__ __launch_bounds__(DIAG_THREADS) void potrf_step_kernel(const MatDesc*
   const MatDesc m = table[mat];
   int bi, bj;
   if (!trail_tile(m.T, row_lo, row_hi, local, bi, bj)) return;
+  if (bj == p) return;                       // tile (p, p): the diagonal block's own workgroup
   const int n = m.n;
   DenseKM P{m.U + (size_t)(p - 1) * DB * n, nullptr, n, n, 0};
   EpiStore epi{m.U, n, n, n, -1.f, 1.f, false};
   gemm_tile(P, P, bi * BM, bj * BN, 0, DB, bi == bj, epi, dsm);
 }
 
-// The row panel (near == 0) or the near update with one block row (near == 1) for
-// launches of few tiles: the same 128x128x128 product, but by 16 waves with one
-// 32x32 block each instead of 4 waves with four.  A tile is a chain of dependent-issue
-// MFMAs, 256 per wave (7.8 us) in the tile engine and 64 here, and at the end of a
-// factorisation nothing else runs beside it.  Both operands are fetched whole (32
-// loads per thread in flight, and the old values of C with them) into 128 KB of LDS.
+// The row panel for launches of few tiles: the same 128x128x128 product, but by 16 waves
+// with one 32x32 block each instead of 4 waves with four.  A tile is a chain of
+// dependent-issue MFMAs, 256 per wave (7.8 us) in the tile engine and 64 here, and at the
+// end of a factorisation nothing else runs beside it.  Both operands are fetched whole (32
+// loads per thread in flight) into 128 KB of LDS.
 constexpr int FINE_THREADS = 1024;
 constexpr int FINE_SMEM_BYTES = 2 * DB * DB * (int)sizeof(float);
 constexpr int FINE_MAX_TILES = 256;      // one workgroup per CU
 
 __global__ __launch_bounds__(FINE_THREADS) void potrf_fine_kernel(const MatDesc* table, int p,
-                                                                  int near, int row_hi,
                                                                   const WorkList wl) {
   extern __shared__ __attribute__((aligned(16))) float fsm[];
   lds_f* const tp = (lds_f*)fsm;
@@ -532,114 +571,79 @@ __global__ __launch_bounds__(FINE_THREADS) void potrf_fine_kernel(const MatDesc*
   work_find(wl, mat, local);
   const MatDesc m = table[mat];
   const int n = m.n;
-  int bi, bj;
-  if (near) {
-    if (!trail_tile(m.T, p + 1, row_hi, local, bi, bj)) return;
-  } else {
-    bi = p;
-    bj = p + 1 + local;
-    if (bj >= m.T) return;
-  }
-  const float* kbase = m.U + (size_t)p * DB * n;            // block row p of U
-  // P(k, i), i < pw;  Q(k, j), j < qw;  C[i][j]
-  const float* P = near ? kbase + bi * DB : m.Y + (size_t)p * DB * n + p * DB;
-  const float* Q = kbase + bj * DB;
-  float* C = m.U + (size_t)bi * DB * n + bj * DB;
-  const int pw = near ? min(DB, n - bi * DB) : DB;
+  const int bj = p + 1 + local;
+  if (bj >= m.T) return;
+  // P(k, i) = Y_pp;  Q(k, j) = A[p, bj], j < qw;  C[i][j] = U[p, bj] over Q
+  const float* P = m.Y + (size_t)p * DB * n + p * DB;
+  const float* Q = m.U + (size_t)p * DB * n + bj * DB;
+  float* C = m.U + (size_t)p * DB * n + bj * DB;
   const int qw = min(DB, n - bj * DB);
-  const bool same = near && bi == bj;
   const int t = threadIdx.x;
   const int wave = t >> 6, lane = t & 63;
   const int r = lane & 31, h = lane >> 5;
   const int wr = wave >> 2, wc = wave & 3;
 
-  {
-    const int mm = t & (DB - 1), kq = t >> 7;
-    const __amdgpu_buffer_rsrc_t rp = make_rsrc(P), rq = make_rsrc(Q);
-    float vp[16], vq[16];
+  const int mm = t & (DB - 1), kq = t >> 7;
+  const __amdgpu_buffer_rsrc_t rp = make_rsrc(P), rq = make_rsrc(Q);
+  float vp[16], vq[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const unsigned off = (unsigned)((kq + 8 * i) * n + mm) * 4u;
-      vp[i] = buffer_load(rp, mm < pw ? off : INV_M);
-      vq[i] = same ? 0.f : buffer_load(rq, mm < qw ? off : INV_M);
-    }
-    float old[16];
-    if (near) {
+  for (int i = 0; i < 16; ++i) {
+    const unsigned off = (unsigned)((kq + 8 * i) * n + mm) * 4u;
+    vp[i] = buffer_load(rp, off);
+    vq[i] = buffer_load(rq, mm < qw ? off : INV_M);
+  }
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = 32 * wr + 8 * (e >> 2) + 4 * h + (e & 3), col = 32 * wc + r;
-        old[e] = (row < pw && col < qw) ? C[(size_t)row * n + col] : 0.f;
-      }
-    }
+  for (int i = 0; i < 16; ++i) {
+    tp[(kq + 8 * i) * DB + mm] = vp[i];
+    tq[(kq + 8 * i) * DB + mm] = vq[i];
+  }
+  __syncthreads();
+  const v16f acc = lds_mma32(tp + 32 * wr, DB, 1, tq + 32 * wc, DB, 1, DB);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      tp[(kq + 8 * i) * DB + mm] = vp[i];
-      if (!same) tq[(kq + 8 * i) * DB + mm] = vq[i];
-    }
-    __syncthreads();
-    const v16f acc = lds_mma32(tp + 32 * wr, DB, 1, (same ? tp : tq) + 32 * wc, DB, 1, DB);
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int row = 32 * wr + 8 * (e >> 2) + 4 * h + (e & 3), col = 32 * wc + r;
-      if (row < pw && col < qw) C[(size_t)row * n + col] = near ? old[e] - acc[e] : acc[e];
-    }
+  for (int e = 0; e < 16; ++e) {
+    const int row = 32 * wr + 8 * (e >> 2) + 4 * h + (e & 3), col = 32 * wc + r;
+    if (col < qw) C[(size_t)row * n + col] = acc[e];
   }
 }
 
-// The same products for launches of very few tiles (at most SUB_MAX_TILES): every tile is
-// dealt to four workgroups, so that four CUs' matrix cores work on it.  A workgroup
-// takes RB x CB blocks of 32x32 (RB * CB == 4) and 8 waves: a wave does one block over
-// half of the 128-deep reduction and the halves are added through LDS.  The near update
-// is cut into 64x64 quarters (2 x 2 blocks).  The row panel overwrites its own right-hand
-// operand, so its pieces must not share columns: four 128x32 column strips (4 x 1 blocks).
+// The same product for launches of very few tiles (at most SUB_MAX_TILES): every tile is
+// dealt to four workgroups, so that four CUs' matrix cores work on it.  The row panel
+// overwrites its own right-hand operand, so the pieces must not share columns: four
+// 128x32 column strips, four 32x32 blocks each.  8 waves: a wave does one block over half
+// of the 128-deep reduction and the halves are added through LDS.
 constexpr int SUB_THREADS = 512;
 constexpr int SUB_SMEM_BYTES = DB * (128 + 32) * (int)sizeof(float);
 constexpr int SUB_MAX_TILES = 64;        // 4 workgroups per tile, one workgroup per CU
 
-template <int RB, int CB>
 __global__ __launch_bounds__(SUB_THREADS) void potrf_sub_kernel(const MatDesc* table, int p,
-                                                                int near, int row_hi,
                                                                 const WorkList wl) {
-  constexpr int WP = 32 * RB, WQ = 32 * CB;
-  static_assert(RB * CB == 4, "a workgroup takes four 32x32 blocks");
-  static_assert(DB * (WP + WQ) * (int)sizeof(float) <= SUB_SMEM_BYTES, "LDS");
+  constexpr int WP = 128, WQ = 32;
   extern __shared__ __attribute__((aligned(16))) float fsm[];
   lds_f* const tp = (lds_f*)fsm;
   lds_f* const tq = tp + DB * WP;
   int mat, item;
   work_find(wl, mat, item);
-  const int local = item >> 2, sub = item & 3;
-  const int si = sub / (4 / CB), sj = sub % (4 / CB);
+  const int local = item >> 2, sj = item & 3;
   const MatDesc m = table[mat];
   const int n = m.n;
-  int bi, bj;
-  if (near) {
-    if (!trail_tile(m.T, p + 1, row_hi, local, bi, bj)) return;
-  } else {
-    bi = p;
-    bj = p + 1 + local;
-    if (bj >= m.T) return;
-  }
-  const float* kbase = m.U + (size_t)p * DB * n;            // block row p of U
-  const float* P = near ? kbase + bi * DB : m.Y + (size_t)p * DB * n + p * DB;
-  const float* Q = kbase + bj * DB;
-  float* C = m.U + (size_t)bi * DB * n + bj * DB;
-  const int pw = near ? min(DB, n - bi * DB) : DB;
+  const int bj = p + 1 + local;
+  if (bj >= m.T) return;
+  const float* P = m.Y + (size_t)p * DB * n + p * DB;
+  const float* Q = m.U + (size_t)p * DB * n + bj * DB;
+  float* C = m.U + (size_t)p * DB * n + bj * DB;
   const int qw = min(DB, n - bj * DB);
   const int t = threadIdx.x;
   const int wave = t >> 6, lane = t & 63;
   const int r = lane & 31, h = lane >> 5;
-  const int blk = wave & 3, khalf = wave >> 2;
-  const int br = blk / CB, bc = blk % CB;
-  const int row0 = WP * si + 32 * br, col0 = WQ * sj + 32 * bc;   // of this wave's block in the tile
+  const int br = wave & 3, khalf = wave >> 2;
+  const int row0 = 32 * br, col0 = WQ * sj;         // of this wave's block in the tile
 
   const __amdgpu_buffer_rsrc_t rp = make_rsrc(P), rq = make_rsrc(Q);
   float vp[WP / 4], vq[WQ / 4];
 #pragma unroll
   for (int i = 0; i < WP / 4; ++i) {
     const int idx = t + SUB_THREADS * i;
-    const int k = idx / WP, col = WP * si + idx % WP;
-    vp[i] = buffer_load(rp, col < pw ? (unsigned)(k * n + col) * 4u : INV_M);
+    vp[i] = buffer_load(rp, (unsigned)((idx / WP) * n + idx % WP) * 4u);
   }
 #pragma unroll
   for (int i = 0; i < WQ / 4; ++i) {
@@ -647,24 +651,16 @@ __global__ __launch_bounds__(SUB_THREADS) void potrf_sub_kernel(const MatDesc* t
     const int k = idx / WQ, col = WQ * sj + idx % WQ;
     vq[i] = buffer_load(rq, col < qw ? (unsigned)(k * n + col) * 4u : INV_M);
   }
-  float old[16];
-  if (near && khalf == 0) {
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int row = row0 + 8 * (e >> 2) + 4 * h + (e & 3), col = col0 + r;
-      old[e] = (row < pw && col < qw) ? C[(size_t)row * n + col] : 0.f;
-    }
-  }
 #pragma unroll
   for (int i = 0; i < WP / 4; ++i) tp[t + SUB_THREADS * i] = vp[i];
 #pragma unroll
   for (int i = 0; i < WQ / 4; ++i) tq[t + SUB_THREADS * i] = vq[i];
   __syncthreads();
-  const v16f acc = lds_mma32(tp + 64 * khalf * WP + 32 * br, WP, 1,
-                             tq + 64 * khalf * WQ + 32 * bc, WQ, 1, 64);
+  const v16f acc = lds_mma32(tp + 64 * khalf * WP + 32 * br, WP, 1, tq + 64 * khalf * WQ, WQ, 1,
+                             64);
   __syncthreads();
   // the second halves of the reduction travel through LDS (the operands are spent)
-  lds_f* const red = tp + blk * 1024;
+  lds_f* const red = tp + br * 1024;
   if (khalf == 1) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) red[e * 64 + lane] = acc[e];
@@ -675,7 +671,7 @@ __global__ __launch_bounds__(SUB_THREADS) void potrf_sub_kernel(const MatDesc* t
     for (int e = 0; e < 16; ++e) {
       const int row = row0 + 8 * (e >> 2) + 4 * h + (e & 3), col = col0 + r;
       const float v = acc[e] + red[e * 64 + lane];
-      if (row < pw && col < qw) C[(size_t)row * n + col] = near ? old[e] - v : v;
+      if (col < qw) C[(size_t)row * n + col] = v;
     }
   }
 }
@@ -984,8 +980,7 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
   if (!enable_large_lds((const void*)potrf_diag_kernel, DIAG_SMEM_BYTES) ||
       !enable_large_lds((const void*)potrf_step_kernel, DIAG_SMEM_BYTES) ||
       !enable_large_lds((const void*)potrf_fine_kernel, FINE_SMEM_BYTES) ||
-      !enable_large_lds((const void*)potrf_sub_kernel<2, 2>, SUB_SMEM_BYTES) ||
-      !enable_large_lds((const void*)potrf_sub_kernel<4, 1>, SUB_SMEM_BYTES))
+      !enable_large_lds((const void*)potrf_sub_kernel, SUB_SMEM_BYTES))
     return KFAC_ERR_LAUNCH;
 
   // descending size order; remember where each caller index went
@@ -1067,13 +1062,15 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
     };
     for (int p = P0; p < Pend; ++p) {
       const int na = active(p + 1);
-      // diagonal block p; beside it, panel p-1's update of the group's rows beyond p
-      // (rows p+1 .. Pend-1; row p got it right after panel p-1)
+      // diagonal block p; from the group's second block on it first takes panel p-1's update
+      // itself, and the same launch holds the tiles that apply that panel to the other rows
+      // of the group (block row p first: the next row panel needs it; nothing else needs any
+      // of them before the next launch)
       auto rest_items = [&](int T) {
-        const int Tr = T - p - 1;      // (all remaining rows: the upper triangle of tiles)
-        return Pend >= T ? Tr * (Tr + 1) / 2 : (Pend - p - 1) * Tr;
+        const int Tr = T - p;          // (all remaining rows: the upper triangle of tiles)
+        return Pend >= T ? Tr * (Tr + 1) / 2 : (Pend - p) * Tr;
       };
-      if (p == P0 || total_items(na, rest_items) == 0) {
+      if (p == P0) {
         hipLaunchKernelGGL(potrf_diag_kernel, dim3(na), dim3(DIAG_THREADS), DIAG_SMEM_BYTES, stream,
                            table, p, info);
       } else {
@@ -1082,7 +1079,7 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
           const int nd = first ? na : 0;
           first = false;
           hipLaunchKernelGGL(potrf_step_kernel, dim3(nd + grid), dim3(DIAG_THREADS), DIAG_SMEM_BYTES,
-                             stream, table, p, info, nd, p + 1, Pend, wl);
+                             stream, table, p, info, nd, p, Pend, wl);
         });
       }
       const int nb = active(p + 2);
@@ -1091,39 +1088,17 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
       if (total_items(nb, panel_items) <= SUB_MAX_TILES) {
         for_worklists(nb, [&](int T) { return 4 * std::max(0, panel_items(T)); },
                       [&](const WorkList& wl, int grid) {
-                        hipLaunchKernelGGL((potrf_sub_kernel<4, 1>), dim3(grid), dim3(SUB_THREADS),
-                                           SUB_SMEM_BYTES, stream, table, p, 0, 0, wl);
+                        hipLaunchKernelGGL(potrf_sub_kernel, dim3(grid), dim3(SUB_THREADS),
+                                           SUB_SMEM_BYTES, stream, table, p, wl);
                       });
       } else
       for_worklists(nb, panel_items, [&](const WorkList& wl, int grid) {
         if (grid <= FINE_MAX_TILES)
           hipLaunchKernelGGL(potrf_fine_kernel, dim3(grid), dim3(FINE_THREADS), FINE_SMEM_BYTES,
-                             stream, table, p, 0, 0, wl);
+                             stream, table, p, wl);
         else
           KFAC_LAUNCH_TILE2(potrf_panel_kernel, dim3(grid), stream, table, p, wl);
       });
-      if (p + 1 < Pend) {
-        // panel p's update of block row p+1 (the next diagonal block and row panel need it);
-        // the group's other rows get it beside the next diagonal block
-        auto row_items = [&](int T) { return T > p + 1 ? T - p - 1 : 0; };
-        if (total_items(nb, row_items) <= SUB_MAX_TILES) {
-          for_worklists(nb, [&](int T) { return 4 * std::max(0, row_items(T)); },
-                        [&](const WorkList& wl, int grid) {
-                          hipLaunchKernelGGL((potrf_sub_kernel<2, 2>), dim3(grid),
-                                             dim3(SUB_THREADS), SUB_SMEM_BYTES, stream, table, p,
-                                             1, p + 2, wl);
-                        });
-        } else
-        for_worklists(nb, row_items,
-                      [&](const WorkList& wl, int grid) {
-                        if (grid <= FINE_MAX_TILES)
-                          hipLaunchKernelGGL(potrf_fine_kernel, dim3(grid), dim3(FINE_THREADS),
-                                             FINE_SMEM_BYTES, stream, table, p, 1, p + 2, wl);
-                        else
-                          KFAC_LAUNCH_TILE2(potrf_trail_kernel, dim3(grid), stream, table, p, 1,
-                                            p + 1, p + 2, wl);
-                      });
-      }
     }
     const int nc = active(Pend + 1);
     if (Pend < Tmax && nc > 0) {
