@@ -56,9 +56,12 @@ size_t kfac_factor_workspace_bytes(int d, int64_t K);
  * bias) and :61-67 with the n^2 rescale of curvature.py:154-155,299-300
  * (G, alpha = n, add_bias = 0).  beta != 0 fuses the accumulation of
  * utils/accumulator.py:23-38 or the running average of curvature.py:185-186
- * into the GEMM epilogue; with beta == 0, neither C nor C_prev is read.  C_prev is
- * taken to be symmetric (what these routines write is, to the bit): only its
- * upper triangle is read, and C is written symmetric. */
+ * into the GEMM epilogue; with beta == 0, neither C nor C_prev is read.  C_prev
+ * must be symmetric (what these routines write is, to the bit): its upper
+ * triangle is read, its lower one only inside the 32x32 blocks on the diagonal,
+ * and C is written symmetric (the blocks below the diagonal are mirror images
+ * of those above); a C_prev that is not symmetric gives neither the
+ * element-wise average nor a symmetric one. */
 int kfac_factor_linear(const float* x, int64_t rows, int f, int64_t ldx, int add_bias,
                        float alpha, float beta, const float* C_prev, float* C,
                        void* workspace, size_t workspace_bytes, void* stream);
@@ -225,11 +228,15 @@ int kfac_damped_inverse_batched(int count, const int* dims, const float* const* 
  * every GPU the library runs on until the process ends), and the call makes no hipMalloc,
  * hipFree or other allocating call.  A list that needs more than that
  * (kfac_inverse_workspace_bytes(count, dims) > kfac_static_workspace_bytes(); e.g. one
- * matrix above 1447 x 1447) is rejected with KFAC_ERR_TOO_LARGE before anything is
- * launched.  The first call on a device looks up the array's address on that device (and
- * raises the LDS limit of the kernels); make that call outside a capture.  All calls on one
- * GPU share the array: calls that overlap in time on one GPU (two streams, two threads)
- * race; calls in stream order on one stream do not. */
+ * matrix above 1448 x 1448) is rejected with KFAC_ERR_TOO_LARGE before anything is
+ * launched.  The first call on a device looks up the array's address on that device,
+ * creates the event below (and raises the LDS limit of the kernels); make that call outside
+ * a capture.  All calls on one GPU share the array; they are put in order: a call's stream
+ * first waits for an event that the previous call on that GPU recorded behind its last
+ * kernel, so calls on two streams or from two threads run one after the other instead of
+ * racing.  A stream under graph capture takes no part in that (inside a graph the graph's
+ * own order applies): calls captured into graphs that may run at the same time still
+ * race. */
 size_t kfac_static_workspace_bytes(void);
 int kfac_damped_inverse_batched_static(int count, const int* dims, const float* const* src,
                                        const float* damp, float* const* dst, int* info,

@@ -439,10 +439,12 @@ static GroupedPlan make_plan(int count, const kfac_factor_job* jobs) {
 // step after step: the last plans of every host thread are kept (never freed: objects of
 // this library have no destructors that could run at process exit).
 struct JobShape {
-  int kind, add_bias, c, H, W, kh, kw, sh, sw, ph, pw, dh, dw;
   int64_t rows;
+  int kind, add_bias, c, H, W, kh, kw, sh, sw, ph, pw, dh, dw, unused;
   bool operator==(const JobShape& o) const { return memcmp(this, &o, sizeof(JobShape)) == 0; }
 };
+static_assert(sizeof(JobShape) == sizeof(int64_t) + 14 * sizeof(int),
+              "no padding: the shapes are compared as bytes");
 
 static JobShape shape_of(const kfac_factor_job& j) {
   JobShape s;

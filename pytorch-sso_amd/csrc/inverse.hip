@@ -24,6 +24,7 @@
 // sequence each.
 #include <algorithm>
 #include <atomic>
+#include <mutex>
 #include <vector>
 
 #include "common.h"
@@ -1179,6 +1180,24 @@ static void* static_scratch() {
   return ptr;
 }
 
+// Calls that share the array are put in order: each call records an event behind its last
+// kernel, and the next call on that device makes its stream wait for it first (a no-op for
+// the single-stream caller).  The events are created on a device's first call.  A stream
+// under graph capture takes no part: an event recorded outside a capture cannot be waited
+// for inside one, and inside a graph the graph's own order applies.
+static std::mutex scratch_mutex;
+static hipEvent_t scratch_done[SCRATCH_MAX_DEVICES];    // (never destroyed: no teardown order)
+static bool scratch_done_set[SCRATCH_MAX_DEVICES];
+
+static bool stream_is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return st != hipStreamCaptureStatusNone;
+}
+
 }  // namespace kfac
 
 using namespace kfac;
@@ -1203,7 +1222,23 @@ int kfac_damped_inverse_batched_static(int count, const int* dims, const float* 
   if (inverse_workspace_bytes(d) > STATIC_SCRATCH_BYTES) return KFAC_ERR_TOO_LARGE;
   void* ptr = static_scratch();
   if (ptr == nullptr) return KFAC_ERR_LAUNCH;
-  return run_batched(mats, MODE_INVERSE, info, ptr, STATIC_SCRATCH_BYTES, (hipStream_t)stream);
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SCRATCH_MAX_DEVICES) return KFAC_ERR_LAUNCH;
+  hipStream_t st = (hipStream_t)stream;
+  std::lock_guard<std::mutex> order(scratch_mutex);
+  const bool ordered = !stream_is_capturing(st);
+  if (ordered) {
+    if (!scratch_done_set[dev]) {
+      if (hipEventCreateWithFlags(&scratch_done[dev], hipEventDisableTiming) != hipSuccess)
+        return KFAC_ERR_LAUNCH;
+      scratch_done_set[dev] = true;
+    } else if (hipStreamWaitEvent(st, scratch_done[dev], 0) != hipSuccess) {
+      return KFAC_ERR_LAUNCH;
+    }
+  }
+  const int status = run_batched(mats, MODE_INVERSE, info, ptr, STATIC_SCRATCH_BYTES, st);
+  if (ordered && hipEventRecord(scratch_done[dev], st) != hipSuccess) return KFAC_ERR_LAUNCH;
+  return status;
 }
 
 size_t kfac_inverse_workspace_bytes(int count, const int* dims) {

@@ -199,6 +199,9 @@ def _run_deferred(only=None):
                         side.wait_event(done)
         for st in others:
             target.wait_stream(st)
+        # (the call's workspace is the cached scratch of the stream it runs on; a pass under
+        # no_grad leaves its inputs referenced in the queue, or in `_inflight`, until the
+        # next flush or join)
         _ops.factor_grouped(jobs, device, stream=side)
         if side is not None:
             # the tensors stay referenced until the caller's stream has been made to wait
@@ -269,7 +272,16 @@ def join(device=None):
         for lane in lanes:
             cur.wait_stream(_streams[i][lane][0])
         with _lock:
-            _inflight.pop(i, None)      # (what these calls read may be freed from here on)
+            held = _inflight.pop(i, None) or []
+        # What these calls read may be freed from here on, and the allocator hands a freed
+        # block out again on the stream it was allocated under: a hook that ran under
+        # another stream than this one has that stream wait for the call too.
+        for done, items, _ in held:
+            waited = []
+            for _, _, st in items:
+                if st != cur and st not in waited:
+                    waited.append(st)
+                    st.wait_event(done)
 
 
 def _at_exit():

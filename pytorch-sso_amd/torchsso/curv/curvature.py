@@ -574,6 +574,7 @@ def update_inv_all(curvs, with_std=()):
             info = _ops.pi_damped_inverse_factored_batched(*args, column(0, 0), column(0, 1),
                                                            column(1, 0), column(1, 1))
             for c in kron:
+                c._info_reversed = False
                 if id(c) in wanted:
                     c._std_current = False
         elif wanted:
@@ -583,8 +584,12 @@ def update_inv_all(curvs, with_std=()):
                 if id(c) in wanted:
                     c._std_current = True      # update_std_all has nothing to do for it
                     c.std_info = None          # (a failure shows in `info`)
+            for c in kron:
+                c._info_reversed = id(c) in wanted
         else:
             _, _, info = _ops.pi_damped_inverse_batched(*args, column(0, 0), column(0, 1))
+            for c in kron:
+                c._info_reversed = False
         for i, c in enumerate(kron):
             c.info = info[2 * i:2 * i + 2]
     if diag:
@@ -665,8 +670,13 @@ def check_spd_all(curvs):
     for k, (li, c, what) in enumerate(owners):
         for side, code in zip(('A', 'G'), flat[2 * k:2 * k + 2]):
             if code != 0:
-                bad.append('layer %d (%s): %s of factor %s failed, leading minor of order %d is '
-                           'not positive' % (li, type(c.module).__name__, what, side, code))
+                # (a factor inverted together with its std is factored back to front: the
+                # status word then counts a leading minor of the matrix with its rows and
+                # columns reversed, i.e. a trailing minor of the factor)
+                which = ('trailing' if what == 'inverse' and getattr(c, '_info_reversed', False)
+                         else 'leading')
+                bad.append('layer %d (%s): %s of factor %s failed, %s minor of order %d is '
+                           'not positive' % (li, type(c.module).__name__, what, side, which, code))
     if bad:
         raise NotPositiveDefiniteError(
             'curvature factors that are not positive definite (raise `damping`):\n  '

@@ -253,6 +253,13 @@ class SecondOrderOptimizer(Optimizer):
             if curv is not None and curv.kind == 'kron' and not curv.fuse_ema:
                 curv.accumulate_into(group['acc_curv'], weight)
 
+    def _end_accumulation(self):
+        """The hooks store their factors again (the accumulators keep what they hold)."""
+        for group in self.param_groups:
+            curv = group['curv']
+            if curv is not None and curv.kind == 'kron':
+                curv.accumulate_into(None, 0.)
+
     def _accumulate(self, weight):
         """Adds weight * (current gradients, current curvature data) of every group to the
         group's accumulators (reference: secondorder.py:175-182, vi.py:211-220)."""

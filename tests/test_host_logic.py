@@ -325,6 +325,42 @@ def test_accumulation_steps_average_gradients_and_factors(oracle_ops):
     assert torch.allclose(opt.param_groups[0]['curv'].ema[0], 0.5 * (A0 + A1), atol=1e-6)
 
 
+def test_vi_forward_pass_between_micro_steps_leaves_the_accumulators_alone(oracle_ops):
+    """acc_steps = 2: a prediction() (or any forward pass) between the two micro-steps must
+    not add its input factor to the accumulated curvature; the reference only adds curv.data
+    inside its MC loop (vi.py:211-220)."""
+    def run(predict_between, fail_first=False):
+        torch.manual_seed(0)
+        model = nn.Sequential(nn.Linear(4, 3))
+        xs = [torch.randn(5, 4) for _ in range(3)]
+        ys = [torch.randint(0, 3, (5,)) for _ in range(2)]
+        opt = torchsso.optim.VIOptimizer(model, 100, 'Cov', {'Linear': 'Kron'},
+                                         {'damping': 1e-2, 'ema_decay': 1.}, num_mc_samples=2,
+                                         prior_variance=0, acc_steps=2)
+        if fail_first:
+            def broken():
+                model(xs[2])
+                raise RuntimeError('closure failed')
+            with pytest.raises(RuntimeError):
+                opt.step(closure=broken)
+            curv = opt.param_groups[0]['curv']
+            assert curv._acc_into is None
+            model(xs[2])               # a pass after the failure is not accumulated either
+            return None
+        opt.step(closure=_closure(model, xs[0], ys[0]))
+        assert opt.optim_state == {'step': 0, 'acc_step': 1}
+        if predict_between:
+            opt.prediction(xs[2])
+            model(xs[2])
+        opt.step(closure=_closure(model, xs[1], ys[1]))
+        assert opt.optim_state == {'step': 1, 'acc_step': 0}
+        return [e.clone() for e in opt.param_groups[0]['curv'].ema]
+    plain, disturbed = run(False), run(True)
+    for a, b in zip(plain, disturbed):
+        assert torch.equal(a, b)
+    run(False, fail_first=True)
+
+
 def test_checkpoint_is_tensor_only_and_resumes_exactly(oracle_ops, tmp_path):
     import copy
     gold = T.load_golden('ref_convnet_kfac')

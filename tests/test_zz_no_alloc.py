@@ -66,6 +66,46 @@ def test_static_scratch_inverse_equals_workspace_inverse_twice_in_a_row():
             assert err < 1e-4, (m.shape[0], err)
 
 
+def test_static_scratch_calls_on_two_streams_are_put_in_order():
+    """Two calls on two streams share the one array: the library makes the second wait for
+    the first (an event per device), so both give the bits of the workspace entry point."""
+    lib = _hip.load()
+    dev = torch.device('cuda:0')
+    gen = torch.Generator().manual_seed(11)
+    lists = [[_spd(n, gen, dev) for n in (900, 130)], [_spd(n, gen, dev) for n in (640, 257, 5)]]
+    streams = [torch.cuda.Stream(device=dev), torch.cuda.Stream(device=dev)]
+    keep, got, want = [], [], []
+    torch.cuda.synchronize()
+    for rep in range(3):
+        for mats, st in zip(lists, streams):
+            dims = _hip.int_array([m.shape[0] for m in mats])
+            damp = _hip.f32_array([1e-3] * len(mats))
+            outs = [torch.full_like(m, float('nan')) for m in mats]
+            info = torch.full((len(mats),), -1, dtype=torch.int32, device=dev)
+            src, dst = _hip.ptr_array(mats, 'matrix'), _hip.ptr_array(outs, 'out')
+            keep.append((dims, damp, src, dst, info))
+            # (the tensors were made on the default stream, idle since the synchronisation)
+            assert lib.kfac_damped_inverse_batched_static(len(mats), dims, src, damp, dst,
+                                                          info.data_ptr(), st.cuda_stream) == 0
+            got.append(outs)
+    torch.cuda.synchronize()
+    for mats in lists:
+        dims = _hip.int_array([m.shape[0] for m in mats])
+        damp = _hip.f32_array([1e-3] * len(mats))
+        outs = [torch.empty_like(m) for m in mats]
+        info = torch.zeros(len(mats), dtype=torch.int32, device=dev)
+        need = lib.kfac_inverse_workspace_bytes(len(mats), dims)
+        ws = torch.empty(need, dtype=torch.uint8, device=dev)
+        assert lib.kfac_damped_inverse_batched(len(mats), dims, _hip.ptr_array(mats, 'matrix'), damp,
+                                               _hip.ptr_array(outs, 'out'), info.data_ptr(),
+                                               ws.data_ptr(), need, _hip.stream_ptr(dev)) == 0
+        want.append(outs)
+    torch.cuda.synchronize()
+    for i, outs in enumerate(got):
+        for w, g in zip(want[i % 2], outs):
+            assert torch.equal(w, g), 'call %d on stream %d differs' % (i, i % 2)
+
+
 def test_static_scratch_rejects_what_does_not_fit():
     lib = _hip.load()
     dev = torch.device('cuda:0')
