@@ -3,7 +3,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
                     [--workload resnet50|alexnet_fc|convnet|mlp|noisy_kfac|resnet50_train]
                     [--factor-mode grouped|eager] [--factor-streams N] [--factor-flush-work W]
-                    [--explicit-inverse] [--no-cpu-baseline] [--copy-calibration]
+                    [--explicit-inverse] [--no-cpu-baseline] [--no-other-workloads]
+                    [--copy-calibration]
 
 A "step" is one pass of the K-FAC hot path over one batch of synthetic input,
 driven through the public torchsso API: for every layer the two Kronecker
@@ -253,6 +254,32 @@ def factor_executed_flops(specs, batch):
     return total
 
 
+def inverse_precondition_executed_flops(specs, batch):
+    """(inversion, preconditioning) fp32 MFMA flops executed per step, from the library's
+    plan queries: whole 128 x 128 tiles; factors kept as the triangular factor of their
+    inverse (KronCurvature.factored_inverse_min_dim) skip the Y Y^T third of the inversion
+    and are applied as two triangular products."""
+    from torchsso import _hip
+    from torchsso.curv.curvature import KronCurvature
+    lib = _hip.load()
+    min_dim = KronCurvature.factored_inverse_min_dim
+    fact = (lambda d: 0) if min_dim is None else (lambda d: int(d >= min_dim))
+    dims, dG, dA = [], [], []
+    for s in specs:
+        if s['kind'] == 'bn':
+            continue
+        a, g, _ = spec_dims(s, batch)
+        dims += [a, g]
+        dA.append(a)
+        dG.append(g)
+    inv = lib.kfac_inverse_executed_flops(len(dims), _hip.int_array(dims),
+                                          _hip.int_array([fact(d) for d in dims]))
+    pre = lib.kfac_precondition_executed_flops(len(dG), _hip.int_array(dG), _hip.int_array(dA),
+                                               _hip.int_array([fact(d) for d in dG]),
+                                               _hip.int_array([fact(d) for d in dA]))
+    return inv, pre
+
+
 # ---------------------------------------------------------------------------
 # GPU side
 # ---------------------------------------------------------------------------
@@ -415,15 +442,67 @@ def time_steps(step, steps, warmup):
     return max(wall_ms, ev_ms), ev_ms, host_ms
 
 
-def run_gpu(args, specs, batch):
+def run_gpu(specs, batch, steps, warmup):
     import torch
     dev = torch.device('cuda:0')
     ls = LayerSet(specs, batch, dev)
-    ms, ev_ms, host_ms = time_steps(ls.step, args.steps, args.warmup)
-    phases = ls.timed_phases(max(2, min(args.steps, 5)))
+    ms, ev_ms, host_ms = time_steps(ls.step, steps, warmup)
+    phases = ls.timed_phases(max(2, min(steps, 5)))
     infos = [c.info for c in ls.curvs if c.kind == 'kron']
     not_spd = int(sum(int((i != 0).sum().item()) for i in infos))
-    return ms, ev_ms, host_ms, phases, ls.bytes_resident(), not_spd
+    resident = ls.bytes_resident()
+    del ls
+    torch.cuda.empty_cache()
+    return ms, ev_ms, host_ms, phases, resident, not_spd
+
+
+PEAK_HBM_TBS = 8.0
+
+
+def phase_records(work, executed, phases):
+    """Per phase of a step: algorithmic and executed work over the phase's HIP-event time.
+    MFMA phases in TFLOP/s against the fp32 matrix peak, HBM-bound tails in TB/s against
+    8 TB/s (algorithmic bytes: BatchNorm 8*n*c*h*w, update 20*|p|, running average
+    12*d^2 where a separate launch does it)."""
+    f_ms, bn_ms, ema_ms, inv_ms, pre_ms, upd_ms = phases
+    mfma = {}
+    for name, key, t in (('factor', 'factor', f_ms), ('invert', 'inverse', inv_ms),
+                         ('precondition', 'precondition', pre_ms)):
+        alg, exe = work[key], executed[key]
+        mfma[name] = {'ms': round(t, 4), 'algorithmic_gflop': round(alg / 1e9, 1),
+                      'executed_gflop': round(exe / 1e9, 1),
+                      'algorithmic_tflops': round(alg / t / 1e9, 2),
+                      'executed_tflops': round(exe / t / 1e9, 2),
+                      'executed_frac': round(exe / t / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)}
+    hbm = {}
+    for name, nbytes, t in (('batchnorm_diag', work['bn_bytes'], bn_ms),
+                            ('update', work['update_bytes'], upd_ms),
+                            ('ema', work['ema_bytes'], ema_ms)):
+        if nbytes <= 0 or t < 0.02:
+            # (with acc_steps == 1 the factor products write the running averages themselves
+            # and the `ema` phase is a buffer swap: nothing to price)
+            continue
+        hbm[name] = {'ms': round(t, 4), 'algorithmic_GB': round(nbytes / 1e9, 3),
+                     'TB_per_s': round(nbytes / t / 1e9, 3),
+                     'frac': round(nbytes / t / 1e9 / PEAK_HBM_TBS, 4)}
+    return mfma, hbm
+
+
+def layerset_summary(workload, steps, warmup):
+    """One LayerSet workload, timed like the headline one: step ms and the phases."""
+    make, batch, label = WORKLOADS[workload]
+    specs = make()
+    if workload == 'alexnet_fc':
+        for s in specs:
+            s['relu_input'] = True
+    work = algorithmic_work(specs, batch)
+    inv_x, pre_x = inverse_precondition_executed_flops(specs, batch)
+    executed = {'factor': factor_executed_flops(specs, batch), 'inverse': inv_x, 'precondition': pre_x}
+    ms, ev_ms, host_ms, phases, resident, not_spd = run_gpu(specs, batch, steps, warmup)
+    mfma, hbm = phase_records(work, executed, phases)
+    return {'workload': label, 'ms_per_step': round(ms, 4), 'steps': steps, 'warmup': warmup,
+            'host_enqueue_ms': round(host_ms, 4), 'not_spd_factors': not_spd,
+            'phases': mfma, 'hbm': hbm}
 
 
 # ---------------------------------------------------------------------------
@@ -761,6 +840,9 @@ def main():
                     help='grouped mode: multiply-adds of queued products from which the queue runs '
                          'without waiting for a reader (library default: 2.5e11); "none": never')
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--no-other-workloads', action='store_true',
+                    help='resnet50 only: leave out the short runs of the other BASELINE '
+                         'configurations that the line carries in `other_workloads`')
     ap.add_argument('--factored-min-dim', type=int, default=None,
                     help='rows from which update_inv keeps an inverse as its triangular factor '
                          '(library default: KronCurvature.factored_inverse_min_dim)')
@@ -827,8 +909,12 @@ def main():
             s['relu_input'] = True
     work = algorithmic_work(specs, batch)
     executed = factor_executed_flops(specs, batch)
+    inv_x, pre_x = inverse_precondition_executed_flops(specs, batch)
+    mfma_phases, hbm_phases = None, None
 
-    ms, ev_ms, host_ms, phases, resident, not_spd = run_gpu(args, specs, batch)
+    ms, ev_ms, host_ms, phases, resident, not_spd = run_gpu(specs, batch, args.steps, args.warmup)
+    mfma_phases, hbm_phases = phase_records(
+        work, {'factor': executed, 'inverse': inv_x, 'precondition': pre_x}, phases)
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device='cuda:0').normal_()
         dst = torch.empty_like(src)
@@ -856,6 +942,9 @@ def main():
                       'ema': round(ema_ms, 4),
                       'invert': round(inv_ms, 4), 'precondition': round(pre_ms, 4),
                       'update': round(upd_ms, 4)},
+        # algorithmic flops (dense convention: 2*d^2*L per factor, n^3 per inverse,
+        # 2*dG*dA*(dG+dA) per layer) over the phase time; what the matrix cores execute is in
+        # roofline.phases
         'phases_tflops': {'factor': round(work['factor'] / f_ms / 1e9, 2),
                           'invert': round(work['inverse'] / inv_ms / 1e9, 2),
                           'precondition': round(work['precondition'] / pre_ms / 1e9, 2)},
@@ -875,7 +964,12 @@ def main():
                              'derived from the library\'s tile / split plan',
                      'executed_gflop': round(executed / 1e9, 1),
                      'executed_tflops': round(executed / f_ms / 1e9, 2),
-                     'executed_frac': round(executed / f_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)},
+                     'executed_frac': round(executed / f_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4),
+                     # every MFMA phase and every HBM-bound tail of the step, each over its
+                     # own HIP-event time: algorithmic and executed work (executed: the
+                     # library's tile plans; the inversion forms no Y Y^T for the factors it
+                     # keeps in triangular form, so it executes less than n^3)
+                     'phases': mfma_phases, 'hbm': hbm_phases},
     }
     if args.workload == 'resnet50':
         pmc = read_pmc_summary()
@@ -883,6 +977,9 @@ def main():
         if seen and abs(executed - seen) <= 0.03 * seen:
             out['roofline']['traffic'] = pmc.get('traffic_bytes_per_launch')
             out['roofline']['executed_gflop_pmc'] = round(seen / 1e9, 1)
+            # (counter runs cannot be made from inside this script: both figures are read
+            # from the summary of the rocprofv3 --pmc runs, not measured in this run)
+            out['roofline']['traffic_source'] = os.path.relpath(PMC_SUMMARY, ROOT)
         else:
             msg = ('the factor plan executes %.1f GFLOP per step but the counter summary %s was '
                    'taken at %s: the plan changed since, traffic and the PMC cross-check are '
@@ -891,6 +988,17 @@ def main():
                       'no reading' if not seen else '%.1f GFLOP' % (seen / 1e9)))
             print('bench.py: WARNING: ' + msg, file=sys.stderr)
             out['roofline']['pmc_check'] = 'STALE: ' + msg
+    if args.workload == 'resnet50' and not args.no_other_workloads:
+        # the other BASELINE configurations, timed in this same run (fewer steps): parity-test
+        # cases, not the headline
+        others = [layerset_summary(w, 10, 3) for w in ('mlp', 'convnet', 'alexnet_fc')]
+        oargs = argparse.Namespace(steps=10, warmup=3)
+        nk = run_noisy_kfac(oargs)
+        others.append({'workload': nk['config']['workload'], 'ms_per_step': nk['value'],
+                       'steps': 10, 'warmup': 3, 'host_enqueue_ms': nk['host_enqueue_ms'],
+                       'not_spd_factors': nk['not_spd_factors'], 'phases_ms': nk['phases_ms'],
+                       'step_includes': nk['config']['step_includes']})
+        out['other_workloads'] = others
     if not args.no_cpu_baseline:
         cpu_ms, cores, threads, sample = run_cpu_baseline(specs, batch)
         out['cpu_baseline'] = {'value': round(cpu_ms, 1), 'unit': 'ms', 'cores': cores,

@@ -156,6 +156,12 @@ double kfac_factor_grouped_executed_flops(int count, const kfac_factor_job* jobs
  * n x n buffer per matrix.  `dims` is a HOST array of `count` sizes. */
 size_t kfac_inverse_workspace_bytes(int count, const int* dims);
 
+/* Plan query: the fp32 MFMA flops the batched inversion executes for matrices of these
+ * sizes (HOST arrays): blocked Cholesky (diagonal blocks, row panels, trailing updates
+ * with whole diagonal tiles), the triangular inverse, and Y Y^T for the matrices whose
+ * explicit inverse is formed (factored[i] == 0, or factored == NULL). */
+double kfac_inverse_executed_flops(int count, const int* dims, const int* factored);
+
 /* For every layer l:  pi = sqrt((tr A/dA) / (tr G/dG)), r = sqrt(damping[l]),
  *   Ainv = (A + r*pi*I)^-1 ,  Ginv = (G + (r/pi)*I)^-1 .
  * The traces, pi and the diagonal shift are computed on the device and the
@@ -254,6 +260,13 @@ int kfac_cholesky_upper_batched(int count, const int* dims, const float* const* 
 
 /* Scratch for the two routines below (dG, dA: HOST arrays). */
 size_t kfac_precondition_workspace_bytes(int layers, const int* dG, const int* dA);
+
+/* Plan query: the fp32 MFMA flops the preconditioning of these layers executes (HOST
+ * arrays; a NULL flag array: no side is given by its triangular factor): whole 128 x 128
+ * tiles; a triangular operand is applied twice, each time over the non-zero part of the
+ * reduction (the diagonal tiles' zero half included). */
+double kfac_precondition_executed_flops(int layers, const int* dG, const int* dA,
+                                        const int* g_factored, const int* a_factored);
 
 /* For every layer:  [gradW | gradb] <- Ginv * [gradW | gradb] * Ainv, in place.
  * gradW is [dG, dA - 1] when gradb[l] != NULL (dA counts the bias column,

@@ -1241,6 +1241,35 @@ int kfac_damped_inverse_batched_static(int count, const int* dims, const float* 
   return status;
 }
 
+double kfac_inverse_executed_flops(int count, const int* dims, const int* factored) {
+  if (count <= 0 || !dims) return 0.;
+  const double B = 2. * DB * DB * DB;       // one 128-deep step of a 128 x 128 tile
+  // diagonal block: per strip 4 waves x 15 rank-2 steps x 2 blocks, the updates by finished
+  // strips (12 + 8 blocks, 32 deep), the pending panel (10 blocks, 128 deep)
+  const double diag = 4096. * (4 * 120 + 20 * 16 + 10 * 64);
+  double total = 0.;
+  for (int i = 0; i < count; ++i) {
+    const double T = cdiv(dims[i], DB);
+    // Cholesky: row panels, trailing updates (whole diagonal tiles)
+    total += T * diag + B * (T * (T - 1) / 2 + (T - 1) * T * (T + 1) / 6);
+    // triangular inverse: per merge of r x c blocks, W tiles reduce over 1..c blocks,
+    // Y tiles over r..1
+    const int Ti = (int)T;
+    int D = 0;
+    while ((1 << D) < Ti) ++D;
+    for (int depth = 0; depth < D; ++depth)
+      for (int P = 0; P < (1 << depth); ++P) {
+        const Segment sg = segment(P, depth, Ti);
+        const double r = sg.mid - sg.p0, c = sg.p1 - sg.mid;
+        total += B * (r * c * (c + 1) / 2 + c * r * (r + 1) / 2);
+      }
+    // Y Y^T where the explicit inverse is formed: tile (bi <= bj) reduces over T - bj blocks
+    if (!(factored && factored[i]))
+      for (int bj = 0; bj < Ti; ++bj) total += B * (bj + 1.) * (T - bj);
+  }
+  return total;
+}
+
 size_t kfac_inverse_workspace_bytes(int count, const int* dims) {
   if (count <= 0 || !dims) return 0;
   std::vector<int> d(dims, dims + count);

@@ -516,6 +516,21 @@ using namespace kfac;
 
 extern "C" {
 
+double kfac_precondition_executed_flops(int layers, const int* dG, const int* dA,
+                                        const int* g_factored, const int* a_factored) {
+  if (layers <= 0 || !dG || !dA) return 0.;
+  double blocks = 0.;      // 128-deep steps of 128 x 128 tiles
+  for (int l = 0; l < layers; ++l) {
+    const double ta = cdiv(dA[l], BN), tg = cdiv(dG[l], BM);
+    const bool gfac = g_factored && g_factored[l], afac = a_factored && a_factored[l];
+    // a dense operand: every tile reduces over all blocks of that side; a triangular one:
+    // over 1..t blocks, twice (the factor and its transpose)
+    blocks += gfac ? 2 * ta * tg * (tg + 1) / 2 : ta * tg * tg;
+    blocks += afac ? 2 * tg * ta * (ta + 1) / 2 : tg * ta * ta;
+  }
+  return blocks * 2. * BM * BN * 128.;
+}
+
 size_t kfac_precondition_workspace_bytes(int layers, const int* dG, const int* dA) {
   if (layers <= 0 || !dG || !dA) return 0;
   return precond_workspace(layers, dG, dA, false);

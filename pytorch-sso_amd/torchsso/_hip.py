@@ -61,6 +61,8 @@ _SIGNATURES = {
                                    c_ptr, c_size, c_ptr]),
     'kfac_factor_grouped_workspace_bytes': (c_size, [c_int, c_ptr]),
     'kfac_factor_grouped_executed_flops': (ctypes.c_double, [c_int, c_ptr]),
+    'kfac_inverse_executed_flops': (ctypes.c_double, [c_int, c_ptr, c_ptr]),
+    'kfac_precondition_executed_flops': (ctypes.c_double, [c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     'kfac_factor_grouped': (c_int, [c_int, c_ptr, c_ptr, c_size, c_ptr]),
     'kfac_inverse_workspace_bytes': (c_size, [c_int, c_ptr]),
     'kfac_pi_damped_inverse_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
