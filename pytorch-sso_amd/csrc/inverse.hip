@@ -311,22 +311,23 @@ __device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, f
     }
   }
   __syncthreads();
-  if (pending) {
-    // S -= W^T W, W = tile (p-1, p) of U (in Z for now): the ten 32x32 blocks on and above
-    // the diagonal, one per wave, 128 deep
-    if (wave < 10) {
-      int bi, bj;
-      upper_tile(wave, 4, bi, bj);
-      const v16f acc = lds_mma32(Z + 32 * bi, DLD, 1, Z + 32 * bj, DLD, 1, DB);
-      lds_f* const c = S + (32 * bi + 4 * h) * DLD + 32 * bj + r;
-      float old[16];
+  // S -= W^T W, W = tile (p-1, p) of U (in Z for now), 128 deep, by 32x32 blocks: the four
+  // blocks of the first strip's rows now (waves 4-7, one per SIMD), the other six while
+  // that strip is eliminated (it writes Z in the columns of its own block only, which
+  // those six do not read; later strips find W spent)
+  auto pending_block = [&](int blk) {
+    int bi, bj;
+    upper_tile(blk, 4, bi, bj);
+    const v16f acc = lds_mma32(Z + 32 * bi, DLD, 1, Z + 32 * bj, DLD, 1, DB);
+    lds_f* const c = S + (32 * bi + 4 * h) * DLD + 32 * bj + r;
+    float old[16];
 #pragma unroll
-      for (int e = 0; e < 16; ++e) old[e] = c[(8 * (e >> 2) + (e & 3)) * DLD];
+    for (int e = 0; e < 16; ++e) old[e] = c[(8 * (e >> 2) + (e & 3)) * DLD];
 #pragma unroll
-      for (int e = 0; e < 16; ++e) c[(8 * (e >> 2) + (e & 3)) * DLD] = old[e] - acc[e];
-    }
-    // (the loop over the strips starts with a barrier; nothing there reads Z before writing it)
-  }
+    for (int e = 0; e < 16; ++e) c[(8 * (e >> 2) + (e & 3)) * DLD] = old[e] - acc[e];
+  };
+  if (pending && wave >= 4 && wave < 8) pending_block(wave - 4);
+  // (the loop over the strips starts with a barrier)
 
   typedef __attribute__((address_space(1))) float global_f;
   global_f* const gU = (global_f*)(m.U + (size_t)r0 * n + r0);
@@ -405,12 +406,12 @@ __device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, f
 #pragma unroll
           for (int e = 0; e < 16; ++e) P[e] = 8 * (e >> 2) + 4 * h + (e & 3) == r ? 1.f : 0.f;
         }
-        // (block (0, 3) of Z, above its diagonal, is never used; the lane's column made
+        // (block (3, 0) of S, below its diagonal, is never used; the lane's column made
         // opaque per strip, so that the lane masks derived from it are computed where they
         // are used instead of being kept, and spilled, across the loop over the strips)
         int rr = r;
         asm volatile("" : "+v"(rr));
-        lds_f* const leaf_rows = (wave == 0 ? S + c0 * DLD + c0 : Z + 96) + h * DLD + r;
+        lds_f* const leaf_rows = (wave == 0 ? S + c0 * DLD + c0 : S + 96 * DLD) + h * DLD + r;
         lds_f* const blk_rows = (panel ? S + c0 * DLD + 32 * jb : Z + c0 * DLD + 32 * s) + h * DLD + r;
         float pmin = 1.f, piv[32];
         // every wave has its copy of the leaf in registers before wave 0 writes U_qq over it
@@ -433,6 +434,7 @@ __device__ __forceinline__ void diag_block(const MatDesc& m, int p, int* info, f
     } else {
       __syncthreads();
       // meanwhile: the strip above's update of the rows further down, and its rows to memory
+      if (q == 0 && pending && wave < 10) pending_block(wave);      // blocks 4..9
       if (q > 0) {
       int first = 0;
       for (int i = q + 1; i < nq; ++i) first += update_row(q - 1, i, first, 8);

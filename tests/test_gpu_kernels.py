@@ -500,7 +500,7 @@ def test_large_inverse_at_benchmark_sizes(ops, dev):
         outs, info = ops.damped_inverse_batched([X], [damp])
         assert info.cpu().tolist() == [0]
         Xd = X.double()
-        _, err, err_ref, _ = inverse_record('random rank-%d factor' % L, Xd, damp, outs[0])
+        _, err, err_ref, _, _ = inverse_record('random rank-%d factor' % L, Xd, damp, outs[0])
         Xd.diagonal().add_(damp)
         Y = outs[0].double()
         R = torch.eye(n, device=dev, dtype=D) - Xd @ Y

@@ -108,7 +108,7 @@ def test_resnet50_step_on_real_activations():
         r = 1e-3 ** 0.5
         for tag, X, shift, Y in (('A', eA, r * pi, curv.inv[0]), ('G', eG, r / pi, curv.inv[1])):
             key = '%s %s inverse' % (name, tag)
-            _, e_dev, e_ref, _ = inverse_record(key, X, shift.item(), Y)
+            _, e_dev, e_ref, _, _ = inverse_record(key, X, shift.item(), Y)
             worst[key] = e_dev
             bounds[key] = max(TOL, 1.5 * e_ref)
         V = raw[i][0].reshape(raw[i][0].shape[0], -1).double()
