@@ -422,6 +422,17 @@ int kfac_bn_diag_cov(const float* g, int n, int channels, int len, const float* 
                      float* w_curv, float* b_curv, void* workspace, size_t workspace_bytes,
                      void* stream);
 
+/* kfac_bn_diag_cov for the BatchNorm layers of a whole backward pass in ONE launch (HOST arrays
+ * of length `count`; b_curv may be NULL, or hold NULLs): a workgroup takes one channel of
+ * one layer, so the small layers at the end of a network (a few MB each, a launch of their
+ * own lasts as long as its latency) share the chip with the large ones.  Same formulas,
+ * cov/batchnorm.py:38-49 with the rescale of curvature.py:154-158; n[i] <= 2048. */
+size_t kfac_bn_diag_cov_batched_workspace_bytes(int count);
+int kfac_bn_diag_cov_batched(int count, const float* const* g, const int* n, const int* channels,
+                             const int* len, const float* const* sx, const float* alpha,
+                             float* const* w_curv, float* const* b_curv, void* workspace,
+                             size_t workspace_bytes, void* stream);
+
 /* ---- Wire format: triangular packing ------------------------------------ */
 
 /* The reference ships factors between ranks as one flat fp32 buffer: arrays back

@@ -365,15 +365,36 @@ __global__ __launch_bounds__(256) void bn_combine_kernel(const float* sx, const 
 // (no per-row index arithmetic, few shuffles).
 constexpr int BN_MAX_ROWS = 2048;      // samples per workgroup
 
+// The sums over n of one channel, from its row sums in LDS (all threads of the workgroup
+// call this; `prod`: BN_MAX_ROWS floats of LDS)
+__device__ __forceinline__ void bn_finish_channel(const float* rowsum, float* prod,
+                                                  const float* sx, int N, int C, int c,
+                                                  float alpha, float* w_curv, float* b_curv) {
+  __syncthreads();
+  // sx[n][c] * rowsum[n] by all threads, then one thread adds over n in order
+  for (int q = threadIdx.x; q < N; q += 256) prod[q] = sx[(long)q * C + c] * rowsum[q];
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float sw = 0.f, sb = 0.f;
+#pragma unroll 8
+    for (int n = 0; n < N; ++n) {
+      sw += prod[n];
+      sb += rowsum[n];
+    }
+    w_curv[c] = alpha * sw;
+    if (b_curv) b_curv[c] = alpha * sb;
+  }
+}
+
+// (channel c; `rowsum`, `prod`: BN_MAX_ROWS floats of LDS each, used with COMBINE)
 template <int CHUNKS, bool VEC, bool COMBINE>
-__global__ __launch_bounds__(256) void bn_rows_kernel(const float* x, const float* scale,
-                                                      const float* shift, int N, int C, int len,
-                                                      const float* sx, float alpha, float* out,
-                                                      float* w_curv, float* b_curv) {
+__device__ __forceinline__ void bn_rows_body(const float* x, const float* scale,
+                                             const float* shift, int N, int C, int len,
+                                             const float* sx, float alpha, float* out,
+                                             float* w_curv, float* b_curv, int c, float* rowsum,
+                                             float* prod) {
   constexpr int UNROLL = CHUNKS == 4 ? 4 : 8;      // rows in flight per wave
-  __shared__ float rowsum[COMBINE ? BN_MAX_ROWS : 1];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int c = blockIdx.x;
   const int units = VEC ? len >> 2 : len;          // loads per row
   const float sh = shift ? shift[c] : 0.f;
   const float rs = scale ? 1.f / scale[c] : 1.f;
@@ -436,23 +457,90 @@ __global__ __launch_bounds__(256) void bn_rows_kernel(const float* x, const floa
         out[(long)q * C + c] = r;
     }
   }
-  if (COMBINE) {
-    __shared__ float prod[BN_MAX_ROWS];
-    __syncthreads();
-    // sx[n][c] * rowsum[n] by all threads, then one thread adds over n in order
-    for (int q = threadIdx.x; q < N; q += 256) prod[q] = sx[(long)q * C + c] * rowsum[q];
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      float sw = 0.f, sb = 0.f;
-#pragma unroll 8
-      for (int n = 0; n < N; ++n) {
-        sw += prod[n];
-        sb += rowsum[n];
-      }
-      w_curv[c] = alpha * sw;
-      if (b_curv) b_curv[c] = alpha * sb;
-    }
+  if (COMBINE) bn_finish_channel(rowsum, prod, sx, N, C, c, alpha, w_curv, b_curv);
+}
+
+template <int CHUNKS, bool VEC, bool COMBINE>
+__global__ __launch_bounds__(256) void bn_rows_kernel(const float* x, const float* scale,
+                                                      const float* shift, int N, int C, int len,
+                                                      const float* sx, float alpha, float* out,
+                                                      float* w_curv, float* b_curv) {
+  __shared__ float rowsum[COMBINE ? BN_MAX_ROWS : 1];
+  __shared__ float prod[COMBINE ? BN_MAX_ROWS : 1];
+  bn_rows_body<CHUNKS, VEC, COMBINE>(x, scale, shift, N, C, len, sx, alpha, out, w_curv, b_curv,
+                                     (int)blockIdx.x, rowsum, prod);
+}
+
+// The backward half of the BatchNorm curvature for MANY layers in one launch: a workgroup
+// takes one channel of one layer (found by binary search in the table of first items; the
+// layers with the longest rows first).  Rows of up to 1024 elements run the code of
+// bn_rows_kernel; longer rows are walked by one wave per sample, 8 loads in flight per lane.
+struct BnJob {
+  const float* g;
+  const float* sx;
+  float* w_curv;
+  float* b_curv;
+  int N, C, len, variant;       // variant: 2 * log2(chunks) + vec for short rows, 6: long rows
+  float alpha;
+  int pad;
+};
+constexpr int BN_LONG = 6;
+
+__global__ __launch_bounds__(256) void bn_grouped_kernel(const BnJob* __restrict__ jobs,
+                                                         const int* __restrict__ cum, int njobs) {
+  __shared__ float rowsum[BN_MAX_ROWS];
+  __shared__ float prod[BN_MAX_ROWS];
+  int lo = 0, hi = njobs;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cum[mid] <= (int)blockIdx.x) lo = mid; else hi = mid;
   }
+  const BnJob jb = jobs[lo];
+  const int c = (int)blockIdx.x - cum[lo];
+#define KFAC_BN_BODY(CH, V)                                                                   \
+  bn_rows_body<CH, V, true>(jb.g, nullptr, nullptr, jb.N, jb.C, jb.len, jb.sx, jb.alpha, nullptr, \
+                            jb.w_curv, jb.b_curv, c, rowsum, prod)
+  switch (jb.variant) {
+    case 0: KFAC_BN_BODY(1, false); return;
+    case 1: KFAC_BN_BODY(1, true); return;
+    case 2: KFAC_BN_BODY(2, false); return;
+    case 3: KFAC_BN_BODY(2, true); return;
+    case 4: KFAC_BN_BODY(4, false); return;
+    case 5: KFAC_BN_BODY(4, true); return;
+    default: break;
+  }
+#undef KFAC_BN_BODY
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int len = jb.len;
+  const bool vec = (len & 3) == 0 && ((uintptr_t)jb.g & 15) == 0;
+  for (int q = wave; q < jb.N; q += 4) {
+    const float* p = jb.g + ((long)q * jb.C + c) * len;
+    float s = 0.f;
+    if (vec) {
+      const float4* p4 = reinterpret_cast<const float4*>(p);
+      const int len4 = len >> 2;
+      for (int i = lane; i < len4; i += 64 * 8) {
+        float4 v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          v[k] = i + 64 * k < len4 ? p4[i + 64 * k] : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) s += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+      }
+    } else {
+      for (int i = lane; i < len; i += 64 * 8) {
+        float v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = i + 64 * k < len ? p[i + 64 * k] : 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) s += v[k] * v[k];
+      }
+    }
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) s += __shfl_xor(s, m);
+    if (lane == 0) rowsum[q] = s;
+  }
+  bn_finish_channel(rowsum, prod, jb.sx, jb.N, jb.C, c, jb.alpha, jb.w_curv, jb.b_curv);
 }
 
 // Launch of bn_rows_kernel when the shape suits it (false: the caller takes the
@@ -646,6 +734,58 @@ int kfac_bn_diag_cov(const float* g, int n, int channels, int len, const float* 
   launch_rowsq(g, (int64_t)n * channels, channels, len, nullptr, nullptr, sg, st);
   hipLaunchKernelGGL(bn_combine_kernel, dim3(cdiv(channels, 64)), dim3(256), 0, st, sx, sg, n,
                      channels, alpha, w_curv, b_curv);
+  return launch_status();
+}
+
+size_t kfac_bn_diag_cov_batched_workspace_bytes(int count) {
+  if (count <= 0) return 0;
+  return (((size_t)count * sizeof(BnJob) + 255) & ~(size_t)255) + ((size_t)count + 1) * sizeof(int);
+}
+
+int kfac_bn_diag_cov_batched(int count, const float* const* g, const int* n, const int* channels,
+                             const int* len, const float* const* sx, const float* alpha,
+                             float* const* w_curv, float* const* b_curv, void* workspace,
+                             size_t workspace_bytes, void* stream) {
+  if (count < 0 || (count > 0 && (!g || !n || !channels || !len || !sx || !alpha || !w_curv)))
+    return KFAC_ERR_ARG;
+  if (count == 0) return KFAC_OK;
+  if (!workspace || workspace_bytes < kfac_bn_diag_cov_batched_workspace_bytes(count))
+    return KFAC_ERR_WORKSPACE;
+  long items = 0;
+  for (int i = 0; i < count; ++i) {
+    if (!g[i] || !sx[i] || !w_curv[i] || n[i] <= 0 || n[i] > BN_MAX_ROWS || channels[i] <= 0 ||
+        len[i] <= 0 || (int64_t)n[i] * channels[i] >= (int64_t)1 << 31)
+      return KFAC_ERR_ARG;
+    items += channels[i];
+  }
+  if (items >= (long)1 << 31) return KFAC_ERR_ARG;
+  // the layers with the longest rows first: their workgroups last longest
+  std::vector<int> order(count);
+  for (int i = 0; i < count; ++i) order[i] = i;
+  std::stable_sort(order.begin(), order.end(), [&](int a, int b) {
+    return (long)len[a] * n[a] > (long)len[b] * n[b];
+  });
+  const size_t jobs_bytes = ((size_t)count * sizeof(BnJob) + 255) & ~(size_t)255;
+  std::vector<unsigned> words((jobs_bytes + ((size_t)count + 1) * sizeof(int)) / 4, 0u);
+  BnJob* jobs = (BnJob*)words.data();
+  int* cum = (int*)((char*)words.data() + jobs_bytes);
+  int at = 0;
+  for (int k = 0; k < count; ++k) {
+    const int i = order[k];
+    const bool vec = (len[i] & 3) == 0 && ((uintptr_t)g[i] & 15) == 0;
+    const int units = vec ? len[i] >> 2 : len[i];
+    const int variant = units > 256 ? BN_LONG
+                                    : 2 * (units <= 64 ? 0 : (units <= 128 ? 1 : 2)) + (vec ? 1 : 0);
+    jobs[k] = BnJob{g[i], sx[i], w_curv[i], b_curv ? b_curv[i] : nullptr, n[i], channels[i],
+                    len[i], variant, alpha[i], 0};
+    cum[k] = at;
+    at += channels[i];
+  }
+  cum[count] = at;
+  hipStream_t st = (hipStream_t)stream;
+  upload_table(words.data(), words.size() * 4, workspace, st);
+  hipLaunchKernelGGL(bn_grouped_kernel, dim3(at), dim3(256), 0, st, (const BnJob*)workspace,
+                     (const int*)((char*)workspace + jobs_bytes), count);
   return launch_status();
 }
 

@@ -116,6 +116,9 @@ _SIGNATURES = {
     'kfac_bn_diag_cov_workspace_bytes': (c_size, [c_int, c_int]),
     'kfac_bn_diag_cov': (c_int, [c_ptr, c_int, c_int, c_int, c_ptr, c_f32, c_ptr, c_ptr, c_ptr,
                                  c_size, c_ptr]),
+    'kfac_bn_diag_cov_batched_workspace_bytes': (c_size, [c_int]),
+    'kfac_bn_diag_cov_batched': (c_int, [c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
+                                         c_ptr, c_ptr, c_size, c_ptr]),
 }
 
 

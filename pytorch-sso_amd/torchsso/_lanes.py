@@ -42,17 +42,21 @@ _count = 2
 _mode = 'grouped'
 _lock = threading.Lock()
 _flush_work = 2.5e11
+# queued BatchNorm reductions run once the output gradients they keep alive reach this size
+_BN_FLUSH_BYTES = 4e8
 
 
 class _Queue(object):
     """Factor products of one device waiting for their engine call."""
-    __slots__ = ('keys', 'items', 'work', 'forward')
+    __slots__ = ('keys', 'items', 'work', 'forward', 'bn', 'bn_bytes')
 
     def __init__(self):
         self.keys = set()
         self.items = []      # (job, tensors kept alive, stream of the hook)
         self.work = 0.
         self.forward = False    # holds products queued by forward hooks
+        self.bn = []         # BatchNorm backward reductions: (job tuple, stream of the hook)
+        self.bn_bytes = 0    # output gradients those keep alive
 
 
 _deferred = {}     # device index -> _Queue
@@ -132,6 +136,32 @@ def defer(device, key, job, keep, work=0., backward=False):
         _run_deferred(idx)
 
 
+def defer_bn(device, key, job):
+    """Queues the backward half of a BatchNorm layer's diagonal curvature: `job` =
+    (grad_output, channels, sx, alpha, w, b) as `_ops.bn_diag_cov_batched` takes them (its
+    tensors stay referenced until the reduction has been enqueued).  All queued layers run
+    in ONE launch on the caller's stream when the queue runs.  A backward hook: the first
+    one of a pass runs what the forward hooks have queued."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    stream = torch.cuda.current_stream(device)
+    with _lock:
+        q = _deferred.get(idx)
+        if q is None:
+            q = _deferred[idx] = _Queue()
+        run_first = key in q.keys or q.forward
+    if run_first:
+        _run_deferred(idx)
+    with _lock:
+        q = _deferred[idx]
+        q.keys.add(key)
+        q.bn.append((job, stream))
+        q.bn_bytes += job[0].numel() * 4
+        full = q.bn_bytes >= _BN_FLUSH_BYTES
+    if full:
+        # (the reductions alone: the factor products keep waiting for their own trigger)
+        _run_deferred(idx, bn_only=True)
+
+
 def flush_if_queued(device, key):
     """Runs the queue of `device` if it holds a product for `key` (the caller is about to
     reuse that product's job object or output buffer)."""
@@ -146,20 +176,41 @@ def flush_if_queued(device, key):
 def deferred_count():
     """Products queued and not yet handed to the engine (all devices)."""
     with _lock:
-        return sum(len(q.items) for q in _deferred.values())
+        return sum(len(q.items) + len(q.bn) for q in _deferred.values())
 
 
-def _run_deferred(only=None):
+def _run_deferred(only=None, bn_only=False):
     from torchsso import _ops
     with _lock:
         todo = []
         for i, q in _deferred.items():
-            if q.items and (only is None or only == i):
-                todo.append((i, q.items))
+            if bn_only:
+                if q.bn and only == i:
+                    todo.append((i, [], q.bn))
+                    q.keys.difference_update(key for key in list(q.keys) if key[1] == 'bn')
+                    q.bn, q.bn_bytes = [], 0
+            elif (q.items or q.bn) and (only is None or only == i):
+                todo.append((i, q.items, q.bn))
                 _deferred[i] = _Queue()
-    for i, items in todo:
+    for i, items, bn in todo:
         device = torch.device('cuda', i)
         cur = torch.cuda.current_stream(i)
+        if bn:
+            # the BatchNorm reductions stay on the caller's stream (one launch for all queued
+            # layers): they are bound by memory and run beside the factor products of the
+            # side streams; whoever reads their outputs does so on this stream, behind them
+            waited = []
+            for job, st in bn:
+                if st != cur:
+                    if st not in waited:
+                        waited.append(st)
+                        cur.wait_stream(st)
+                    for t in (job[0], job[2]) + tuple(job[4:]):
+                        if t is not None:
+                            t.record_stream(cur)
+            _ops.bn_diag_cov_batched([job for job, _ in bn], device)
+        if not items:
+            continue
         side = None
         if _count > 0:
             # the engine call goes to a side stream (the calls of a pass take turns), so

@@ -619,6 +619,40 @@ def bn_diag_cov(grad_output, channels, sx, alpha, bias):
     return w, b
 
 
+BN_BATCH_MAX_ROWS = 2048     # samples per layer the batched BatchNorm call takes
+
+
+def bn_diag_cov_batched(jobs, device, stream=None):
+    """bn_diag_cov for a list of layers in one launch.  jobs: (grad_output, channels, sx,
+    alpha, w, b) with grad_output contiguous [n, c, ...], sx [n, c], and w, b (b may be
+    None) the [c] outputs, written in place."""
+    if not jobs:
+        return
+    lib = _hip.load()
+    gs, ns, cs, ls, sxs, alphas, ws_, bs = [], [], [], [], [], [], [], []
+    for g, channels, sx, alpha, w, b in jobs:
+        n = g.shape[0]
+        if g.shape[1] != channels or tuple(sx.shape) != (n, channels) or n > BN_BATCH_MAX_ROWS:
+            raise _hip.KfacHipError('bn_diag_cov_batched: grad_output %s, sums %s, %d channels'
+                                    % (tuple(g.shape), tuple(sx.shape), channels))
+        gs.append(g)
+        ns.append(n)
+        cs.append(channels)
+        ls.append(g.numel() // (n * channels))
+        sxs.append(sx)
+        alphas.append(alpha)
+        ws_.append(w)
+        bs.append(b)
+    count = len(jobs)
+    ws, ws_bytes = _hip.workspace(device, lib.kfac_bn_diag_cov_batched_workspace_bytes(count), stream)
+    st = lib.kfac_bn_diag_cov_batched(
+        count, _hip.ptr_array(gs, 'grad_output'), _hip.int_array(ns), _hip.int_array(cs),
+        _hip.int_array(ls), _hip.ptr_array(sxs, 'sx'), _hip.f32_array(alphas),
+        _hip.ptr_array(ws_, 'w_curv'), _hip.ptr_array(bs, 'b_curv', allow_none=True),
+        _ws_ptr(ws), ws_bytes, _hip.stream_ptr(device, stream))
+    _hip.check(st, 'kfac_bn_diag_cov_batched')
+
+
 def scale_rows(x, w, use_sqrt):
     """x[r] * (sqrt(w[r]) if use_sqrt else w[r]) for every row r = index along dim 0 (new tensor)."""
     lib = _hip.load()

@@ -7,9 +7,10 @@ x_hat = (out - bias) / weight is the normalised input (curvature.py:123-134).
 sum_hw x_hat^2 is reduced straight from the layer output in the forward hook
 (before an in-place activation can touch it) and x_hat itself is never stored.
 """
+import torch
 import torch.nn as nn
 
-from torchsso import _ops
+from torchsso import _lanes, _ops
 from torchsso.curv.curvature import Curvature, DiagCurvature
 
 
@@ -52,10 +53,43 @@ class _DiagCovBatchNorm(DiagCurvature):
         if output.requires_grad:
             output.register_hook(self._on_grad_output)
 
+    # In grouped mode the backward reduction is only queued by the hook (the output gradient
+    # stays referenced) and runs with those of the other BatchNorm layers in ONE launch when
+    # the queue runs (torchsso._lanes); whoever reads `data` first has it run.
+    _queued = False
+
+    @property
+    def data(self):
+        if self._queued:
+            self._queued = False
+            _lanes.join()
+        return self._data
+
+    @data.setter
+    def data(self, value):
+        if self._queued:            # (the queued reduction writes the tensors it was given)
+            self._queued = False
+            _lanes.join()
+        self._data = value
+
+    def adjust_data_scale(self, scale):
+        self.data                   # (runs a queued reduction first)
+        super(_DiagCovBatchNorm, self).adjust_data_scale(scale)
+
     def update_in_backward(self, grad_output):
         n = grad_output.shape[0]
-        w, b = _ops.bn_diag_cov(grad_output, self._module.num_features, self._sx, float(n),
-                                self.bias)                                # n^2 / n
+        channels = self._module.num_features
+        device = grad_output.device
+        if (_lanes.mode() == 'grouped' and device.type == 'cuda'
+                and n <= _ops.BN_BATCH_MAX_ROWS):
+            g = grad_output.contiguous()
+            w = torch.empty(channels, dtype=torch.float32, device=device)
+            b = torch.empty(channels, dtype=torch.float32, device=device) if self.bias else None
+            _lanes.defer_bn(device, (id(self), 'bn'), (g, channels, self._sx, float(n), w, b))
+            self._data = [w] if b is None else [w, b]
+            self._queued = True
+            return
+        w, b = _ops.bn_diag_cov(grad_output, channels, self._sx, float(n), self.bias)   # n^2 / n
         self._data = [w] if b is None else [w, b]
 
 

@@ -478,6 +478,39 @@ def test_batchnorm_diag(ops, dev, shape, bias):
     assert (bf is None) == (not bias)
 
 
+def test_batchnorm_diag_of_many_layers_in_one_launch(ops, dev):
+    """kfac_bn_diag_cov_batched: every row-length class in one call (1 element, rows with
+    and without float4 alignment in the three load counts, rows beyond 1024 elements), with
+    and without a bias output, against the float64 oracle; the short-row layers give the
+    bits of the single-layer call (same code), and a second call the same bits."""
+    torch.manual_seed(6)
+    shapes = [(6, 10, 5, 5), (4, 3, 1, 1), (8, 16, 56, 56), (16, 7), (32, 96, 7, 7),
+              (32, 130, 14, 14), (8, 70, 28, 28), (5, 33, 10, 13), (3, 300, 9, 9),
+              (7, 18, 16, 20), (2, 9, 33, 33), (40, 6, 2, 2), (4, 5, 112, 112), (3, 4, 41, 37)]
+    jobs, refs, singles = [], [], []
+    for k, shape in enumerate(shapes):
+        c, n, bias = shape[1], shape[0], k % 3 != 0
+        out = torch.randn(*shape)
+        w, b = torch.rand(c) + 0.5, torch.randn(c)
+        g = (torch.randn(*shape) * 1e-2).to(dev)
+        refs.append(O.bn_diag(O.bn_restore_input(out.double(), w.double(), b.double()), g.cpu(), bias, D))
+        sx = ops.rowsq_sum(out.to(dev), c, w.to(dev), b.to(dev))
+        wo = torch.full((c,), float('nan'), device=dev)
+        bo = torch.full((c,), float('nan'), device=dev) if bias else None
+        jobs.append((g, c, sx, float(n), wo, bo))
+        singles.append(ops.bn_diag_cov(g, c, sx, float(n), bias))
+    ops.bn_diag_cov_batched(jobs, dev)
+    first = [(j[4].clone(), None if j[5] is None else j[5].clone()) for j in jobs]
+    ops.bn_diag_cov_batched(jobs, dev)
+    for shape, job, ref, one, again in zip(shapes, jobs, refs, singles, first):
+        wo, bo = job[4], job[5]
+        assert O.rel_fro(wo, ref[0]) < TOL, shape
+        assert bo is None or O.rel_fro(bo, ref[1]) < TOL, shape
+        assert torch.equal(wo, again[0]) and (bo is None or torch.equal(bo, again[1])), shape
+        if job[0].numel() // (shape[0] * shape[1]) <= 256:
+            assert torch.equal(wo, one[0]) and (bo is None or torch.equal(bo, one[1])), shape
+
+
 # ---- size-independent properties at the benchmark's sizes ---------------------
 
 def test_large_inverse_at_benchmark_sizes(ops, dev):
