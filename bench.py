@@ -190,7 +190,7 @@ def spec_dims(s, batch):
 
 def algorithmic_work(specs, batch):
     """Flops of the dense formulation (what the reference's einsum / mm / potrf+potri do)."""
-    w = dict(factor=0., inverse=0., precondition=0., bn_bytes=0., ema_bytes=0., update_bytes=0.)
+    w = dict(factor=0., inverse=0., precondition=0., bn_bytes=0., update_bytes=0.)
     for s in specs:
         if s['kind'] == 'bn':
             w['bn_bytes'] += 8. * batch * s['c'] * s['h'] * s['h']
@@ -199,7 +199,6 @@ def algorithmic_work(specs, batch):
         w['factor'] += 2. * dA * dA * L + 2. * dG * dG * L
         w['inverse'] += float(dA) ** 3 + float(dG) ** 3
         w['precondition'] += 2. * dG * dG * dA + 2. * dG * dA * dA
-        w['ema_bytes'] += 12. * (dA * dA + dG * dG)
         w['update_bytes'] += 20. * dG * dA
     return w
 
@@ -462,8 +461,7 @@ PEAK_HBM_TBS = 8.0
 def phase_records(work, executed, phases):
     """Per phase of a step: algorithmic and executed work over the phase's HIP-event time.
     MFMA phases in TFLOP/s against the fp32 matrix peak, HBM-bound tails in TB/s against
-    8 TB/s (algorithmic bytes: BatchNorm 8*n*c*h*w, update 20*|p|, running average
-    12*d^2 where a separate launch does it)."""
+    8 TB/s (algorithmic bytes: BatchNorm 8*n*c*h*w, update 20*|p|)."""
     f_ms, bn_ms, ema_ms, inv_ms, pre_ms, upd_ms = phases
     mfma = {}
     for name, key, t in (('factor', 'factor', f_ms), ('invert', 'inverse', inv_ms),
@@ -475,12 +473,13 @@ def phase_records(work, executed, phases):
                       'executed_tflops': round(exe / t / 1e9, 2),
                       'executed_frac': round(exe / t / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)}
     hbm = {}
-    for name, nbytes, t in (('batchnorm_diag', work['bn_bytes'], bn_ms),
-                            ('update', work['update_bytes'], upd_ms),
-                            ('ema', work['ema_bytes'], ema_ms)):
+    # The factor products write the running averages of the Kronecker factors themselves
+    # (no accumulation steps here), so the `ema` phase holds no pass over the factors: what
+    # runs there is the tail of the BatchNorm work (the queued backward reductions not yet
+    # flushed and the running average of the diagonals), priced with BatchNorm.
+    for name, nbytes, t in (('batchnorm_diag', work['bn_bytes'], bn_ms + ema_ms),
+                            ('update', work['update_bytes'], upd_ms)):
         if nbytes <= 0 or t < 0.02:
-            # (with acc_steps == 1 the factor products write the running averages themselves
-            # and the `ema` phase is a buffer swap: nothing to price)
             continue
         hbm[name] = {'ms': round(t, 4), 'algorithmic_GB': round(nbytes / 1e9, 3),
                      'TB_per_s': round(nbytes / t / 1e9, 3),
