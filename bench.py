@@ -848,6 +848,10 @@ def main():
     ap.add_argument('--explicit-inverse', action='store_true',
                     help='form A^-1 and G^-1 explicitly in update_inv (as the reference does) '
                          'instead of keeping their triangular factors and applying those')
+    ap.add_argument('--one-curvature-stream', action='store_true',
+                    help='inversion and preconditioning of all layers on the caller\'s stream '
+                         '(default: the layers with small factors take theirs to a side stream '
+                         'beside the factorisation chain of the largest factors)')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run a plain 1 GiB device copy (reference for rocprofv3 --pmc '
                          'FETCH_SIZE / WRITE_SIZE readings)')
@@ -870,7 +874,10 @@ def main():
         torchsso.set_factor_flush_work(None if args.factor_flush_work == 'none'
                                        else float(args.factor_flush_work))
     factor_streams = torchsso.factor_streams()
+    from torchsso.curv import curvature as _curvature
     from torchsso.curv.curvature import KronCurvature
+    if args.one_curvature_stream:
+        _curvature.two_stream_min_dim = None
     if args.explicit_inverse:
         KronCurvature.factored_inverse_min_dim = None
     elif args.factored_min_dim is not None:
@@ -933,6 +940,7 @@ def main():
                    'kron_layers': sum(1 for s in specs if s['kind'] != 'bn'),
                    'bn_layers': sum(1 for s in specs if s['kind'] == 'bn'),
                    'damping': 1e-3, 'ema_decay': 0.95, 'invert_every_step': True, 'inverse_form': inverse_form,
+                   'curvature_streams': 1 if _curvature.two_stream_min_dim is None else 2,
                    'factor_mode': torchsso.factor_mode(), 'factor_side_streams': factor_streams,
                    'inputs_resident_GB': round(resident / 1e9, 3)},
         'tflops': round(total_flops / (ms * 1e-3) / 1e12, 2),

@@ -194,9 +194,14 @@ struct GroupPlan {
   }
 };
 
+// 64-wide tiles (one wave each) up to 192 rows; from there a 128-wide tile has at most a
+// quarter of padding and loads half as many operand elements per matrix instruction
+// (factors of 256 rows: 7 % faster on 128-wide tiles).
+constexpr int GROUP_W1_MAX_DIM = 192;
+
 static GroupPlan plan_group(int d, long K, long target) {
   GroupPlan p;
-  p.w = d <= 256 ? 1 : 2;
+  p.w = d <= GROUP_W1_MAX_DIM ? 1 : 2;
   p.ts = 64 * p.w;
   p.T = cdiv(d, p.ts);
   p.ntiles = p.T * (p.T + 1) / 2;
@@ -381,7 +386,7 @@ static GroupedPlan make_plan(int count, const kfac_factor_job* jobs) {
               : kfac_factor_executed_flops(c.d, c.K);
       continue;
     }
-    const int w = c.d <= 256 ? 1 : 2;
+    const int w = c.d <= GROUP_W1_MAX_DIM ? 1 : 2;
     gp.members[c.path][w - 1].push_back(i);
     if (c.path == P_CONVP && c.copy_bytes) {
       gp.copies.push_back(i);

@@ -306,6 +306,20 @@ def run(device, key, reads, launch):
     return out
 
 
+_curvature_streams = {}    # device index -> torch.cuda.Stream
+
+
+def curvature_stream(device):
+    """A library-owned default-priority stream for the part of the curvature phase
+    (inversion, preconditioning) that runs beside the caller's stream."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    with _lock:
+        st = _curvature_streams.get(idx)
+        if st is None:
+            st = _curvature_streams[idx] = torch.cuda.Stream(device=idx)
+    return st
+
+
 def join(device=None):
     """The current stream of `device` (all devices if None) waits for the factor
     products enqueued so far."""
@@ -344,6 +358,12 @@ def _at_exit():
                 side.synchronize()
     except Exception:
         pass
+    try:
+        for st in _curvature_streams.values():
+            st.synchronize()
+    except Exception:
+        pass
+    _curvature_streams.clear()
     _pending.clear()
     _streams.clear()
     _deferred.clear()

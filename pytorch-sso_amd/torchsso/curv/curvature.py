@@ -697,6 +697,65 @@ def step_all(curvs, update_std=False, update_inv=True):
         update_std_all(sel)
 
 
+# The blocked Cholesky factorisation of the largest factors is a chain of small launches
+# (two per 128 rows) that leaves most of the chip idle; smaller factors ride along in the
+# same launches for nothing, but their triangular inverses and the preconditioning of
+# their layers would still queue up behind the end of that chain.  When the largest factor
+# has at least this many rows, the layers whose factors are at most half its size take
+# their whole curvature phase (running average, inversion, preconditioning) to a side
+# stream, where their dense launches fill the chip beside the chain.  None: one stream.
+two_stream_min_dim = 2048
+
+
+def _chain_split(pairs):
+    """(layers holding the longest factorisations, the other layers) or None."""
+    if two_stream_min_dim is None or len(pairs) < 2:
+        return None
+    dims, devices = [], set()
+    for c, params in pairs:
+        w = params[0]
+        if not w.is_cuda:
+            return None
+        devices.add(w.device)
+        dims.append(max(w.shape[0], w[0].numel() + (1 if c.bias else 0))
+                    if c.kind == 'kron' else 0)
+    dmax = max(dims)
+    if dmax < two_stream_min_dim or len(devices) != 1:
+        return None
+    late = [p for p, d in zip(pairs, dims) if 2 * d > dmax]
+    early = [p for p, d in zip(pairs, dims) if 2 * d <= dmax]
+    if not early or not any(c.kind == 'kron' for c, _ in early):
+        return None
+    return late, early
+
+
+def step_and_precondition_all(pairs, update_std=False, update_inv=True, precondition=True):
+    """step_all for the curvatures of `pairs` (a list of (curvature, params)), then
+    precondition_all(pairs) if asked; on two streams where that pays (see
+    `two_stream_min_dim`): the layers are independent of one another, so the results are
+    those of one stream."""
+    curvs = [c for c, _ in pairs]
+    plain_std = not isinstance(update_std, (list, tuple)) and not update_std
+    split = _chain_split(pairs) if (update_inv and precondition and plain_std) else None
+    if split is None:
+        step_all(curvs, update_std=update_std, update_inv=update_inv)
+        if precondition:
+            precondition_all(pairs)
+        return
+    late, early = split
+    device = late[0][1][0].device
+    _lanes.join()                       # (on the caller's stream: the side stream inherits it)
+    cur = torch.cuda.current_stream(device)
+    side = _lanes.curvature_stream(device)
+    side.wait_stream(cur)
+    step_all([c for c, _ in late])
+    precondition_all(late)
+    with torch.cuda.stream(side):
+        step_all([c for c, _ in early])
+        precondition_all(early)
+    cur.wait_stream(side)
+
+
 def precondition_all(pairs):
     """precondition_grad for a list of (curvature, params): grads are replaced
     in place by G^-1 [dW|db] A^-1 (reference: cov/linear.py:69-84,

@@ -282,12 +282,15 @@ class SecondOrderOptimizer(Optimizer):
         if curvs:
             if isinstance(update_std, (list, tuple)):
                 update_std = [u for g, u in zip(groups, update_std) if g['curv'] is not None]
-            _curv.step_all(curvs, update_std=update_std, update_inv=update_inv)
+            pairs = [(g['curv'], g[target]) for g in groups if g['curv'] is not None]
             if getattr(self, 'check_spd', False):
-                _curv.check_spd_all(curvs)
-            if precondition:
-                _curv.precondition_all([(g['curv'], g[target]) for g in groups
-                                        if g['curv'] is not None])
+                _curv.step_all(curvs, update_std=update_std, update_inv=update_inv)
+                _curv.check_spd_all(curvs)       # (before anything is preconditioned)
+                if precondition:
+                    _curv.precondition_all(pairs)
+            else:
+                _curv.step_and_precondition_all(pairs, update_std=update_std,
+                                                update_inv=update_inv, precondition=precondition)
 
         fused = []
         for group in groups:

@@ -43,6 +43,48 @@ def test_layer_set_step_is_bit_identical_with_side_streams(count):
         assert torch.equal(a, b), 'tensor %d differs with %d streams' % (i, count)
 
 
+def test_curvature_phase_on_two_streams_gives_the_same_step():
+    """A layer with a factor of 2048 rows or more sends the layers whose factors are at
+    most half as large to a side stream for their inversion and preconditioning
+    (curvature.step_and_precondition_all).  Same parameters, running averages and
+    inverses as on one stream: the running averages bit for bit, the rest to rounding
+    (how a batched call groups its panel updates and cuts its reductions depends on the
+    largest matrix of the call, so the order of the sums changes with the list)."""
+    from torchsso.curv import curvature as C
+    specs = [dict(kind='linear', name='wide', fin=2100, fout=300, bias=True),
+             dict(kind='linear', name='mid', fin=900, fout=260, bias=True),
+             bench.conv_spec('conv', 16, 32, 3, 1, 1, 12, bias=False),
+             dict(kind='bn', name='bn', c=32, h=12),
+             dict(kind='linear', name='small', fin=120, fout=10, bias=False)]
+    before = C.two_stream_min_dim
+    try:
+        C.two_stream_min_dim = 2048
+        ls = bench.LayerSet(specs, 32, torch.device('cuda:0'), seed=3)
+        pairs = [(g['curv'], g['params']) for g in ls.opt.param_groups]
+        late, early = C._chain_split(pairs)
+        assert [c.module.in_features for c, _ in late] == [2100] and len(early) == 4
+        del ls
+        two = layer_set_state(2, specs)
+        C.two_stream_min_dim = None
+        one = layer_set_state(2, specs)
+    finally:
+        C.two_stream_min_dim = before
+    assert len(one) == len(two)
+    worst = 0.
+    for i, (a, b) in enumerate(zip(one, two)):
+        err = ((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-30)).item()
+        worst = max(worst, err)
+        assert err <= 1e-4, 'tensor %d: one vs two curvature streams differ by %.3g' % (i, err)
+    print('one vs two curvature streams: worst relative difference %.3g' % worst)
+    n_params = sum(1 for _ in bench.LayerSet(specs, 32, torch.device('cuda:0')).model.parameters())
+    k = n_params
+    for c_specs in specs:                 # per curvature: ema tensors, then inverses
+        n = 2
+        for j in range(n):
+            assert torch.equal(one[k + j], two[k + j]), 'running average %d differs' % (k + j)
+        k += 2 * n
+
+
 class Net(nn.Module):
     def __init__(self):
         super().__init__()
