@@ -306,17 +306,17 @@ def run(device, key, reads, launch):
     return out
 
 
-_curvature_streams = {}    # device index -> torch.cuda.Stream
+_curvature_streams = {}    # (device index, k) -> torch.cuda.Stream
 
 
-def curvature_stream(device):
-    """A library-owned default-priority stream for the part of the curvature phase
-    (inversion, preconditioning) that runs beside the caller's stream."""
+def curvature_stream(device, k=0):
+    """The k-th library-owned default-priority stream for the parts of the curvature phase
+    (inversion, preconditioning) that run beside the caller's stream."""
     idx = device.index if device.index is not None else torch.cuda.current_device()
     with _lock:
-        st = _curvature_streams.get(idx)
+        st = _curvature_streams.get((idx, k))
         if st is None:
-            st = _curvature_streams[idx] = torch.cuda.Stream(device=idx)
+            st = _curvature_streams[(idx, k)] = torch.cuda.Stream(device=idx)
     return st
 
 

@@ -707,8 +707,15 @@ def step_all(curvs, update_std=False, update_inv=True):
 two_stream_min_dim = 2048
 
 
+# (classes of layers that get a stream each; with three, the smaller factors no longer ride
+# along in the launches of the middle ones and the step is as slow as on one stream)
+curvature_streams_max = 2
+
+
 def _chain_split(pairs):
-    """(layers holding the longest factorisations, the other layers) or None."""
+    """The layers in classes by the length of their longest factorisation, longest
+    first (every class: factors at most half as large as the largest of the class
+    before), or None where one stream serves."""
     if two_stream_min_dim is None or len(pairs) < 2:
         return None
     dims, devices = [], set()
@@ -719,21 +726,34 @@ def _chain_split(pairs):
         devices.add(w.device)
         dims.append(max(w.shape[0], w[0].numel() + (1 if c.bias else 0))
                     if c.kind == 'kron' else 0)
-    dmax = max(dims)
-    if dmax < two_stream_min_dim or len(devices) != 1:
+    if len(devices) != 1:
         return None
-    late = [p for p, d in zip(pairs, dims) if 2 * d > dmax]
-    early = [p for p, d in zip(pairs, dims) if 2 * d <= dmax]
-    if not early or not any(c.kind == 'kron' for c, _ in early):
+    classes = []
+    rest = list(zip(pairs, dims))
+    while rest:
+        dmax = max(d for _, d in rest)
+        if dmax < two_stream_min_dim or len(classes) + 1 >= curvature_streams_max:
+            break
+        head = [(p, d) for p, d in rest if 2 * d > dmax]
+        tail = [(p, d) for p, d in rest if 2 * d <= dmax]
+        if not any(p[0].kind == 'kron' for p, _ in tail):
+            break
+        classes.append([p for p, _ in head])
+        rest = tail
+    if not classes:
         return None
-    return late, early
+    classes.append([p for p, _ in rest])
+    return classes
 
 
-def step_and_precondition_all(pairs, update_std=False, update_inv=True, precondition=True):
+def step_and_precondition_all(pairs, update_std=False, update_inv=True, precondition=True,
+                              then=None):
     """step_all for the curvatures of `pairs` (a list of (curvature, params)), then
-    precondition_all(pairs) if asked; on two streams where that pays (see
+    precondition_all(pairs) if asked; on several streams where that pays (see
     `two_stream_min_dim`): the layers are independent of one another, so the results are
-    those of one stream."""
+    those of one stream.  `then(sub_pairs)`: called for every part of the list right behind
+    its preconditioning, on the stream that did it (the parameter update of those layers);
+    when this function returns, the caller's stream has been made to wait for all of it."""
     curvs = [c for c, _ in pairs]
     plain_std = not isinstance(update_std, (list, tuple)) and not update_std
     split = _chain_split(pairs) if (update_inv and precondition and plain_std) else None
@@ -741,19 +761,23 @@ def step_and_precondition_all(pairs, update_std=False, update_inv=True, precondi
         step_all(curvs, update_std=update_std, update_inv=update_inv)
         if precondition:
             precondition_all(pairs)
+        if then is not None:
+            then(pairs)
         return
-    late, early = split
-    device = late[0][1][0].device
-    _lanes.join()                       # (on the caller's stream: the side stream inherits it)
+    device = pairs[0][1][0].device
+    _lanes.join()                       # (on the caller's stream: the side streams inherit it)
     cur = torch.cuda.current_stream(device)
-    side = _lanes.curvature_stream(device)
-    side.wait_stream(cur)
-    step_all([c for c, _ in late])
-    precondition_all(late)
-    with torch.cuda.stream(side):
-        step_all([c for c, _ in early])
-        precondition_all(early)
-    cur.wait_stream(side)
+    sides = [_lanes.curvature_stream(device, k) for k in range(len(split) - 1)]
+    for side in sides:
+        side.wait_stream(cur)
+    for part, stream in zip(split, [cur] + sides):
+        with torch.cuda.stream(stream):
+            step_all([c for c, _ in part])
+            precondition_all(part)
+            if then is not None:
+                then(part)
+    for side in sides:
+        cur.wait_stream(side)
 
 
 def precondition_all(pairs):

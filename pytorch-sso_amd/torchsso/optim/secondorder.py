@@ -278,30 +278,40 @@ class SecondOrderOptimizer(Optimizer):
         for group in groups:
             self.update_preprocess(group, target=target, grad_type='raw', l2_done=True)
 
-        curvs = [g['curv'] for g in groups if g['curv'] is not None]
+        def finish(sub):
+            """Everything behind the preconditioning, for the groups in `sub`."""
+            fused = []
+            for group in sub:
+                if self._can_fuse_update(group):
+                    fused.append(group)
+                else:
+                    self.update_preprocess(group, target=target, grad_type='preconditioned')
+                    self.update(group, target=target)
+            self._fused_update(fused, target)
+            for group in sub:
+                self.update_postprocess(group, target=target)
+
+        with_curv = [g for g in groups if g['curv'] is not None]
+        curvs = [g['curv'] for g in with_curv]
         if curvs:
             if isinstance(update_std, (list, tuple)):
                 update_std = [u for g, u in zip(groups, update_std) if g['curv'] is not None]
-            pairs = [(g['curv'], g[target]) for g in groups if g['curv'] is not None]
+            pairs = [(g['curv'], g[target]) for g in with_curv]
+            by_curv = {id(g['curv']): g for g in with_curv}
+            finish_pairs = lambda sub: finish([by_curv[id(c)] for c, _ in sub])
             if getattr(self, 'check_spd', False):
                 _curv.step_all(curvs, update_std=update_std, update_inv=update_inv)
                 _curv.check_spd_all(curvs)       # (before anything is preconditioned)
                 if precondition:
                     _curv.precondition_all(pairs)
+                finish(with_curv)
             else:
+                # (the layers are independent: where the curvature phase runs on two
+                # streams, each part's update follows its preconditioning on its stream)
                 _curv.step_and_precondition_all(pairs, update_std=update_std,
-                                                update_inv=update_inv, precondition=precondition)
-
-        fused = []
-        for group in groups:
-            if self._can_fuse_update(group):
-                fused.append(group)
-            else:
-                self.update_preprocess(group, target=target, grad_type='preconditioned')
-                self.update(group, target=target)
-        self._fused_update(fused, target)
-        for group in groups:
-            self.update_postprocess(group, target=target)
+                                                update_inv=update_inv, precondition=precondition,
+                                                then=finish_pairs)
+        finish([g for g in groups if g['curv'] is None])
 
     def backward_postprocess(self, target='params'):
         """Accumulated gradients and factors become the current ones

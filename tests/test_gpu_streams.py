@@ -61,7 +61,7 @@ def test_curvature_phase_on_two_streams_gives_the_same_step():
         C.two_stream_min_dim = 2048
         ls = bench.LayerSet(specs, 32, torch.device('cuda:0'), seed=3)
         pairs = [(g['curv'], g['params']) for g in ls.opt.param_groups]
-        late, early = C._chain_split(pairs)
+        late, early = C._chain_split(pairs)          # (two classes)
         assert [c.module.in_features for c, _ in late] == [2100] and len(early) == 4
         del ls
         two = layer_set_state(2, specs)
