@@ -30,6 +30,9 @@ namespace kfac {
 struct DenseKM {
   static constexpr int layout = KM;
   static constexpr bool has_second = true;
+  static constexpr bool vec4 = true;
+  // (the columns in memory; the optional last one is not)
+  __device__ __forceinline__ int vec_cols() const { return extra ? M - 1 : M; }
   const float* p;
   const float* vec;
   int ld, M, extra;
