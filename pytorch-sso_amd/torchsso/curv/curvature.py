@@ -712,10 +712,34 @@ two_stream_min_dim = 2048
 curvature_streams_max = 2
 
 
+def chain_classes(dims, min_dim, max_classes):
+    """Indices of the layers in classes by the length of their longest factorisation,
+    longest first: `dims[i]` is the largest factor dimension of layer i (0 for a layer
+    without Kronecker factors).  A class is split off while the largest dimension left is
+    at least `min_dim`: it takes the layers with a factor of more than half that size, and
+    the rest must still hold a Kronecker layer.  None where one class (one stream) serves."""
+    if min_dim is None:
+        return None
+    classes = []
+    rest = list(range(len(dims)))
+    while rest and len(classes) + 1 < max_classes:
+        dmax = max(dims[i] for i in rest)
+        if dmax < min_dim:
+            break
+        head = [i for i in rest if 2 * dims[i] > dmax]
+        tail = [i for i in rest if 2 * dims[i] <= dmax]
+        if not any(dims[i] > 0 for i in tail):
+            break
+        classes.append(head)
+        rest = tail
+    if not classes:
+        return None
+    classes.append(rest)
+    return classes
+
+
 def _chain_split(pairs):
-    """The layers in classes by the length of their longest factorisation, longest
-    first (every class: factors at most half as large as the largest of the class
-    before), or None where one stream serves."""
+    """The (curvature, params) pairs in the classes of `chain_classes`, or None."""
     if two_stream_min_dim is None or len(pairs) < 2:
         return None
     dims, devices = [], set()
@@ -728,22 +752,8 @@ def _chain_split(pairs):
                     if c.kind == 'kron' else 0)
     if len(devices) != 1:
         return None
-    classes = []
-    rest = list(zip(pairs, dims))
-    while rest:
-        dmax = max(d for _, d in rest)
-        if dmax < two_stream_min_dim or len(classes) + 1 >= curvature_streams_max:
-            break
-        head = [(p, d) for p, d in rest if 2 * d > dmax]
-        tail = [(p, d) for p, d in rest if 2 * d <= dmax]
-        if not any(p[0].kind == 'kron' for p, _ in tail):
-            break
-        classes.append([p for p, _ in head])
-        rest = tail
-    if not classes:
-        return None
-    classes.append([p for p, _ in rest])
-    return classes
+    classes = chain_classes(dims, two_stream_min_dim, curvature_streams_max)
+    return None if classes is None else [[pairs[i] for i in cls] for cls in classes]
 
 
 def step_and_precondition_all(pairs, update_std=False, update_inv=True, precondition=True,

@@ -727,3 +727,25 @@ def test_fisher_closure_exact_and_mc(oracle_ops):
     assert (opt.param_groups[0]['curv'].G - exact_first).norm() / exact_first.norm() < 0.15
     with pytest.raises(ValueError):
         torchsso.get_closure_for_fisher(opt, model, x, y, approx_type='bogus')()
+
+
+def test_layers_are_sorted_into_classes_by_the_length_of_their_factorisation():
+    """curvature.chain_classes: which layers keep the caller's stream in the curvature phase
+    (those holding a factor of more than half the largest dimension) and which go to the
+    side stream; one class where the largest factor is small or nothing would be left."""
+    from torchsso.curv.curvature import chain_classes
+    # ResNet-50-like: three 4608-row layers, 2304 / 2048-row ones, small ones, BatchNorm (0)
+    dims = [147, 0, 576, 4608, 2304, 0, 2048, 4608, 1024, 2049, 4608]
+    assert chain_classes(dims, 2048, 2) == [[3, 7, 10], [0, 1, 2, 4, 5, 6, 8, 9]]
+    # exactly half the largest dimension belongs to the second class, one more row does not
+    assert chain_classes([4608, 2304, 2305], 2048, 2) == [[0, 2], [1]]
+    # AlexNet's classifier: fc6 against fc7 / fc8
+    assert chain_classes([9217, 4097, 4097], 2048, 2) == [[0], [1, 2]]
+    # three classes when allowed
+    assert chain_classes([9217, 4097, 1000, 0], 2048, 3) == [[0], [1], [2, 3]]
+    # small factors, a single class, or only layers without factors left: one stream
+    assert chain_classes([1001, 1000, 11], 2048, 2) is None
+    assert chain_classes([4608, 4000], 2048, 2) is None
+    assert chain_classes([4608, 0, 0], 2048, 2) is None
+    assert chain_classes([4608, 100], None, 2) is None
+    assert chain_classes([4608, 100], 2048, 1) is None
