@@ -531,29 +531,41 @@ __global__ __launch_bounds__(NTHREADS, 3) void potrf_trail_kernel(const MatDesc*
 // before the next row panel:   A[i,j] -= U[p-1,i]^T U[p-1,j]   for block rows
 // row_lo <= i < row_hi (row_lo = p + 1: row p got its update in a launch of its own).
 // The first `ndiag` workgroups take one diagonal block each (potrf_diag_kernel's work),
-// the others one tile each.  The launch carries the diagonal block's LDS, so one
+// the others `tpw` tiles each.  The launch carries the diagonal block's LDS, so one
 // workgroup runs per CU: the tile workgroups use the CUs that the few diagonal blocks
-// leave idle, for about as long as a diagonal block takes.
+// leave idle, for about as long as a diagonal block takes; a launch with more tiles than
+// CUs puts up to three tiles into a workgroup, as many waves per CU as in a launch of
+// their own.
+constexpr int STEP_TILES_PER_WG = DIAG_THREADS / NTHREADS;
+static_assert(STEP_TILES_PER_WG * SMEM_FLOATS * (int)sizeof(float) <= DIAG_SMEM_BYTES,
+              "the tiles of a workgroup share the diagonal block's LDS");
+
 __global__ __launch_bounds__(DIAG_THREADS) void potrf_step_kernel(const MatDesc* table, int p,
                                                                    int* info, int ndiag,
-                                                                   int row_lo, int row_hi,
+                                                                   int row_lo, int row_hi, int tpw,
                                                                    const WorkList wl) {
   extern __shared__ __attribute__((aligned(16))) float dsm[];
   if ((int)blockIdx.x < ndiag) {
     diag_block(table[blockIdx.x], p, info, dsm, true);
     return;
   }
-  if (threadIdx.x >= NTHREADS) return;       // a tile is the work of four waves
-  int mat, local;
-  work_find_item(wl, (int)blockIdx.x - ndiag, mat, local);
-  const MatDesc m = table[mat];
-  int bi, bj;
-  if (!trail_tile(m.T, row_lo, row_hi, local, bi, bj)) return;
+  // A tile is the work of four waves.  A launch with more tiles than compute units packs
+  // `tpw` (up to three) of them into a workgroup, each group of four waves with its own
+  // 40 KB of the launch's LDS; every tile of this launch reduces over the same 128 rows, so
+  // the groups meet at the same barriers (a group that has returned no longer counts).
+  const int group = (int)threadIdx.x / NTHREADS;
+  if (group >= tpw) return;
+  const int item = ((int)blockIdx.x - ndiag) * tpw + group;
+  if (item >= wl.cum[wl.n]) return;
+  int mat, local, bi, bj;
+  work_find_item(wl, item, mat, local);
+  if (!trail_tile(table[mat].T, row_lo, row_hi, local, bi, bj)) return;
   if (bj == p) return;                       // tile (p, p): the diagonal block's own workgroup
+  const MatDesc m = table[mat];
   const int n = m.n;
   DenseKM P{m.U + (size_t)(p - 1) * DB * n, nullptr, n, n, 0};
   EpiStore epi{m.U, n, n, n, -1.f, 1.f, false};
-  gemm_tile(P, P, bi * BM, bj * BN, 0, DB, bi == bj, epi, dsm);
+  gemm_tile(P, P, bi * BM, bj * BN, 0, DB, bi == bj, epi, dsm + group * SMEM_FLOATS);
 }
 
 // The row panel for launches of few tiles: the same 128x128x128 product, but by 16 waves
@@ -1081,8 +1093,10 @@ static int run_batched(std::vector<HostMat>& mats, int mode, int* info, void* wo
         for_worklists(na, rest_items, [&](const WorkList& wl, int grid) {
           const int nd = first ? na : 0;
           first = false;
-          hipLaunchKernelGGL(potrf_step_kernel, dim3(nd + grid), dim3(DIAG_THREADS), DIAG_SMEM_BYTES,
-                             stream, table, p, info, nd, p, Pend, wl);
+          // (one workgroup runs per compute unit: beyond 256 tiles, up to three to a workgroup)
+          const int tpw = std::min(STEP_TILES_PER_WG, std::max(1, cdiv(grid, 256)));
+          hipLaunchKernelGGL(potrf_step_kernel, dim3(nd + cdiv(grid, tpw)), dim3(DIAG_THREADS),
+                             DIAG_SMEM_BYTES, stream, table, p, info, nd, p, Pend, tpw, wl);
         });
       }
       const int nb = active(p + 2);
