@@ -507,10 +507,11 @@ constexpr int GROUP_BLOCKS = 4;
 // The last TAIL_BLOCKS diagonal blocks of the largest matrices form one group: the deeper
 // update of the rows beyond a group is a launch that lasts as long as one 512-deep tile
 // (50 us) however few tiles it has, while the rank-128 updates of a short trailing matrix
-// all fit beside the next diagonal block (one workgroup per compute unit there).
-// (config 3: inversion 5.14 ms without, 5.09 / 5.04 / 5.05 / 5.14 ms with 8 / 12 / 16 / 24;
-// three 9217 / 4097 / 4097 matrices: 10.63 without, 10.60 / 10.57 / 10.52 / 10.46 ms)
-constexpr int TAIL_BLOCKS = 16;
+// all fit beside the next diagonal block (up to three tiles per compute unit there).
+// (with the tiles packed three to a workgroup: config 3 inversion 4.75 / 4.77 / 4.90 / 5.16 ms
+// with 16 / 24 / 32 / 40; a 3201^2 and a 1601^2 matrix 1.68 / 1.58 / 1.53 / 1.53 ms; three
+// 9217 / 4097 / 4097 matrices 10.12 / 10.03 / 9.95 / 9.92 ms and 10.58 ms with 64)
+constexpr int TAIL_BLOCKS = 24;
 
 __global__ __launch_bounds__(NTHREADS, 3) void potrf_trail_kernel(const MatDesc* table, int kb0,
                                                                int nk, int row_lo, int row_hi,
