@@ -51,7 +51,7 @@ struct ShiftX {
     const int rem = k - n * hh * ww;
     const int ry = by_ww.div(rem);
     const int rx = rem - ry * ww;
-    return KS{valid ? (unsigned)(n * C * H * W + (u0 + ry) * W + v0 + rx) * 4u : INV_K};
+    return KS{k_offset_or_invalid((unsigned)(n * C * H * W + (u0 + ry) * W + v0 + rx) * 4u, valid)};
   }
   __device__ __forceinline__ unsigned off(const MS& m, const KS& k) const { return m.off + k.off; }
   __device__ __forceinline__ bool is_one(const MS&) const { return false; }
